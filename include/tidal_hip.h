@@ -1,0 +1,227 @@
+/*
+ * tidal_hip.h -- C ABI of libtidal_hip.so, the gfx950 (MI355X) implementation of the
+ * TidalDecode decode-attention path.
+ *
+ * Every entry point takes raw device pointers, plain integer sizes and a hipStream_t passed as
+ * void*.  No torch types cross this boundary.  All functions return 0 (TD_OK) on success and a
+ * non-zero td_status otherwise; td_last_error() then holds a human-readable message for the
+ * calling thread.  Nothing here synchronises the stream and nothing copies device -> host.
+ *
+ * Each declaration cites the interface of the reference (DerrickYLJ/TidalDecode) that it
+ * replaces; paths are relative to the reference checkout.
+ */
+#ifndef TIDAL_HIP_H_
+#define TIDAL_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  TD_OK = 0,
+  TD_ERR_INVALID_ARG = 1, /* shape / pointer / range check failed */
+  TD_ERR_UNSUPPORTED = 2, /* dtype, head_dim or group size has no kernel ("failed to dispatch") */
+  TD_ERR_STATE = 3,       /* workspace too small for the plan */
+  TD_ERR_HIP = 4          /* a HIP runtime call failed */
+} td_status;
+
+/* Element types.  KV cache, q, k, v, o are TD_F16 or TD_BF16; scores may be TD_F32 as well. */
+typedef enum { TD_F16 = 0, TD_BF16 = 1, TD_F32 = 2 } td_dtype;
+
+/* Layout of the last three page dimensions, tidal/utils/utils.py:1-5. */
+typedef enum { TD_NHD = 0, TD_HND = 1 } td_layout;
+
+/* How one row of the sparse index list is interpreted by td_decode_attn. */
+typedef enum {
+  /* Entries are physical page ids; every listed page contributes page_size tokens.  This is the
+   * reference's meaning (kernels/include/decode/decode_page.cuh:320-346). */
+  TD_IDX_PAGES = 0,
+  /* Entries are physical token slots, slot = page_id * page_size + entry.  Extension for
+   * token-granular selection with page_size > 1. */
+  TD_IDX_SLOTS = 1
+} td_idx_kind;
+
+/* How scores are reduced before selection (td_score_reduce). */
+typedef enum {
+  TD_REDUCE_HEAD_SUM = 0, /* softmax probabilities summed over all query heads -> 1 row   */
+  TD_REDUCE_GROUP_SUM = 1 /* summed over the query heads of each KV head      -> H_kv rows */
+} td_reduce_mode;
+
+/*
+ * Paged KV pool of one layer.
+ * data: [max_pages, 2, page_size, num_kv_heads, head_dim] (TD_NHD) or
+ *       [max_pages, 2, num_kv_heads, page_size, head_dim] (TD_HND), index 1 = 0 for K, 1 for V.
+ * Mirrors paged_kv_t, kernels/include/decode/decode_page.cuh:73-252.
+ */
+typedef struct {
+  void* data;
+  int64_t max_pages; /* capacity; slots are clamped to it inside the kernels */
+  int32_t num_kv_heads;
+  int32_t head_dim; /* 64, 128 or 256 */
+  int32_t page_size;
+  int32_t layout; /* td_layout */
+  int32_t dtype;  /* td_dtype: TD_F16 or TD_BF16 */
+} td_paged_kv;
+
+/*
+ * Per-call description of which tokens each sequence attends to.
+ *
+ * idx is a 2-D int32 array with `idx_rows` rows of `idx_row_stride` elements.  Sequence b uses
+ * columns [indptr[b], indptr[b+1]) of every row (indptr lives on the device; if indptr is NULL
+ * the call is for one sequence that uses columns [0, n_list_host)).  Row r belongs to query
+ * head r (idx_rows == num_qo_heads), to KV head r (idx_rows == num_kv_heads) or to everybody
+ * (idx_rows == 1).
+ *
+ * After the listed entries every sequence may attend to one more, partially filled page: the
+ * first last_page_len entries of page last_page_idx ("forced last page",
+ * decode_page.cuh:326-329, decode_attn.cuh:726-730).  The *_arr pointers (device, [batch]) take
+ * precedence over the scalars; last_page_len == 0 disables it.
+ */
+typedef struct {
+  const int32_t* idx;
+  int32_t idx_rows;
+  int32_t idx_row_stride;
+  int32_t kind; /* td_idx_kind */
+  const int32_t* indptr; /* device [batch+1] or NULL */
+  int32_t n_list_host;   /* used when indptr == NULL; else an upper bound of the per-sequence count */
+  const int32_t* last_page_len_arr; /* device [batch] or NULL */
+  const int32_t* last_page_idx_arr; /* device [batch] or NULL */
+  int32_t last_page_len;
+  int32_t last_page_idx;
+} td_index_list;
+
+/*
+ * Split plan of one decode-attention call: how many tokens one workgroup covers and how many
+ * partial results per head that makes.  Pure host arithmetic (no device access); replaces
+ * BatchDecodeHandler::BeginForward + BatchDecodeWithPagedKVCacheWorkEstimation +
+ * PartitionPagedKVCacheComputeAuxiliaryInfo (kernels/include/decode/decode_handler.cuh:39-175,
+ * decode_attn.cuh:687-906; binding tidal/ops/csrc/approx_attn.cu:27-66).
+ */
+typedef struct {
+  int32_t chunk_tokens;    /* tokens per workgroup and head group */
+  int32_t max_splits;      /* upper bound of partial results per head */
+  int32_t waves_per_block; /* 4, 8 or 16 */
+  int32_t fused_merge;     /* 1: last workgroup merges in-kernel; 0: second kernel */
+  int64_t workspace_bytes; /* device scratch the call needs (partials + tickets) */
+} td_decode_plan;
+
+/* Thread-local message of the last failing call. */
+const char* td_last_error(void);
+
+/* Library ABI version (bumped on any signature change). */
+int td_version(void);
+
+/* Number of compute units of the current device (used by the planner; cached). */
+int td_num_cus(void);
+
+/*
+ * Rotate-half (Llama) RoPE applied in place to q [n_tokens, num_qo_heads, head_dim] and
+ * k [n_tokens, num_kv_heads, head_dim]; token i sits at position past_kv_len + i; angle =
+ * position / rope_scale * rope_theta^(-2(j mod D/2)/D).
+ * Replaces apply_rope_in_place (tidal/ops/csrc/bsk_ops.h:23-27, page.cu:212-253) and
+ * QKApplyRotaryInPlace (kernels/include/decode/decode_page.cuh:639-723).
+ */
+int td_rope_in_place(void* q, void* k, int32_t n_tokens, int32_t num_qo_heads,
+                     int32_t num_kv_heads, int32_t head_dim, int64_t past_kv_len, float rope_scale,
+                     float rope_theta, int32_t dtype, void* stream);
+
+/*
+ * Append n_tokens new (k, v) rows [n_tokens, num_kv_heads, head_dim] to one sequence.
+ * The sequence owns pages kv_indices[kv_indptr[0] .. kv_indptr[1]) and, after the append, holds
+ * seq_len = (n_pages - 1) * page_size + last_page_len tokens; the new rows are its last
+ * n_tokens.  n_tokens == 1 is the decode case.  kv_indices / kv_indptr are device arrays.
+ * If meta != NULL, meta_indices/meta_indptr/meta_last_page_len describe a second paged pool
+ * that keeps, per KV page, the running element-wise max (K plane) and min (V plane) of the keys
+ * of that page (one metadata entry per KV page), as the reference does for its page estimator.
+ * Replaces append_kv_cache_decode / append_kv_cache_prefill (bsk_ops.h:52-78, page.cu:6-210),
+ * AppendPagedKVCacheDecode/Prefill (decode_page.cuh:387-627).
+ */
+int td_append_kv(const td_paged_kv* kv, const void* k, const void* v, int32_t n_tokens,
+                 const int32_t* kv_indices, const int32_t* kv_indptr, int32_t last_page_len,
+                 const td_paged_kv* meta, const int32_t* meta_indices, const int32_t* meta_indptr,
+                 int32_t meta_last_page_len, void* stream);
+
+/*
+ * Decode-step fusion of the two calls above for a batch of sequences: rotates q [batch,
+ * num_qo_heads, D] in place, rotates k [batch, num_kv_heads, D] and writes it together with
+ * v into physical slot dst_slot[b] (= page_id * page_size + entry) of the pool.  positions[b]
+ * is the token position of sequence b.  dst_slot and positions are device int32 [batch].
+ * No counterpart as one call in the reference; it fuses apply_rope_in_place + append_kv_cache_decode
+ * (tidal/models/SearchAttention.py:131-150).
+ */
+int td_rope_append_decode(const td_paged_kv* kv, void* q, const void* k, const void* v,
+                          int32_t batch, int32_t num_qo_heads, const int32_t* positions,
+                          const int32_t* dst_slot, float rope_scale, float rope_theta,
+                          void* stream);
+
+/*
+ * Choose the split of a decode-attention call.  max_items is an upper bound of the tokens any
+ * sequence attends to; idx_rows as in td_index_list.  waves_per_block / fused_merge may be
+ * preset to non-zero / non-negative values in *plan to override the heuristics (pass a
+ * zero-initialised struct with fused_merge = -1 for defaults).
+ */
+int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t num_kv_heads, int32_t head_dim,
+                   int32_t idx_rows, int64_t max_items, td_decode_plan* plan);
+
+/*
+ * Decode attention of one new token per sequence over the listed tokens of a paged KV pool:
+ * o[b,h,:] = softmax(q[b,h,:] . K_sel^T / sqrt(D)) V_sel, online softmax in base 2, fp32
+ * accumulation, split over tokens and merged by log-sum-exp.
+ *   q, o       [batch, num_qo_heads, head_dim], dtype of the pool
+ *   scores     optional [batch, num_qo_heads, score_stride]: element i = q . k_i / sqrt(D) of the
+ *              i-th attended token in list order (td_dtype scores_dtype); NULL to skip
+ *   lse        optional float [batch, num_qo_heads]: natural-log sum of exp of the logits
+ *   workspace  device scratch of plan->workspace_bytes, zero-filled once before first use; the
+ *              call leaves its ticket counters zero again.  Calls that share a workspace must
+ *              be ordered on one stream.
+ * Replaces BatchDecodeWithPagedKVCachePyTorchWrapper::Forward (bsk_ops.h:104-113,
+ * tidal/ops/csrc/approx_attn.cu:68-151), BatchDecodeWithPagedKVCacheKernel
+ * (kernels/include/decode/decode_attn.cuh:432-658) including its score output
+ * (decode_attn.cuh:107-109) and VariableLengthMergeStates (decode_attn.cuh:1011-1020).
+ */
+int td_decode_attn(const td_paged_kv* kv, const td_index_list* list, const td_decode_plan* plan,
+                   const void* q, void* o, int32_t batch, int32_t num_qo_heads, float sm_scale,
+                   void* scores, int32_t scores_dtype, int64_t score_stride, float* lse,
+                   void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
+ * Cross-head reduction of selection-layer scores: out[r, i] = sum over the query heads h of
+ * row r of exp(logits[h, i] - lse[h]) (i < n), fp32.  rows = 1 (TD_REDUCE_HEAD_SUM) or
+ * num_kv_heads (TD_REDUCE_GROUP_SUM).  logits is float [num_qo_heads, logits_stride].
+ * No counterpart in the reference (its selection is per head); implements the cross-head sum
+ * of the benchmark configuration.
+ */
+int td_score_reduce(const float* logits, int64_t logits_stride, const float* lse,
+                    int32_t num_qo_heads, int32_t num_kv_heads, int32_t n, int32_t mode,
+                    float* out, int64_t out_stride, void* stream);
+
+/*
+ * Row-wise top-k: for each of `rows` rows of `values` (length len, row stride values_stride)
+ * select the k largest elements; ties at the threshold go to the lower position.  Outputs, per
+ * row, sorted by ascending position: out_values[r, j] (same dtype as values, may be NULL) and
+ * out_idx[r, j] = payload of the selected position p:
+ *     in_idx != NULL              -> in_idx[r * in_idx_stride + p]   (reference meaning)
+ *     page_table != NULL          -> page_table[p / page_size] * page_size + p % page_size
+ *     both NULL                   -> p
+ * k is clamped to len.  NaNs order above +inf.  out rows have stride out_stride.
+ * Replaces topk_filtering (bsk_ops.h:34-39, tidal/ops/csrc/topk.cu:7-44) and decode_select_k
+ * (kernels/include/topk/decode_select_k.cuh:25-62; RAFT radix_topk_one_block_kernel).
+ */
+int td_topk(const void* values, int32_t values_dtype, int64_t values_stride, int32_t rows,
+            int32_t len, int32_t k, const int32_t* in_idx, int64_t in_idx_stride,
+            const int32_t* page_table, int32_t page_size, void* out_values, int32_t* out_idx,
+            int64_t out_stride, void* stream);
+
+/*
+ * RMSNorm: out[r, :] = x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * weight, fp32 math.
+ * Replaces rms_norm_forward (bsk_ops.h:29-32, tidal/ops/csrc/rms_norm.cu:160-212).
+ */
+int td_rms_norm(const void* x, const void* weight, void* out, int32_t rows, int32_t cols,
+                float eps, int32_t dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TIDAL_HIP_H_ */

@@ -1,0 +1,321 @@
+"""GPU parity: decode attention through the C ABI (td_decode_attn) against the CPU oracle.
+
+Tolerance: max-abs 2e-3 for fp16 and 1e-2 for bf16 against the fp32 oracle evaluated on the same,
+identically rounded inputs.  The parameter grid follows the reference's own decode test
+(kernels/src/test/test_batch_decode.cu:215-267: sequence lengths, page sizes, page budgets, head
+dims; per-head page lists drawn from a shuffled iota with the forced last page, :57-76).
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from _util import ATOL, PagedCase, randn, tolerance_report
+
+pytestmark = pytest.mark.gpu
+
+
+def _wrapper(layout, hq, hkv, d, page, dtype, **knobs):
+    from tidaldecode_amd import _kernels
+
+    w = _kernels.BatchDecodeWithPagedKVCachePyTorchWrapper(layout)
+    for key, val in knobs.items():
+        setattr(w, key, val)
+    w.begin_forward(None, hq, hkv, d, page, torch.empty(0, dtype=dtype))
+    return w
+
+
+def _oracle_paged(q, case, lists, last_idx, last_len, kind):
+    from oracle import tidal_oracle as orc
+
+    o, logits = orc.paged_selected_attention(q.numpy(), case.pool_np, lists.numpy(), last_idx, last_len,
+                                             layout=case.layout, kind=kind)
+    return torch.from_numpy(o), logits
+
+
+def _per_head_page_lists(case, hq, budget, seed):
+    """first budget-1 entries of a shuffled iota(num_pages-1) per head, as physical pages"""
+    g = torch.Generator().manual_seed(seed)
+    rows = []
+    for _ in range(hq):
+        perm = torch.randperm(case.n_pages - 1, generator=g)[: budget - 1]
+        rows.append(case.page_table[perm])
+    return torch.stack(rows).to(torch.int32)
+
+
+SEQ_LENS = [63, 127, 213, 1110, 2000, 4099, 8192, 8222, 12345, 28837]
+
+
+@pytest.mark.parametrize("head_dim", [64, 128])
+@pytest.mark.parametrize("seq_len", SEQ_LENS)
+def test_reference_grid_page_lists(cuda, seq_len, head_dim):
+    """fp16, NHD, 32/32 heads: page sizes x page budgets of the reference's test."""
+    h, dtype = 32, torch.float16
+    worst = 0.0
+    kv = (randn((seq_len, h, head_dim), seq_len, dtype), randn((seq_len, h, head_dim), seq_len + 1, dtype))
+    for page_size in [1, 3, 7, 16, 32]:
+        case = PagedCase(seq_len, h, head_dim, page_size, dtype, seed=seq_len + page_size, kv=kv)
+        pool = case.pool.to(cuda)
+        q = randn((h, head_dim), seq_len * 31 + page_size, dtype)
+        for budget in [16, 32, 64, 128]:
+            budget = min(budget, case.n_pages)
+            if budget < 2:
+                continue
+            lists = _per_head_page_lists(case, h, budget, seed=budget)
+            last_idx = int(case.page_table[-1])
+            want, _ = _oracle_paged(q, case, lists, last_idx, case.last_page_len, "pages")
+            w = _wrapper(0, h, h, head_dim, page_size, dtype)
+            qd = q.to(dtype).to(cuda).unsqueeze(0)
+            od = torch.full_like(qd, float("nan"))
+            # the reference passes a [H, budget] buffer of which the first budget-1 columns count
+            idx_buf = torch.zeros((h, budget), dtype=torch.int32)
+            idx_buf[:, : budget - 1] = lists
+            indptr = torch.tensor([0, budget - 1], dtype=torch.int32, device=cuda)
+            w.forward(qd, od, pool, idx_buf.to(cuda), indptr, case.last_page_len, last_idx, None)
+            torch.cuda.synchronize()
+            err = tolerance_report(od[0], want)
+            worst = max(worst, err)
+            assert err <= ATOL[dtype], (seq_len, head_dim, page_size, budget, err)
+    print(f"seq_len={seq_len} D={head_dim} worst max-abs {worst:.2e}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("layout", [0, 1])
+def test_c_restatement_of_reference_checker(cuda, dtype, layout):
+    """Same comparison against the C restatement of cpu_reference::selected_single_mha, which
+    works on a contiguous cache with logical page numbers."""
+    from oracle import cref
+
+    h, d, n, page_size, budget = 32, 128, 2000, 16, 32
+    case = PagedCase(n, h, d, page_size, dtype, layout=layout, seed=5)
+    q = randn((h, d), 99, dtype)
+    g = torch.Generator().manual_seed(1)
+    logical = torch.stack([torch.randperm(case.n_pages - 1, generator=g)[: budget - 1]
+                           for _ in range(h)])
+    sel = torch.cat([logical, torch.full((h, 1), case.n_pages - 1)], dim=1).to(torch.int32)
+    kc, vc = case.k.numpy(), case.v.numpy()
+    if layout == 1:
+        kc, vc = kc.transpose(1, 0, 2).copy(), vc.transpose(1, 0, 2).copy()
+    want = torch.from_numpy(cref.selected_single_mha(q.numpy(), kc, vc, sel.numpy(),
+                                                     case.last_page_len, page_size, layout))
+    phys = case.page_table[logical].to(torch.int32)
+    w = _wrapper(layout, h, h, d, page_size, dtype)
+    qd = q.to(dtype).to(cuda).unsqueeze(0)
+    od = torch.empty_like(qd)
+    w.forward(qd, od, case.pool.to(cuda), phys.to(cuda), None, case.last_page_len,
+              int(case.page_table[-1]), None)
+    torch.cuda.synchronize()
+    assert tolerance_report(od[0], want) <= ATOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("hq,hkv,rows", [(32, 32, 32), (32, 32, 1), (32, 8, 32), (32, 8, 8),
+                                         (32, 8, 1), (16, 8, 8), (64, 8, 8), (40, 40, 40)])
+def test_token_slot_lists(cuda, dtype, hq, hkv, rows):
+    """Token-granular lists (slots) with page size 16: per query head, per KV head, shared."""
+    from oracle import tidal_oracle as orc
+
+    d, n, page_size, k = 128, 3000, 16, 257
+    case = PagedCase(n, hkv, d, page_size, dtype, seed=hq + hkv + rows)
+    q = randn((hq, d), 17, dtype)
+    g = torch.Generator().manual_seed(3)
+    pos = torch.stack([torch.randperm(n, generator=g)[:k] for _ in range(rows)])
+    want = orc.sparse_layer_gather(q, case.k, case.v, pos)
+    # the reference's own definition: dense logits with masked_fill(finfo.min)
+    want2 = orc.sparse_layer(q, case.k, case.v, orc.mask_from_indices(pos, hq, n))
+    assert (want - want2).abs().max() < 1e-5
+    slots = case.slots_of(pos).to(torch.int32)
+    w = _wrapper(0, hq, hkv, d, page_size, dtype)
+    qd = q.to(dtype).to(cuda).unsqueeze(0)
+    od = torch.empty_like(qd)
+    w.forward(qd, od, case.pool.to(cuda), slots.to(cuda), None, 0, 0, None, index_kind="slots")
+    torch.cuda.synchronize()
+    assert tolerance_report(od[0], want) <= ATOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("hq,hkv", [(32, 32), (32, 8)])
+@pytest.mark.parametrize("n", [1, 15, 16, 17, 1000, 4099, 33000])
+def test_full_attention_with_scores(cuda, dtype, hq, hkv, n):
+    """Selection-layer mode: the whole page table in order (shared row), logits and lse out.
+    Pinned twice: the oracle's dense attention and torch's scaled_dot_product_attention."""
+    from oracle import tidal_oracle as orc
+
+    d, page_size = 128, 16
+    case = PagedCase(n, hkv, d, page_size, dtype, seed=n)
+    q = randn((hq, d), n + 1, dtype)
+    logits = orc.attn_logits(q, case.k)
+    want = orc.softmax_pv(logits, case.v)
+    kk = orc.repeat_kv(case.k, hq // hkv).permute(1, 0, 2)[None]
+    vv = orc.repeat_kv(case.v, hq // hkv).permute(1, 0, 2)[None]
+    sdpa = torch.nn.functional.scaled_dot_product_attention(q[None, :, None, :], kk, vv)[0, :, 0]
+    assert (want - sdpa).abs().max() < 1e-5
+    w = _wrapper(0, hq, hkv, d, page_size, dtype)
+    qd = q.to(dtype).to(cuda).unsqueeze(0)
+    od = torch.empty_like(qd)
+    stride = case.n_pages * page_size
+    scores = torch.full((hq, stride), float("nan"), dtype=torch.float32, device=cuda)
+    lse = torch.empty((1, hq), dtype=torch.float32, device=cuda)
+    table = case.page_table[:-1].to(torch.int32).unsqueeze(0)
+    w.forward(qd, od, case.pool.to(cuda), table.to(cuda), None, case.last_page_len,
+              int(case.page_table[-1]), scores, lse=lse)
+    torch.cuda.synchronize()
+    assert tolerance_report(od[0], want) <= ATOL[dtype]
+    got_logits = scores[:, :n].cpu()
+    assert (got_logits - logits).abs().max() <= 2e-4 * max(1.0, logits.abs().max().item())
+    assert torch.isnan(scores[:, n:]).all()  # nothing written past the sequence
+    assert (lse[0].cpu() - torch.logsumexp(logits, -1)).abs().max() <= 1e-3
+
+
+def test_batch_ragged_slots(cuda):
+    """Batch of 8 sequences with different lengths sharing one pool; per-head slot lists with
+    per-sequence counts through indptr."""
+    from oracle import tidal_oracle as orc
+
+    dtype, h, d, page_size = torch.float16, 32, 128, 16
+    g = torch.Generator().manual_seed(0)
+    lens = torch.randint(300, 5000, (8,), generator=g).tolist()
+    ks = [int(x) for x in torch.randint(1, 300, (8,), generator=g)]
+    total_pages = sum((n + page_size - 1) // page_size for n in lens) + 5
+    perm = torch.randperm(total_pages, generator=g)
+    pool = torch.full((total_pages, 2, page_size, h, d), 55.0)
+    qs, wants, rows, used = [], [], [], 0
+    for b, n in enumerate(lens):
+        k = randn((n, h, d), 100 + b, dtype)
+        v = randn((n, h, d), 200 + b, dtype)
+        npg = (n + page_size - 1) // page_size
+        table = perm[used: used + npg]
+        used += npg
+        pad = npg * page_size - n
+        pool[table, 0] = torch.cat([k, torch.zeros(pad, h, d)]).view(npg, page_size, h, d)
+        pool[table, 1] = torch.cat([v, torch.zeros(pad, h, d)]).view(npg, page_size, h, d)
+        q = randn((h, d), 300 + b, dtype)
+        pos = torch.stack([torch.randperm(n, generator=g)[: ks[b]] for _ in range(h)])
+        wants.append(orc.sparse_layer_gather(q, k, v, pos))
+        rows.append((table[pos // page_size] * page_size + pos % page_size).to(torch.int32))
+        qs.append(q)
+    indptr = torch.tensor([0] + list(np.cumsum(ks)), dtype=torch.int32)
+    idx = torch.cat(rows, dim=1).contiguous()
+    w = _wrapper(0, h, h, d, page_size, dtype)
+    qd = torch.stack(qs).to(dtype).to(cuda)
+    od = torch.empty_like(qd)
+    zeros = torch.zeros(8, dtype=torch.int32, device=cuda)
+    w.forward(qd, od, pool.to(dtype).to(cuda), idx.to(cuda), indptr.to(cuda), zeros, zeros, None,
+              index_kind="slots", n_list=max(ks))
+    torch.cuda.synchronize()
+    for b in range(8):
+        assert tolerance_report(od[b], wants[b]) <= ATOL[dtype], b
+
+
+@pytest.mark.parametrize("knobs", [dict(waves_per_block=8, fused_merge=1),
+                                   dict(waves_per_block=16, fused_merge=1),
+                                   dict(waves_per_block=8, fused_merge=0),
+                                   dict(waves_per_block=8, fused_merge=1, chunk_tokens=32),
+                                   dict(waves_per_block=8, fused_merge=0, chunk_tokens=32),
+                                   dict(waves_per_block=16, fused_merge=1, chunk_tokens=100000)])
+def test_split_merge_is_an_identity(cuda, knobs):
+    """Any partition of the token list (1 ... 64 splits, either merge path) gives the unsplit
+    result; repeated calls reuse the ticket counters."""
+    from oracle import tidal_oracle as orc
+
+    dtype, h, d, page_size, n, k = torch.bfloat16, 32, 128, 16, 9000, 2048
+    case = PagedCase(n, h, d, page_size, dtype, seed=11)
+    q = randn((h, d), 12, dtype)
+    g = torch.Generator().manual_seed(13)
+    pos = torch.stack([torch.randperm(n, generator=g)[:k] for _ in range(h)])
+    want = orc.sparse_layer_gather(q, case.k, case.v, pos)
+    slots = case.slots_of(pos).to(torch.int32).to(cuda)
+    w = _wrapper(0, h, h, d, page_size, dtype, **knobs)
+    qd = q.to(dtype).to(cuda).unsqueeze(0)
+    pool = case.pool.to(cuda)
+    for _ in range(3):
+        od = torch.full_like(qd, float("nan"))
+        w.forward(qd, od, pool, slots, None, 0, 0, None, index_kind="slots")
+        torch.cuda.synchronize()
+        assert tolerance_report(od[0], want) <= ATOL[dtype]
+
+
+def test_special_cases(cuda):
+    """k = 1 returns the value row; k = N equals full attention; order of the list is irrelevant;
+    an empty list with no last page returns zeros."""
+    from oracle import tidal_oracle as orc
+
+    dtype, h, d, page_size, n = torch.float16, 32, 128, 16, 777
+    case = PagedCase(n, h, d, page_size, dtype, seed=21)
+    q = randn((h, d), 22, dtype)
+    pool = case.pool.to(cuda)
+    qd = q.to(dtype).to(cuda).unsqueeze(0)
+    w = _wrapper(0, h, h, d, page_size, dtype)
+
+    def run(pos):
+        od = torch.full_like(qd, float("nan"))
+        slots = case.slots_of(pos).to(torch.int32).to(cuda).contiguous()
+        w.forward(qd, od, pool, slots, None, 0, 0, None, index_kind="slots")
+        torch.cuda.synchronize()
+        return od[0].float().cpu()
+
+    one = torch.randint(0, n, (h, 1), generator=torch.Generator().manual_seed(1))
+    got = run(one)
+    assert torch.equal(got, case.v[one[:, 0], torch.arange(h)])  # softmax over one token is 1
+    everything = torch.arange(n).repeat(h, 1)
+    assert (run(everything) - orc.full_attention(q, case.k, case.v)).abs().max() <= ATOL[dtype]
+    g = torch.Generator().manual_seed(2)
+    pos = torch.stack([torch.randperm(n, generator=g)[:100] for _ in range(h)])
+    a = run(pos)
+    b = run(pos[:, torch.randperm(100, generator=g)])
+    assert (a - b).abs().max() <= 1e-3
+    od = torch.full_like(qd, float("nan"))
+    empty = torch.zeros((h, 0), dtype=torch.int32, device=cuda)
+    w.forward(qd, od, pool, empty, None, 0, 0, None, index_kind="slots")
+    torch.cuda.synchronize()
+    assert torch.equal(od.float().cpu(), torch.zeros(1, h, d))
+
+
+def test_out_of_range_indices_are_clamped_not_faulting(cuda):
+    """Indices outside the pool read the pool's last slot instead of faulting."""
+    dtype, h, d, page_size, n = torch.float16, 32, 128, 16, 100
+    case = PagedCase(n, h, d, page_size, dtype, seed=31)
+    w = _wrapper(0, h, h, d, page_size, dtype)
+    qd = randn((1, h, d), 1, dtype).to(dtype).to(cuda)
+    od = torch.empty_like(qd)
+    bad = torch.full((h, 8), 2**30, dtype=torch.int32, device=cuda)
+    bad[:, 1] = -5
+    w.forward(qd, od, case.pool.to(cuda), bad, None, 0, 0, None, index_kind="slots")
+    torch.cuda.synchronize()
+    assert torch.isfinite(od.float()).all()
+
+
+def test_error_paths(cuda):
+    """forward before begin_forward, unsupported dtype, wrong shapes: RuntimeError, as the
+    reference's TORCH_CHECKs / handler raise."""
+    from tidaldecode_amd import _kernels
+
+    w = _kernels.BatchDecodeWithPagedKVCachePyTorchWrapper(0)
+    q = torch.zeros((1, 32, 128), dtype=torch.float16, device=cuda)
+    pool = torch.zeros((4, 2, 16, 32, 128), dtype=torch.float16, device=cuda)
+    idx = torch.zeros((32, 4), dtype=torch.int32, device=cuda)
+    with pytest.raises(RuntimeError, match="BeginForward"):
+        w.forward(q, q.clone(), pool, idx, None, 1, 0, None)
+    with pytest.raises(RuntimeError, match="failed to dispatch"):
+        w.begin_forward(None, 32, 32, 128, 16, torch.empty(0, dtype=torch.float32))
+    with pytest.raises(RuntimeError, match="multiple"):
+        w.begin_forward(None, 32, 5, 128, 16, torch.empty(0, dtype=torch.float16))
+    w.begin_forward(None, 32, 32, 128, 16, torch.empty(0, dtype=torch.float16))
+    with pytest.raises(RuntimeError):
+        w.forward(q, q.clone(), pool, idx.long(), None, 1, 0, None)
+    with pytest.raises(RuntimeError):
+        w.forward(q, q.clone(), pool, idx, None, 17, 0, None)  # last_page_len > page_size
+    with pytest.raises(RuntimeError):
+        w.forward(q, q.clone(), pool, idx, None, 1, 4, None)  # last_page_idx outside the pool
+    with pytest.raises(RuntimeError):
+        w.forward(q.cpu(), q.clone(), pool, idx, None, 1, 0, None)
+    w.end_forward()
+    with pytest.raises(RuntimeError, match="BeginForward"):
+        w.forward(q, q.clone(), pool, idx, None, 1, 0, None)
+    w48 = _kernels.BatchDecodeWithPagedKVCachePyTorchWrapper(0)
+    w48.begin_forward(None, 32, 32, 48, 16, torch.empty(0, dtype=torch.float16))
+    q48 = torch.zeros((1, 32, 48), dtype=torch.float16, device=cuda)
+    pool48 = torch.zeros((4, 2, 16, 32, 48), dtype=torch.float16, device=cuda)
+    with pytest.raises(RuntimeError, match="head_dim"):
+        w48.forward(q48, q48.clone(), pool48, idx, None, 1, 0, None)

@@ -1,0 +1,211 @@
+"""GPU parity: RoPE, paged append (with the per-page key max/min metadata), their fusion, RMSNorm.
+
+RoPE tolerance.  The GPU forms the angle in float64 and rounds only sin/cos, so it is compared with
+the float64 closed form; the error budget is one rounding of the output dtype plus fp32 evaluation
+of x*cos +- y*sin: |err| <= 2^-11 |y| (fp16) / 2^-8 |y| (bf16) + 1e-6.  The reference's two own
+fp32 formulas (cpu_reference.h:36-53 and the model's, llama_tidaldecoding.py:248-279) differ from
+that closed form by up to position * 2^-23 rad; test_rope_reference_formulas_within_their_own_error
+checks both stay inside that bound at the positions the benchmark uses.
+Append must be bit-exact (copies); max/min metadata bit-exact against brute force.
+"""
+import numpy as np
+import pytest
+import torch
+
+from _util import PagedCase, randn
+
+pytestmark = pytest.mark.gpu
+
+ULP = {torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}
+
+
+def _rope_tol(want, dtype):
+    return ULP[dtype] * want.abs() * 1.01 + 2e-6
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("d", [64, 128, 256])
+@pytest.mark.parametrize("past,n_tok,theta,scale", [(0, 1, 1e4, 1.0), (4095, 1, 1e4, 1.0),
+                                                    (32767, 1, 1e4, 1.0), (102399, 1, 5e5, 1.0),
+                                                    (0, 300, 1e4, 1.0), (1000, 17, 5e5, 4.0)])
+def test_rope_in_place_against_closed_form(cuda, dtype, d, past, n_tok, theta, scale):
+    from oracle import tidal_oracle as orc
+    from tidaldecode_amd import _kernels
+
+    hq, hkv = 32, 8
+    q = randn((n_tok, hq, d), past + d, dtype)
+    k = randn((n_tok, hkv, d), past + d + 1, dtype)
+    pos = np.arange(past, past + n_tok)
+    want_q = torch.from_numpy(orc.rope_closed_form(q.numpy(), pos, theta, scale))
+    want_k = torch.from_numpy(orc.rope_closed_form(k.numpy(), pos, theta, scale))
+    qd, kd = q.to(dtype).to(cuda), k.to(dtype).to(cuda)
+    _kernels.apply_rope_in_place(qd, kd, past, scale, theta)
+    torch.cuda.synchronize()
+    assert ((qd.double().cpu() - want_q).abs() <= _rope_tol(want_q, dtype)).all()
+    assert ((kd.double().cpu() - want_k).abs() <= _rope_tol(want_k, dtype)).all()
+
+
+def test_rope_invariants(cuda):
+    """position 0 is the identity; pair norms are preserved; q_m . k_n depends on m - n only."""
+    from tidaldecode_amd import _kernels
+
+    dtype, d = torch.float16, 128
+    q = randn((1, 4, d), 1, dtype).to(dtype).to(cuda)
+    k = randn((1, 4, d), 2, dtype).to(dtype).to(cuda)
+    q0, k0 = q.clone(), k.clone()
+    _kernels.apply_rope_in_place(q, k, 0, 1.0, 1e4)
+    assert torch.equal(q, q0) and torch.equal(k, k0)
+    dots = []
+    for m, n in ((10, 3), (1010, 1003), (30010, 30003)):
+        qa, kb = q0.clone(), k0.clone()
+        dummy = torch.zeros_like(k0)
+        _kernels.apply_rope_in_place(qa, dummy, m, 1.0, 1e4)
+        dummy = torch.zeros_like(q0)
+        _kernels.apply_rope_in_place(dummy, kb, n, 1.0, 1e4)
+        dots.append((qa.float() * kb.float()).sum(-1))
+        pair = lambda x: x.float()[..., : d // 2] ** 2 + x.float()[..., d // 2:] ** 2
+        assert (pair(qa) - pair(q0)).abs().max() < 2e-2
+    assert (dots[0] - dots[1]).abs().max() < 0.1 and (dots[0] - dots[2]).abs().max() < 0.1
+
+
+def _append_case(cuda, dtype, layout, page_size, seq_before, n_new, d=128, h=8, with_meta=True):
+    """Append n_new tokens to a sequence holding seq_before tokens; returns device pools + oracle."""
+    from oracle import tidal_oracle as orc
+    from tidaldecode_amd import _kernels
+
+    seq_after = seq_before + n_new
+    case = PagedCase(seq_after, h, d, page_size, dtype, layout=layout, seed=seq_after + page_size)
+    # pool as it was before the append: oracle-append of the first seq_before tokens into garbage
+    shape = orc.pool_shape(case.max_pages, page_size, h, d, layout)
+    before = np.full(shape, 33.0, dtype=np.float32)
+    if seq_before:
+        orc.paged_append(before, case.page_table.tolist(), seq_before, case.k[:seq_before].numpy(),
+                         case.v[:seq_before].numpy(), layout)
+    want = before.copy()
+    orc.paged_append(want, case.page_table.tolist(), seq_after, case.k[seq_before:].numpy(),
+                     case.v[seq_before:].numpy(), layout)
+    pool = torch.from_numpy(before).to(dtype).to(cuda)
+    indices = case.page_table.to(torch.int32).to(cuda)
+    indptr = torch.tensor([0, case.n_pages], dtype=torch.int32, device=cuda)
+    # metadata pool: one entry per KV page, same page size; state before = brute force over the
+    # tokens already present
+    n_meta_pages = (case.n_pages + page_size - 1) // page_size
+    meta_table = torch.randperm(n_meta_pages + 2, generator=torch.Generator().manual_seed(1))[:n_meta_pages]
+    meta_shape = orc.pool_shape(n_meta_pages + 2, page_size, h, d, layout)
+    meta_before = np.full(meta_shape, 9.0, dtype=np.float32)
+    meta_want = None
+    if with_meta:
+        def brute(upto):
+            m = np.full(meta_shape, 9.0, dtype=np.float32)
+            for pg in range((upto + page_size - 1) // page_size):
+                rows = case.k[pg * page_size: min(upto, (pg + 1) * page_size)].numpy()
+                mp, me = int(meta_table[pg // page_size]), pg % page_size
+                if layout == 1:
+                    m[mp, 0, :, me, :], m[mp, 1, :, me, :] = rows.max(0), rows.min(0)
+                else:
+                    m[mp, 0, me, :, :], m[mp, 1, me, :, :] = rows.max(0), rows.min(0)
+            return m
+        meta_before = brute(seq_before)
+        meta_want = brute(seq_after)
+    meta = torch.from_numpy(meta_before).to(dtype).to(cuda)
+    fn = _kernels.append_kv_cache_decode if n_new == 1 else _kernels.append_kv_cache_prefill
+    kd = case.k[seq_before:].to(dtype).to(cuda).contiguous()
+    vd = case.v[seq_before:].to(dtype).to(cuda).contiguous()
+    fn(kd, vd, pool, indices, indptr, case.last_page_len, int(case.page_table[-1]),
+       meta if with_meta else torch.empty(0, device=cuda), meta_table.to(torch.int32).to(cuda),
+       torch.tensor([0, n_meta_pages], dtype=torch.int32, device=cuda),
+       (case.n_pages - 1) % page_size + 1, int(meta_table[-1]), layout)
+    torch.cuda.synchronize()
+    return pool.float().cpu().numpy(), want, meta.float().cpu().numpy(), meta_want
+
+
+@pytest.mark.parametrize("layout", [0, 1])
+@pytest.mark.parametrize("page_size", [1, 3, 7, 16, 31])
+def test_append_decode_and_prefill_bit_exact(cuda, layout, page_size):
+    """page sizes and lengths of the reference's page test (kernels/src/test/test_page.cu:620-684)"""
+    for dtype in (torch.float16, torch.bfloat16):
+        for seq_before, n_new in ((0, 17), (16, 1), (0, 1), (30, 1), (31, 1), (5, 250), (100, 4000 // 16),
+                                  (4099, 1)):
+            got, want, mgot, mwant = _append_case(cuda, dtype, layout, page_size, seq_before, n_new)
+            assert np.array_equal(got, want), (layout, page_size, dtype, seq_before, n_new)
+            assert np.array_equal(mgot, mwant), ("metadata", layout, page_size, dtype, seq_before, n_new)
+
+
+def test_multi_turn_append_round_trip(cuda):
+    """alternate prefill (<= 256 tokens) and decode appends, then gather through the page table
+    equals the contiguous K, V (test_page.cu multi-turn case)."""
+    from tidaldecode_amd import _kernels
+
+    dtype, h, d, page_size = torch.float16, 8, 128, 7
+    g = torch.Generator().manual_seed(3)
+    chunks = []
+    for i in range(10):
+        chunks.append(int(torch.randint(1, 257, (1,), generator=g)) if i % 2 == 0 else 1)
+    total = sum(chunks)
+    case = PagedCase(total, h, d, page_size, dtype, seed=77)
+    pool = torch.full(case.pool.shape, 5.0, dtype=dtype, device=cuda)
+    empty = torch.empty(0, device=cuda)
+    done = 0
+    for n_new in chunks:
+        done += n_new
+        n_pages = (done + page_size - 1) // page_size
+        idx = case.page_table[:n_pages].to(torch.int32).to(cuda)
+        indptr = torch.tensor([0, n_pages], dtype=torch.int32, device=cuda)
+        kd = case.k[done - n_new: done].to(dtype).to(cuda).contiguous()
+        vd = case.v[done - n_new: done].to(dtype).to(cuda).contiguous()
+        fn = _kernels.append_kv_cache_decode if n_new == 1 else _kernels.append_kv_cache_prefill
+        fn(kd, vd, pool, idx, indptr, (done - 1) % page_size + 1, int(idx[-1]), empty, idx, indptr,
+           1, 0, 0)
+    torch.cuda.synchronize()
+    pages = pool[case.page_table.to(cuda)]
+    kk = pages[:, 0].reshape(-1, h, d)[:total].float().cpu()
+    vv = pages[:, 1].reshape(-1, h, d)[:total].float().cpu()
+    assert torch.equal(kk, case.k) and torch.equal(vv, case.v)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("layout", [0, 1])
+def test_fused_rope_append_equals_the_two_calls(cuda, dtype, layout):
+    from oracle import tidal_oracle as orc
+    from tidaldecode_amd import _kernels
+
+    b, hq, hkv, d, page_size, pages = 5, 32, 8, 128, 16, 40
+    theta, scale = 5e5, 1.0
+    q = randn((b, hq, d), 1, dtype)
+    k = randn((b, hkv, d), 2, dtype)
+    v = randn((b, hkv, d), 3, dtype)
+    positions = torch.tensor([0, 15, 16, 333, 100000], dtype=torch.int32)
+    slots = torch.tensor([7 * 16 + 0, 2 * 16 + 15, 39 * 16 + 0, 11 * 16 + 13, 0 * 16 + 1], dtype=torch.int32)
+    shape = orc.pool_shape(pages, page_size, hkv, d, layout)
+    pool = torch.full(shape, 3.0, dtype=dtype, device=cuda)
+    qd = q.to(dtype).to(cuda)
+    _kernels.rope_append_decode(qd, k.to(dtype).to(cuda), v.to(dtype).to(cuda), pool,
+                                positions.to(cuda), slots.to(cuda), layout, scale, theta)
+    torch.cuda.synchronize()
+    want_pool = np.full(shape, 3.0, dtype=np.float32)
+    for i in range(b):
+        qi, ki = q[i:i + 1].to(dtype).to(cuda), k[i:i + 1].to(dtype).to(cuda)
+        _kernels.apply_rope_in_place(qi, ki, int(positions[i]), scale, theta)
+        assert torch.equal(qi[0], qd[i])
+        page, entry = int(slots[i]) // page_size, int(slots[i]) % page_size
+        if layout == 1:
+            want_pool[page, 0, :, entry, :] = ki[0].float().cpu().numpy()
+            want_pool[page, 1, :, entry, :] = v[i].numpy()
+        else:
+            want_pool[page, 0, entry, :, :] = ki[0].float().cpu().numpy()
+            want_pool[page, 1, entry, :, :] = v[i].numpy()
+    assert np.array_equal(pool.float().cpu().numpy(), want_pool)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rows,cols", [(1, 4096), (7, 5120), (300, 128), (2, 33)])
+def test_rms_norm(cuda, dtype, rows, cols):
+    from tidaldecode_amd import _kernels
+
+    x = randn((1, rows, cols), rows + cols, dtype)
+    w = randn((cols,), cols, dtype)
+    want = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-5) * w
+    out = torch.empty((1, rows, cols), dtype=dtype, device=cuda)
+    _kernels.rms_norm_forward(x.to(dtype).to(cuda), w.to(dtype).to(cuda), out, 1e-5)
+    torch.cuda.synchronize()
+    assert ((out.float().cpu() - want).abs() <= ULP[dtype] * 1.01 * want.abs() + 1e-6).all()

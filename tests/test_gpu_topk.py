@@ -1,0 +1,148 @@
+"""GPU parity: top-k selection (td_topk) and the cross-head score reduction (td_score_reduce).
+
+The index sets must be BIT-EXACT against the oracle's stable rule (k largest, ties to the lower
+position) when both see the same scores.  The oracle's rule itself is pinned in
+tests/test_oracle.py (torch.topk as sets, brute force on ties, the independent C qsort).
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _gpu_topk(values, k, cuda, in_idx=None, page_table=None, page_size=1, want_vals=True):
+    from tidaldecode_amd import _kernels
+
+    rows = values.shape[0]
+    out_idx = torch.full((rows, k), -1, dtype=torch.int32, device=cuda)
+    out_val = torch.zeros((rows, k), dtype=values.dtype, device=cuda) if want_vals else None
+    _kernels.topk_filtering(values.to(cuda), None if in_idx is None else in_idx.to(cuda), out_val,
+                            out_idx, None, k,
+                            page_table=None if page_table is None else page_table.to(cuda),
+                            page_size=page_size)
+    torch.cuda.synchronize()
+    return out_idx.cpu(), None if out_val is None else out_val.cpu()
+
+
+def _check(values, k, cuda):
+    from oracle import cref, tidal_oracle as orc
+
+    got, vals = _gpu_topk(values, k, cuda)
+    want = orc.stable_topk(values.float(), k)
+    assert torch.equal(got.long(), want), "index set differs from the stable oracle"
+    want_c = cref.stable_topk(values.float().numpy(), k)
+    assert np.array_equal(got.numpy(), want_c)
+    assert torch.equal(vals, torch.gather(values, 1, want))  # values travel with their index
+    return got
+
+
+@pytest.mark.parametrize("rows,n,k", [(32, 4096, 256), (32, 32768, 2048), (1, 32768, 2048),
+                                      (8, 102400, 4096), (32, 8192, 64), (3, 1000, 999),
+                                      (5, 70, 70), (2, 1, 1), (4, 63, 1), (4, 65, 64),
+                                      (2, 1025, 512), (1, 131072, 4096)])
+def test_random_scores_fp32(cuda, rows, n, k):
+    g = torch.Generator().manual_seed(rows * 1000003 + n + k)
+    _check(torch.randn((rows, n), generator=g), k, cuda)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rows,n,k", [(32, 8192, 256), (32, 4097, 128), (2, 50, 7)])
+def test_half_precision_scores_have_many_ties(cuda, dtype, rows, n, k):
+    """The reference feeds fp16 scores (tidal/ops/csrc/topk.cu:31-41): thousands of exact ties."""
+    g = torch.Generator().manual_seed(n + k)
+    _check(torch.randn((rows, n), generator=g).to(dtype), k, cuda)
+
+
+def test_ties_go_to_the_lower_position(cuda):
+    g = torch.Generator().manual_seed(7)
+    # 5 distinct values only: the threshold value occurs thousands of times
+    v = torch.randint(0, 5, (16, 20000), generator=g).float()
+    got = _check(v, 3000, cuda)
+    assert (got[:, 1:] > got[:, :-1]).all()  # ascending, no duplicates
+    # all equal: the first k positions
+    got = _check(torch.full((4, 5000), 1.25), 777, cuda)
+    assert torch.equal(got, torch.arange(777, dtype=torch.int32).repeat(4, 1))
+
+
+def test_signed_zero_inf_and_nan(cuda):
+    v = torch.zeros((2, 300))
+    v[0, 10::7] = -0.0          # -0 and +0 are equal: position decides
+    v[0, 5] = float("inf")
+    v[0, 6] = float("-inf")
+    v[0, 200] = float("nan")    # NaN orders above +inf, as in torch.topk / torch.sort
+    v[1] = -torch.arange(300).float()
+    v[1, 250] = float("nan")
+    for k in (1, 2, 50, 299, 300):
+        _check(v, k, cuda)
+
+
+def test_closed_forms(cuda):
+    g = torch.Generator().manual_seed(11)
+    v = torch.randn((32, 5000), generator=g)
+    got, _ = _gpu_topk(v, 1, cuda)
+    assert torch.equal(got[:, 0].long(), v.argmax(dim=1))
+    got, _ = _gpu_topk(v, 5000, cuda)
+    assert torch.equal(got, torch.arange(5000, dtype=torch.int32).repeat(32, 1))
+    # every unselected score <= the smallest selected one
+    got, vals = _gpu_topk(v, 321, cuda)
+    mask = torch.ones_like(v, dtype=torch.bool).scatter_(1, got.long(), False)
+    assert (v.masked_fill(~mask, float("-inf")).max(1).values <= vals.min(1).values).all()
+    # torch.topk agrees as a set (no ties in continuous data)
+    ref = torch.topk(v, 321, dim=-1).indices.sort(-1).values
+    assert torch.equal(got.long(), ref)
+
+
+def test_payloads(cuda):
+    """in_idx payload (the reference's meaning: physical page of each position), page-table
+    payload (token slots) and plain positions."""
+    from oracle import tidal_oracle as orc
+
+    g = torch.Generator().manual_seed(5)
+    rows, n, k, page = 8, 3000, 100, 16
+    v = torch.randn((rows, n), generator=g)
+    want = orc.stable_topk(v, k)
+    payload = torch.randint(0, 10**6, (rows, n), generator=g, dtype=torch.int32)
+    got, _ = _gpu_topk(v, k, cuda, in_idx=payload)
+    assert torch.equal(got, torch.gather(payload, 1, want))
+    n_pages = (n + page - 1) // page
+    table = torch.randperm(n_pages + 9, generator=g)[:n_pages].to(torch.int32)
+    got, _ = _gpu_topk(v, k, cuda, page_table=table, page_size=page)
+    assert torch.equal(got.long(), table.long()[want // page] * page + want % page)
+    # fewer payload columns than values: only those columns take part
+    got, _ = _gpu_topk(v, k, cuda, in_idx=payload[:, :500].contiguous())
+    assert torch.equal(got, torch.gather(payload, 1, orc.stable_topk(v[:, :500], k)))
+
+
+def test_topk_errors(cuda):
+    from tidaldecode_amd import _kernels
+
+    v = torch.zeros((4, 100), device=cuda)
+    out = torch.zeros((4, 10), dtype=torch.int32, device=cuda)
+    with pytest.raises(RuntimeError):
+        _kernels.topk_filtering(v, None, None, out, None, 11)            # out shape != k
+    with pytest.raises(RuntimeError):
+        _kernels.topk_filtering(v, None, None, out.long(), None, 10)     # not int32
+    with pytest.raises(RuntimeError):
+        _kernels.topk_filtering(v.double(), None, None, out, None, 10)   # dtype dispatch
+    big = torch.zeros((4, 200), dtype=torch.int32, device=cuda)
+    with pytest.raises(RuntimeError):
+        _kernels.topk_filtering(v, None, None, big, None, 200)           # k > len
+
+
+@pytest.mark.parametrize("hq,hkv,n", [(32, 32, 4096), (32, 8, 5000), (40, 40, 33), (32, 8, 1)])
+def test_score_reduce(cuda, hq, hkv, n):
+    """sum over heads of softmax probabilities, from logits + lse, against the closed form."""
+    from oracle import tidal_oracle as orc
+    from tidaldecode_amd import _kernels
+
+    g = torch.Generator().manual_seed(n)
+    logits = torch.randn((hq, n + 7), generator=g) * 3
+    lse = torch.logsumexp(logits[:, :n], dim=-1)
+    for mode, rows in (("head_sum", 1), ("group_sum", hkv)):
+        got = _kernels.score_reduce(logits.to(cuda), lse.to(cuda), hkv, n, mode).cpu()
+        want = orc.head_sum_scores(logits[:, :n], rows)
+        assert got.shape == want.shape
+        assert (got - want).abs().max() <= 2e-6 * hq
+        # probabilities of each head sum to one
+        assert (got.sum() - hq).abs() <= 1e-3 * hq

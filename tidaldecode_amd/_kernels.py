@@ -1,0 +1,447 @@
+"""Drop-in for the reference's PyBind module ``tidal._kernels`` (tidal/ops/csrc/bsk_ops.cu:4-20,
+declarations tidal/ops/csrc/bsk_ops.h:23-118), backed by ``libtidal_hip.so``.
+
+Same names, positional arguments and error behaviour (``RuntimeError`` on a failed check) as the
+reference.  Differences, all additive:
+
+* bf16 next to fp16; grouped-query attention (``num_qo_heads`` a multiple of ``num_kv_heads``);
+  batches (``q`` of shape ``[B, H, D]`` with ``indptr`` of length ``B + 1``); token-granular
+  index lists for ``page_size > 1`` (``index_kind="slots"``).
+* ``forward`` writes ``qk_product`` when a non-empty tensor is passed (the reference's binding
+  drops it, tidal/ops/csrc/approx_attn.cu:137) in list order, as natural-log-domain logits
+  ``q.k/sqrt(D)``.
+* kernels run on torch's current stream (the reference always uses the null stream, which is
+  torch's default current stream).
+"""
+import math
+from typing import Optional
+
+import torch
+
+from . import _lib
+from ._lib import (DecodePlan, IndexList, PagedKV, TD_BF16, TD_F16, TD_F32, TD_HND, TD_IDX_PAGES,
+                   TD_IDX_SLOTS, TD_NHD, check, lib)
+
+_DTYPES = {torch.float16: TD_F16, torch.bfloat16: TD_BF16, torch.float32: TD_F32}
+
+
+def _dtype_code(t: torch.dtype, what: str) -> int:
+    if t not in _DTYPES:
+        raise RuntimeError(f"{what} failed to dispatch with dtype {t}")
+    return _DTYPES[t]
+
+
+def _check_input(x: torch.Tensor, name: str) -> None:
+    # CHECK_INPUT of tidal/ops/csrc/pytorch_extension_utils.h:52-58
+    if not x.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not x.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+
+
+def _check_dim(d: int, x: torch.Tensor, name: str) -> None:
+    if x.dim() != d:
+        raise RuntimeError(f"{name} must be a {d}D tensor")
+
+
+def _check_i32(x: torch.Tensor, name: str) -> None:
+    if x.dtype != torch.int32:
+        raise RuntimeError(f"{name} must be int32")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(x: Optional[torch.Tensor]) -> Optional[int]:
+    return None if x is None or x.numel() == 0 else x.data_ptr()
+
+
+def _pool(kv_data: torch.Tensor, layout: int, name: str = "kv_data") -> PagedKV:
+    _check_input(kv_data, name)
+    _check_dim(5, kv_data, name)
+    if kv_data.size(1) != 2:
+        raise RuntimeError(f"{name}.size(1) must be 2")
+    if layout == TD_HND:
+        heads, page = kv_data.size(2), kv_data.size(3)
+    elif layout == TD_NHD:
+        page, heads = kv_data.size(2), kv_data.size(3)
+    else:
+        raise RuntimeError(f"Invalid layout {layout}")
+    return PagedKV(kv_data.data_ptr(), kv_data.size(0), heads, kv_data.size(4), page, layout,
+                   _dtype_code(kv_data.dtype, name))
+
+
+# ------------------------------------------------------------------------------------------
+# free functions
+# ------------------------------------------------------------------------------------------
+def apply_rope_in_place(q: torch.Tensor, k: torch.Tensor, past_kv_len: int, rope_scale: float,
+                        rope_theta: float) -> None:
+    """bsk_ops.h:23-27 / page.cu:212-253.  q ``[N, H_q, D]``, k ``[N, H_kv, D]``."""
+    _check_input(q, "q")
+    _check_input(k, "k")
+    _check_dim(3, q, "q")
+    _check_dim(3, k, "k")
+    if q.size(0) != k.size(0) or q.size(2) != k.size(2) or q.dtype != k.dtype:
+        raise RuntimeError("q and k must agree in tokens, head_dim and dtype")
+    check(lib.td_rope_in_place(q.data_ptr(), k.data_ptr(), q.size(0), q.size(1), k.size(1),
+                               q.size(2), int(past_kv_len), float(rope_scale), float(rope_theta),
+                               _dtype_code(q.dtype, "apply_rope_in_place"), _stream()))
+
+
+def rms_norm_forward(input: torch.Tensor, weight: torch.Tensor, output: torch.Tensor,
+                     epsilon: float) -> None:
+    """bsk_ops.h:29-32 / rms_norm.cu:160-212.  input/output ``[..., C]``, weight ``[C]``."""
+    _check_input(input, "input")
+    _check_input(weight, "weight")
+    _check_input(output, "output")
+    cols = input.size(-1)
+    if weight.numel() != cols or output.shape != input.shape or weight.dtype != input.dtype \
+            or output.dtype != input.dtype:
+        raise RuntimeError("rms_norm_forward: shape or dtype mismatch")
+    check(lib.td_rms_norm(input.data_ptr(), weight.data_ptr(), output.data_ptr(),
+                          input.numel() // cols, cols, float(epsilon),
+                          _dtype_code(input.dtype, "rms_norm_forward"), _stream()))
+
+
+def topk_filtering(estimated_value: torch.Tensor, estimated_indices: Optional[torch.Tensor],
+                   d_out: Optional[torch.Tensor], indices_out: torch.Tensor,
+                   buf: Optional[torch.Tensor], page_budget: int, *,
+                   page_table: Optional[torch.Tensor] = None, page_size: int = 1) -> None:
+    """bsk_ops.h:34-39 / topk.cu:7-44.  Row-wise top-``page_budget`` of ``estimated_value``
+    ``[H, len]``; ``indices_out[h, j]`` is ``estimated_indices[h, p]`` of the selected position
+    ``p``.  ``buf`` (RAFT scratch in the reference) is accepted and unused.
+
+    Deterministic where the reference is not: ties at the threshold go to the lower position
+    and each output row is sorted by position.  If ``estimated_indices`` has fewer columns than
+    ``estimated_value`` only those leading columns take part (the reference strides both by
+    ``estimated_value.size(1)``, kernels/include/topk/decode_select_k.cuh:53-55).
+
+    Extensions: ``estimated_indices=None`` returns positions, or physical token slots when a
+    ``page_table`` ``[n_pages]`` is given; fp32 values.
+    """
+    _check_input(estimated_value, "estimated_value")
+    _check_dim(2, estimated_value, "estimated_value")
+    rows, length = estimated_value.shape
+    in_ptr, in_stride = None, 0
+    if estimated_indices is not None:
+        _check_input(estimated_indices, "estimated_indices")
+        _check_dim(2, estimated_indices, "estimated_indices")
+        _check_i32(estimated_indices, "estimated_indices")
+        if estimated_indices.size(0) != rows:
+            raise RuntimeError("estimated_value and estimated_indices differ in rows")
+        length = min(length, estimated_indices.size(1))
+        in_ptr, in_stride = estimated_indices.data_ptr(), estimated_indices.size(1)
+    _check_input(indices_out, "indices_out")
+    _check_i32(indices_out, "indices_out")
+    k = int(page_budget)
+    if indices_out.dim() != 2 or indices_out.size(0) != rows or indices_out.size(1) != k:
+        raise RuntimeError(f"indices_out must be [{rows}, {k}]")
+    out_vals = None
+    if d_out is not None and d_out.numel() > 0:
+        _check_input(d_out, "d_out")
+        if d_out.shape != indices_out.shape or d_out.dtype != estimated_value.dtype:
+            raise RuntimeError("d_out must match indices_out in shape and estimated_value in dtype")
+        out_vals = d_out.data_ptr()
+    if k > length:
+        raise RuntimeError(f"page_budget {k} exceeds the row length {length}")
+    pt_ptr = None
+    if page_table is not None:
+        _check_input(page_table, "page_table")
+        _check_i32(page_table, "page_table")
+        if page_table.numel() * page_size < length:
+            raise RuntimeError("page_table does not cover the row")
+        pt_ptr = page_table.data_ptr()
+    check(lib.td_topk(estimated_value.data_ptr(),
+                      _dtype_code(estimated_value.dtype, "Top-k filtering"),
+                      estimated_value.stride(0), rows, length, k, in_ptr, in_stride, pt_ptr,
+                      int(page_size), out_vals, indices_out.data_ptr(), indices_out.stride(0),
+                      _stream()))
+
+
+def estimate_attn_score(*args, **kwargs):
+    """bsk_ops.h:41-48.  Page-level upper-bound estimator inherited from Quest; no TidalDecode
+    model code calls it (only tidal/utils/__init__.py:176-214 wraps it).  Not part of the
+    decode-attention path: raises."""
+    raise NotImplementedError(
+        "estimate_attn_score (Quest page estimator) is not used by TidalDecode's decode path and "
+        "is not provided by tidaldecode_amd")
+
+
+def _append(k, v, kv_data, kv_indices, kv_indptr, kv_last_page_len, metadata_data,
+            metadata_indices, metadata_indptr, metadata_last_page_len, layout, decode: bool):
+    # checks of tidal/ops/csrc/page.cu:19-55
+    for t, n in ((k, "k"), (v, "v"), (kv_indices, "kv_indices")):
+        _check_input(t, n)
+    _check_dim(3, k, "k")
+    _check_dim(3, v, "v")
+    _check_dim(1, kv_indices, "kv_indices")
+    _check_i32(kv_indices, "kv_indices")
+    _check_i32(kv_indptr, "kv_indptr")
+    if decode and (k.size(0) != 1 or v.size(0) != 1):
+        raise RuntimeError("append_kv_cache_decode expects k.size(0) == v.size(0) == 1")
+    if k.shape != v.shape or k.dtype != v.dtype:
+        raise RuntimeError("k and v must agree in shape and dtype")
+    pool = _pool(kv_data, int(layout))
+    if pool.num_kv_heads != k.size(1) or pool.head_dim != k.size(2) or kv_data.dtype != k.dtype:
+        raise RuntimeError("kv_data does not match k in heads, head_dim or dtype")
+    meta = None
+    if metadata_data is not None and metadata_data.numel() > 0:
+        meta = _pool(metadata_data, int(layout), "metadata_data")
+        _check_input(metadata_indices, "metadata_indices")
+        _check_dim(1, metadata_indices, "metadata_indices")
+        _check_i32(metadata_indices, "metadata_indices")
+        _check_i32(metadata_indptr, "metadata_indptr")
+    check(lib.td_append_kv(pool, k.data_ptr(), v.data_ptr(), k.size(0), kv_indices.data_ptr(),
+                           kv_indptr.data_ptr(), int(kv_last_page_len), meta,
+                           _ptr(metadata_indices) if meta is not None else None,
+                           _ptr(metadata_indptr) if meta is not None else None,
+                           int(metadata_last_page_len) if meta is not None else 0, _stream()))
+
+
+def append_kv_cache_prefill(k, v, kv_data, kv_indices, kv_indptr, kv_last_page_len,
+                            kv_last_page_idx, metadata_data, metadata_indices, metadata_indptr,
+                            metadata_last_page_len, metadata_last_page_idx, layout) -> None:
+    """bsk_ops.h:50-63 / page.cu:101-210.  Appends ``k.size(0)`` tokens."""
+    _append(k, v, kv_data, kv_indices, kv_indptr, kv_last_page_len, metadata_data,
+            metadata_indices, metadata_indptr, metadata_last_page_len, layout, decode=False)
+
+
+def append_kv_cache_decode(k, v, kv_data, kv_indices, kv_indptr, kv_last_page_len,
+                           kv_last_page_idx, metadata_data, metadata_indices, metadata_indptr,
+                           metadata_last_page_len, metadata_last_page_idx, layout) -> None:
+    """bsk_ops.h:65-78 / page.cu:6-99.  Appends the single new token."""
+    _append(k, v, kv_data, kv_indices, kv_indptr, kv_last_page_len, metadata_data,
+            metadata_indices, metadata_indptr, metadata_last_page_len, layout, decode=True)
+
+
+def rope_append_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, kv_data: torch.Tensor,
+                       positions: torch.Tensor, dst_slot: torch.Tensor, layout: int,
+                       rope_scale: float = 1.0, rope_theta: float = 1e4) -> None:
+    """Extension: ``apply_rope_in_place`` + ``append_kv_cache_decode`` in one launch for a batch.
+    q ``[B, H_q, D]`` is rotated in place; rotated k and v ``[B, H_kv, D]`` go to physical slot
+    ``dst_slot[b]``; ``positions[b]`` is the token's position."""
+    for t, n in ((q, "q"), (k, "k"), (v, "v"), (positions, "positions"), (dst_slot, "dst_slot")):
+        _check_input(t, n)
+    _check_dim(3, q, "q")
+    _check_dim(3, k, "k")
+    _check_i32(positions, "positions")
+    _check_i32(dst_slot, "dst_slot")
+    pool = _pool(kv_data, int(layout))
+    b = q.size(0)
+    if k.shape != v.shape or k.size(0) != b or k.size(1) != pool.num_kv_heads or \
+            q.size(2) != pool.head_dim or k.size(2) != pool.head_dim or \
+            not (q.dtype == k.dtype == v.dtype == kv_data.dtype):
+        raise RuntimeError("rope_append_decode: q/k/v/kv_data disagree in shape or dtype")
+    if positions.numel() != b or dst_slot.numel() != b:
+        raise RuntimeError("rope_append_decode: positions and dst_slot must hold one entry per sequence")
+    check(lib.td_rope_append_decode(pool, q.data_ptr(), k.data_ptr(), v.data_ptr(), b, q.size(1),
+                                    positions.data_ptr(), dst_slot.data_ptr(), float(rope_scale),
+                                    float(rope_theta), _stream()))
+
+
+def prefill_with_paged_kv_cache(q, kv_data, kv_indices, kv_last_page_len, causal, layout,
+                                allow_fp16_qk_reduction, rope_scale, rope_theta) -> torch.Tensor:
+    """bsk_ops.h:80-88 / batch_prefill.cu:27-117.  Causal attention of the ``q.size(0)`` newest
+    tokens over the paged cache.  Prefill runs once per sequence and is not on the decode path;
+    it is served by gathering the pages and calling torch's fused SDPA on the GPU."""
+    _check_input(q, "q")
+    _check_dim(3, q, "q")
+    pool = _pool(kv_data, int(layout))
+    n_pages = kv_indices.numel()
+    kv_len = (n_pages - 1) * pool.page_size + int(kv_last_page_len)
+    pages = kv_data.index_select(0, kv_indices.long())  # [n, 2, P, H, D] or [n, 2, H, P, D]
+    if int(layout) == TD_HND:
+        pages = pages.permute(0, 1, 3, 2, 4)
+    kk = pages[:, 0].reshape(n_pages * pool.page_size, pool.num_kv_heads, pool.head_dim)[:kv_len]
+    vv = pages[:, 1].reshape(n_pages * pool.page_size, pool.num_kv_heads, pool.head_dim)[:kv_len]
+    hq = q.size(1)
+    group = hq // pool.num_kv_heads
+    qq = q.transpose(0, 1).unsqueeze(0)  # [1, Hq, N, D]
+    kk = kk.transpose(0, 1).repeat_interleave(group, 0).unsqueeze(0)
+    vv = vv.transpose(0, 1).repeat_interleave(group, 0).unsqueeze(0)
+    n = q.size(0)
+    if causal and n == kv_len:
+        o = torch.nn.functional.scaled_dot_product_attention(qq, kk, vv, is_causal=True)
+    else:
+        mask = None
+        if causal and n > 1:
+            qpos = torch.arange(kv_len - n, kv_len, device=q.device).unsqueeze(1)
+            mask = torch.arange(kv_len, device=q.device).unsqueeze(0) <= qpos
+        o = torch.nn.functional.scaled_dot_product_attention(qq, kk, vv, attn_mask=mask)
+    return o.squeeze(0).transpose(0, 1).contiguous()
+
+
+# ------------------------------------------------------------------------------------------
+# decode attention handler
+# ------------------------------------------------------------------------------------------
+class BatchDecodeWithPagedKVCachePyTorchWrapper:
+    """bsk_ops.h:90-118 / approx_attn.cu:27-151.  ``begin_forward`` fixes the head geometry,
+    ``forward`` may then be called for any number of layers, ``end_forward`` closes the
+    bracket.  The split plan is recomputed (host arithmetic only) whenever the list shape
+    changes; the scratch buffer grows on demand and is kept between brackets."""
+
+    def __init__(self, layout: int):
+        if layout not in (TD_NHD, TD_HND):
+            raise RuntimeError(f"Invalid layout {layout}")
+        self._layout = int(layout)
+        self._begun = False
+        self._geom = None
+        self._plans = {}
+        self._workspace = None
+        self.waves_per_block = 0  # 0 = library default; tuning knob
+        self.fused_merge = -1     # -1 = library default
+        self.chunk_tokens = 0     # 0 = library default
+
+    def begin_forward(self, indptr: torch.Tensor, num_qo_heads: int, num_kv_heads: int,
+                      head_dim: int, page_size: int, empty_data: torch.Tensor) -> None:
+        if indptr is not None:
+            _check_dim(1, indptr, "indptr")
+            _check_i32(indptr, "indptr")
+        _dtype_code(empty_data.dtype, "BatchDecodeWithPagedKVCache")
+        if empty_data.dtype == torch.float32:
+            raise RuntimeError("BatchDecodeWithPagedKVCache failed to dispatch with dtype "
+                               f"{empty_data.dtype}")
+        if num_qo_heads % num_kv_heads != 0:
+            raise RuntimeError(f"num_qo_heads {num_qo_heads} is not a multiple of num_kv_heads "
+                               f"{num_kv_heads}")
+        self._geom = (int(num_qo_heads), int(num_kv_heads), int(head_dim), int(page_size),
+                      empty_data.dtype)
+        self._plans.clear()
+        self._begun = True
+
+    def end_forward(self) -> None:
+        self._begun = False
+        self._plans.clear()
+
+    def _plan(self, batch: int, idx_rows: int, max_items: int) -> DecodePlan:
+        key = (batch, idx_rows, max_items, self.waves_per_block, self.fused_merge,
+               self.chunk_tokens)
+        plan = self._plans.get(key)
+        if plan is None:
+            hq, hkv, d, _, _ = self._geom
+            plan = DecodePlan(self.chunk_tokens, 0, self.waves_per_block, self.fused_merge, 0)
+            check(lib.td_decode_make_plan(batch, hq, hkv, d, idx_rows, max_items, plan))
+            self._plans[key] = plan
+        return plan
+
+    def forward(self, q: torch.Tensor, o: torch.Tensor, paged_kv_data: torch.Tensor,
+                paged_kv_indices: torch.Tensor, paged_kv_indptr: Optional[torch.Tensor],
+                paged_kv_last_page_len, paged_kv_last_page_idx,
+                qk_product: Optional[torch.Tensor], rope_scale: float = 1.0,
+                rope_theta: float = 1e4, *, index_kind: str = "pages",
+                lse: Optional[torch.Tensor] = None, n_list: Optional[int] = None) -> None:
+        """q, o ``[B, H_q, D]``; ``paged_kv_indices`` ``[rows, budget]`` int32 with rows in
+        {H_q, H_kv, 1}; sequence b uses columns ``indptr[b]:indptr[b+1]`` of every row and then
+        the first ``last_page_len`` entries of page ``last_page_idx`` (ints, or int32 device
+        tensors ``[B]``).  ``index_kind="slots"`` reads the entries as token slots.
+        ``n_list`` bounds the per-sequence column count (default: all columns).
+        rope_scale / rope_theta are accepted for signature parity; RoPE is applied before the
+        cache is written (RotaryMode::kNone in the reference, approx_attn.cu:52,139)."""
+        if not self._begun:
+            raise RuntimeError("Please call BatchDecodeHandler's BeginForward() before calling "
+                               "BatchDecodeWithPagedKVCacheWrapper()")
+        _check_input(q, "q")
+        _check_input(o, "o")
+        _check_input(paged_kv_indices, "paged_kv_indices")
+        _check_dim(3, q, "q")
+        _check_dim(2, paged_kv_indices, "paged_kv_indices")
+        _check_i32(paged_kv_indices, "paged_kv_indices")
+        pool = _pool(paged_kv_data, self._layout, "paged_kv_data")
+        hq, hkv, d, page, dtype = self._geom
+        batch = q.size(0)
+        if q.size(1) != hq or q.size(2) != d or pool.num_kv_heads != hkv or pool.head_dim != d \
+                or pool.page_size != page:
+            raise RuntimeError("forward: q / paged_kv_data do not match begin_forward's geometry")
+        if q.dtype != dtype or paged_kv_data.dtype != dtype or o.dtype != dtype:
+            raise RuntimeError(f"BatchDecodeWithPagedKVCache failed to dispatch with dtype {q.dtype}")
+        if o.shape != q.shape:
+            raise RuntimeError("o must have the shape of q")
+        rows, budget = paged_kv_indices.shape
+        if rows not in (1, hkv, hq):
+            raise RuntimeError(f"paged_kv_indices.size(0) must be 1, {hkv} or {hq}")
+        if index_kind not in ("pages", "slots"):
+            raise KeyError(f"Invalid index_kind {index_kind}")
+        kind = TD_IDX_PAGES if index_kind == "pages" else TD_IDX_SLOTS
+
+        lst = IndexList()
+        lst.idx = _ptr(paged_kv_indices)
+        lst.idx_rows = rows
+        lst.idx_row_stride = paged_kv_indices.stride(0)
+        lst.kind = kind
+        if paged_kv_indptr is not None:
+            _check_i32(paged_kv_indptr, "paged_kv_indptr")
+            if paged_kv_indptr.numel() != batch + 1:
+                raise RuntimeError("paged_kv_indptr must hold batch + 1 entries")
+            lst.indptr = paged_kv_indptr.data_ptr()
+        lst.n_list_host = budget if n_list is None else min(int(n_list), budget)
+        max_last = 0
+        if isinstance(paged_kv_last_page_len, torch.Tensor):
+            _check_i32(paged_kv_last_page_len, "paged_kv_last_page_len")
+            lst.last_page_len_arr = paged_kv_last_page_len.data_ptr()
+            max_last = page
+        else:
+            lst.last_page_len = int(paged_kv_last_page_len)
+            max_last = lst.last_page_len
+        if isinstance(paged_kv_last_page_idx, torch.Tensor):
+            _check_i32(paged_kv_last_page_idx, "paged_kv_last_page_idx")
+            lst.last_page_idx_arr = paged_kv_last_page_idx.data_ptr()
+        else:
+            lst.last_page_idx = int(paged_kv_last_page_idx)
+
+        max_items = lst.n_list_host * (page if kind == TD_IDX_PAGES else 1) + max_last
+        plan = self._plan(batch, rows, max_items)
+        if plan.workspace_bytes > 0 and (self._workspace is None or
+                                         self._workspace.numel() < plan.workspace_bytes or
+                                         self._workspace.device != q.device):
+            self._workspace = torch.zeros(int(plan.workspace_bytes), dtype=torch.uint8,
+                                          device=q.device)
+
+        scores_ptr, scores_dtype, score_stride = None, TD_F32, 0
+        if qk_product is not None and qk_product.numel() > 0:
+            _check_input(qk_product, "qk_product")
+            if qk_product.numel() % (batch * hq) != 0:
+                raise RuntimeError("qk_product must be [B * H_q, stride]")
+            score_stride = qk_product.numel() // (batch * hq)
+            if score_stride < max_items:
+                raise RuntimeError(f"qk_product rows hold {score_stride} entries, the list has "
+                                   f"up to {max_items}")
+            scores_ptr = qk_product.data_ptr()
+            scores_dtype = _dtype_code(qk_product.dtype, "qk_product")
+        lse_ptr = None
+        if lse is not None:
+            _check_input(lse, "lse")
+            if lse.dtype != torch.float32 or lse.numel() != batch * hq:
+                raise RuntimeError("lse must be float32 [B, H_q]")
+            lse_ptr = lse.data_ptr()
+        ws = self._workspace
+        check(lib.td_decode_attn(pool, lst, plan, q.data_ptr(), o.data_ptr(), batch, hq,
+                                 1.0 / math.sqrt(d), scores_ptr, scores_dtype, score_stride,
+                                 lse_ptr, ws.data_ptr() if ws is not None else None,
+                                 ws.numel() if ws is not None else 0, _stream()))
+
+
+def score_reduce(logits: torch.Tensor, lse: torch.Tensor, num_kv_heads: int, n: int,
+                 mode: str = "head_sum", out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Extension: sum of softmax probabilities over query heads.  logits float32 ``[H_q, stride]``,
+    lse float32 ``[H_q]``; returns float32 ``[1, n]`` (``head_sum``) or ``[H_kv, n]``
+    (``group_sum``)."""
+    _check_input(logits, "logits")
+    _check_input(lse, "lse")
+    _check_dim(2, logits, "logits")
+    if logits.dtype != torch.float32 or lse.dtype != torch.float32:
+        raise RuntimeError("score_reduce expects float32 logits and lse")
+    hq = logits.size(0)
+    if lse.numel() != hq:
+        raise RuntimeError("lse must hold one entry per query head")
+    if mode not in ("head_sum", "group_sum"):
+        raise KeyError(f"Invalid score reduce mode {mode}")
+    rows = 1 if mode == "head_sum" else int(num_kv_heads)
+    if out is None:
+        out = torch.empty((rows, n), dtype=torch.float32, device=logits.device)
+    check(lib.td_score_reduce(logits.data_ptr(), logits.stride(0), lse.data_ptr(), hq,
+                              int(num_kv_heads), int(n),
+                              _lib.TD_REDUCE_HEAD_SUM if mode == "head_sum"
+                              else _lib.TD_REDUCE_GROUP_SUM,
+                              out.data_ptr(), out.stride(0), _stream()))
+    return out

@@ -1,0 +1,159 @@
+// Shared device/host helpers for the gfx950 kernels of libtidal_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "../../include/tidal_hip.h"
+
+namespace tidal {
+
+// ---------------------------------------------------------------------------------------------
+// Error reporting (host)
+// ---------------------------------------------------------------------------------------------
+char* error_buffer();  // thread-local, 512 bytes, defined in capi.hip
+
+inline int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(error_buffer(), 512, fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+#define TD_REQUIRE(cond, ...)                                         \
+  do {                                                                \
+    if (!(cond)) return ::tidal::fail(TD_ERR_INVALID_ARG, __VA_ARGS__); \
+  } while (0)
+
+#define TD_HIP_CHECK(expr)                                                                   \
+  do {                                                                                       \
+    hipError_t e_ = (expr);                                                                  \
+    if (e_ != hipSuccess)                                                                    \
+      return ::tidal::fail(TD_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(e_));       \
+  } while (0)
+
+// ---------------------------------------------------------------------------------------------
+// Vector types: one lane moves 16 bytes (8 two-byte elements) per global access.
+// ---------------------------------------------------------------------------------------------
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+struct F16 {};   // tag types for the two KV element formats
+struct BF16 {};
+
+// dot of two packed pairs, fp32 accumulate (v_dot2_f32_f16 / v_dot2_f32_bf16)
+template <typename T>
+__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c);
+template <>
+__device__ __forceinline__ float dot2<F16>(uint32_t a, uint32_t b, float c) {
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c,
+                                false);
+}
+template <>
+__device__ __forceinline__ float dot2<BF16>(uint32_t a, uint32_t b, float c) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a),
+                                         __builtin_bit_cast(bf16x2, b), c, false);
+}
+
+// unpack a packed pair to two floats
+template <typename T>
+__device__ __forceinline__ void unpack2(uint32_t w, float& lo, float& hi);
+template <>
+__device__ __forceinline__ void unpack2<F16>(uint32_t w, float& lo, float& hi) {
+  f16x2 h = __builtin_bit_cast(f16x2, w);
+  lo = (float)h.x;
+  hi = (float)h.y;
+}
+template <>
+__device__ __forceinline__ void unpack2<BF16>(uint32_t w, float& lo, float& hi) {
+  lo = __builtin_bit_cast(float, w << 16);
+  hi = __builtin_bit_cast(float, w & 0xffff0000u);
+}
+
+// round-to-nearest-even pack of two floats
+template <typename T>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi);
+template <>
+__device__ __forceinline__ uint32_t pack2<F16>(float lo, float hi) {
+  f16x2 h;
+  h.x = (_Float16)lo;
+  h.y = (_Float16)hi;
+  return __builtin_bit_cast(uint32_t, h);
+}
+__device__ __forceinline__ uint32_t bf16_bits_rne(float f) {
+  uint32_t u = __builtin_bit_cast(uint32_t, f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;  // quiet NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+template <>
+__device__ __forceinline__ uint32_t pack2<BF16>(float lo, float hi) {
+  return bf16_bits_rne(lo) | (bf16_bits_rne(hi) << 16);
+}
+
+// scalar conversions (used by the small kernels)
+template <typename T>
+__device__ __forceinline__ float to_float(uint16_t b);
+template <>
+__device__ __forceinline__ float to_float<F16>(uint16_t b) {
+  return (float)__builtin_bit_cast(_Float16, b);
+}
+template <>
+__device__ __forceinline__ float to_float<BF16>(uint16_t b) {
+  return __builtin_bit_cast(float, (uint32_t)b << 16);
+}
+template <typename T>
+__device__ __forceinline__ uint16_t from_float(float f);
+template <>
+__device__ __forceinline__ uint16_t from_float<F16>(float f) {
+  return __builtin_bit_cast(uint16_t, (_Float16)f);
+}
+template <>
+__device__ __forceinline__ uint16_t from_float<BF16>(float f) {
+  return (uint16_t)bf16_bits_rne(f);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Cross-lane sums inside a group of W adjacent lanes (W = 8, 16 or 32) of a 64-wide wavefront,
+// result in every lane of the group.  DPP modifiers fold into the v_add_f32.
+// ---------------------------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float x) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
+}
+
+template <int W>
+__device__ __forceinline__ float group_sum(float x) {
+  static_assert(W == 8 || W == 16 || W == 32, "lane group width");
+  x += dpp_move<0xB1>(x);   // quad_perm [1,0,3,2]
+  x += dpp_move<0x4E>(x);   // quad_perm [2,3,0,1]
+  x += dpp_move<0x141>(x);  // row_half_mirror: other quad of the 8-lane half row
+  if constexpr (W >= 16) x += dpp_move<0x140>(x);  // row_mirror: other half of the 16-lane row
+  if constexpr (W >= 32) {
+    // xor 16 inside each 32-lane half: ds_swizzle bit-mask mode, and=0x1f or=0 xor=0x10
+    x += __builtin_bit_cast(
+        float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, x), (0x10 << 10) | 0x1f));
+  }
+  return x;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr float kNegBig = -1.0e30f;  // finite stand-in for -inf in running maxima
+
+__host__ __device__ __forceinline__ int64_t ceil_div64(int64_t a, int64_t b) {
+  return (a + b - 1) / b;
+}
+
+}  // namespace tidal

@@ -1,0 +1,706 @@
+// Decode attention over a paged KV pool for gfx950 (MI355X): one new query token per sequence
+// attends to a listed subset of the cache (sparse layers), or to the whole cache while emitting
+// per-token logits (token-selection layers).
+//
+// Mapping.  A K or V row of one head is head_dim two-byte elements; LPR = head_dim/8 adjacent
+// lanes hold it, 16 bytes (one global_load_dwordx4) per lane, so a 64-wide wavefront carries
+// HPW = 64/LPR "head rows" at once and never reduces across more than one DPP row for
+// head_dim 128.  A workgroup owns one group of HPW head rows and one chunk of the token list;
+// its waves take interleaved tiles of U tokens, each wave keeping a private online-softmax
+// state in base 2.  Wave states are merged through LDS, workgroup results through a fp32
+// partial buffer that the last-arriving workgroup of a head group reduces (ticket counter), or
+// that a second small kernel reduces when the plan asks for it.
+//
+// With grouped-query attention and an index list shared by the query heads of a KV head
+// (QPG > 1) each lane group loads the KV row once and scores it against QPG query heads.
+//
+// Semantics follow kernels/include/decode/decode_attn.cuh:432-658 of the reference
+// (BatchDecodeWithPagedKVCacheKernel) including the forced last page
+// (decode_page.cuh:320-346) and the logits output (decode_attn.cuh:107-109).
+
+#include "common.cuh"
+
+namespace tidal {
+
+struct DecodeParams {
+  const void* q;
+  void* o;
+  const void* kv;
+  int64_t page_stride;   // elements from page p to page p+1  (2 * P * H_kv * D)
+  int64_t v_offset;      // elements from a K row to its V row (P * H_kv * D)
+  int32_t entry_stride;  // elements between consecutive tokens of a page
+  int32_t head_stride;   // elements between consecutive KV heads of a token
+  int32_t page_size;
+  int32_t page_shift;  // log2(page_size) or -1
+  uint32_t max_slot;   // max_pages * page_size - 1
+  uint32_t max_page;   // max_pages - 1
+  int32_t page_mode;   // 1: list entries are pages, 0: token slots
+  int32_t num_qo_heads;
+  int32_t n_hrows;   // head rows: num_qo_heads (QPG == 1) or num_kv_heads (QPG > 1)
+  int32_t q_per_kv;  // query heads per KV head (used when QPG == 1)
+  // index list
+  const int32_t* idx;
+  int32_t idx_row_stride;  // 0 for a shared row
+  int32_t idx_per_kv;      // 1: rows are per KV head while QPG == 1
+  const int32_t* indptr;
+  int32_t n_list_host;
+  const int32_t* last_len_arr;
+  const int32_t* last_idx_arr;
+  int32_t last_len;
+  int32_t last_idx;
+  // split
+  int32_t chunk_tokens;
+  int32_t max_splits;
+  int32_t fused_merge;
+  float scale_log2;  // sm_scale * log2(e)
+  // outputs
+  void* scores;
+  int32_t scores_f32;
+  int64_t score_stride;
+  float* lse;
+  float* ws_o;      // [batch * H_q * max_splits, D]
+  float* ws_ml;     // [batch * H_q * max_splits, 2]
+  int32_t* ws_cnt;  // [batch * head_groups]
+};
+
+__device__ __forceinline__ void divmod_page(const DecodeParams& p, uint32_t x, uint32_t& page,
+                                            uint32_t& entry) {
+  if (p.page_shift >= 0) {
+    page = x >> p.page_shift;
+    entry = x & ((1u << p.page_shift) - 1u);
+  } else {
+    page = x / (uint32_t)p.page_size;
+    entry = x - page * (uint32_t)p.page_size;
+  }
+}
+
+// Per-sequence view of the token list.
+struct SeqList {
+  const int32_t* row;  // this lane group's index row, already offset to the sequence
+  int32_t n_list;      // listed entries (pages or slots)
+  int32_t n_items;     // tokens attended
+  int32_t last_len;
+  int32_t last_idx;
+};
+
+// Element offset of the K row of item i (slot clamped into the pool); items past the end map
+// to slot 0, a valid address whose contribution is masked out.
+template <bool PAGE_MODE>
+__device__ __forceinline__ int64_t item_offset(const DecodeParams& p, const SeqList& s, int32_t i,
+                                               int32_t kv_head_off) {
+  uint32_t page = 0, entry = 0;
+  if (i < s.n_items) {
+    if constexpr (PAGE_MODE) {
+      uint32_t li, e;
+      divmod_page(p, (uint32_t)i, li, e);
+      page = ((int32_t)li < s.n_list) ? (uint32_t)s.row[li] : (uint32_t)s.last_idx;
+      entry = e;
+      page = page > p.max_page ? p.max_page : page;
+    } else {
+      uint32_t slot = (i < s.n_list) ? (uint32_t)s.row[i]
+                                     : (uint32_t)s.last_idx * (uint32_t)p.page_size +
+                                           (uint32_t)(i - s.n_list);
+      slot = slot > p.max_slot ? p.max_slot : slot;
+      divmod_page(p, slot, page, entry);
+    }
+  }
+  return (int64_t)page * p.page_stride + (int64_t)entry * p.entry_stride + kv_head_off;
+}
+
+template <typename T, int D, int QPG, int U, int NW, bool PAGE_MODE, bool EMIT>
+__global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams p) {
+  constexpr int LPR = D / 8;     // lanes per row
+  constexpr int HPW = 64 / LPR;  // head rows per wave
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int g = lane / LPR;   // lane group = head row inside the wave
+  const int li = lane % LPR;  // 16-byte column of the row
+  const int hg = blockIdx.x;
+  const int split = blockIdx.y;
+  const int b = blockIdx.z;
+
+  const int hrow_raw = hg * HPW + g;
+  const bool head_ok = hrow_raw < p.n_hrows;
+  const int hrow = head_ok ? hrow_raw : p.n_hrows - 1;
+  const int kv_head = (QPG > 1) ? hrow : hrow / p.q_per_kv;
+  const int qh0 = hrow * QPG;  // first query head of this lane group
+
+  // sequence descriptor
+  SeqList s;
+  int list_beg = 0;
+  if (p.indptr) {
+    list_beg = p.indptr[b];
+    s.n_list = p.indptr[b + 1] - list_beg;
+  } else {
+    s.n_list = p.n_list_host;
+  }
+  s.n_list = s.n_list < 0 ? 0 : (s.n_list > p.n_list_host ? p.n_list_host : s.n_list);
+  s.last_len = p.last_len_arr ? p.last_len_arr[b] : p.last_len;
+  s.last_idx = p.last_idx_arr ? p.last_idx_arr[b] : p.last_idx;
+  s.n_items = (PAGE_MODE ? s.n_list * p.page_size : s.n_list) + s.last_len;
+  const int idx_row = (QPG == 1 && p.idx_per_kv) ? kv_head : hrow;
+  s.row = p.idx + (int64_t)idx_row * p.idx_row_stride + list_beg;
+
+  int n_splits = (s.n_items + p.chunk_tokens - 1) / p.chunk_tokens;
+  n_splits = n_splits < 1 ? 1 : n_splits;
+  if (split >= n_splits) return;  // uniform for the whole workgroup
+
+  const int c0 = split * p.chunk_tokens;
+  int c1 = c0 + p.chunk_tokens;
+  c1 = c1 > s.n_items ? s.n_items : c1;
+
+  // query: QPG heads x 8 elements per lane, kept packed in the KV dtype
+  uint32_t qp[QPG][4];
+  {
+    const u32x4* qptr =
+        reinterpret_cast<const u32x4*>(p.q) + ((int64_t)b * p.num_qo_heads + qh0) * LPR + li;
+#pragma unroll
+    for (int j = 0; j < QPG; ++j) {
+      u32x4 v = qptr[j * LPR];
+      qp[j][0] = v.x;
+      qp[j][1] = v.y;
+      qp[j][2] = v.z;
+      qp[j][3] = v.w;
+    }
+  }
+
+  float m[QPG], l[QPG], acc[QPG][8];
+#pragma unroll
+  for (int j = 0; j < QPG; ++j) {
+    m[j] = kNegBig;
+    l[j] = 0.f;
+#pragma unroll
+    for (int d = 0; d < 8; ++d) acc[j][d] = 0.f;
+  }
+
+  const int kv_head_off = kv_head * p.head_stride + li * 8;
+  const uint16_t* kv16 = reinterpret_cast<const uint16_t*>(p.kv);
+
+  // ---- tile pipeline: loads of tile t+1 are in flight while tile t is reduced ----
+  u32x4 kA[U], vA[U], kB[U], vB[U];
+  int64_t offN[U];  // element offsets of the tile whose loads are issued next
+
+  auto lookup = [&](int base) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      int i = base + u;
+      offN[u] = item_offset<PAGE_MODE>(p, s, i < c1 ? i : s.n_items, kv_head_off);
+    }
+  };
+  auto issue = [&](u32x4(&kb)[U], u32x4(&vb)[U]) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      kb[u] = *reinterpret_cast<const u32x4*>(kv16 + offN[u]);
+      vb[u] = *reinterpret_cast<const u32x4*>(kv16 + offN[u] + p.v_offset);
+    }
+  };
+  auto reduce = [&](const u32x4(&kb)[U], const u32x4(&vb)[U], int base) {
+    float sc[QPG][U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const bool valid = base + u < c1;
+#pragma unroll
+      for (int j = 0; j < QPG; ++j) {
+        float a = dot2<T>(qp[j][0], kb[u].x, 0.f);
+        a = dot2<T>(qp[j][1], kb[u].y, a);
+        a = dot2<T>(qp[j][2], kb[u].z, a);
+        a = dot2<T>(qp[j][3], kb[u].w, a);
+        a = group_sum<LPR>(a) * p.scale_log2;
+        sc[j][u] = valid ? a : kNegBig;
+        if constexpr (EMIT) {
+          if (valid && head_ok && li == 0) {
+            const int64_t at =
+                ((int64_t)b * p.num_qo_heads + qh0 + j) * p.score_stride + (base + u);
+            const float nat = a * kLn2;
+            if (p.scores_f32)
+              reinterpret_cast<float*>(p.scores)[at] = nat;
+            else
+              reinterpret_cast<uint16_t*>(p.scores)[at] = from_float<T>(nat);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < QPG; ++j) {
+      float mt = sc[j][0];
+#pragma unroll
+      for (int u = 1; u < U; ++u) mt = fmaxf(mt, sc[j][u]);
+      const float m_new = fmaxf(m[j], mt);
+      const float alpha = fast_exp2(m[j] - m_new);
+      m[j] = m_new;
+      float pr[U];
+      float ps = 0.f;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        pr[u] = (base + u < c1) ? fast_exp2(sc[j][u] - m_new) : 0.f;
+        ps += pr[u];
+      }
+      l[j] = l[j] * alpha + ps;
+#pragma unroll
+      for (int d = 0; d < 8; ++d) acc[j][d] *= alpha;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        float v0, v1, v2, v3, v4, v5, v6, v7;
+        unpack2<T>(vb[u].x, v0, v1);
+        unpack2<T>(vb[u].y, v2, v3);
+        unpack2<T>(vb[u].z, v4, v5);
+        unpack2<T>(vb[u].w, v6, v7);
+        acc[j][0] = fmaf(pr[u], v0, acc[j][0]);
+        acc[j][1] = fmaf(pr[u], v1, acc[j][1]);
+        acc[j][2] = fmaf(pr[u], v2, acc[j][2]);
+        acc[j][3] = fmaf(pr[u], v3, acc[j][3]);
+        acc[j][4] = fmaf(pr[u], v4, acc[j][4]);
+        acc[j][5] = fmaf(pr[u], v5, acc[j][5]);
+        acc[j][6] = fmaf(pr[u], v6, acc[j][6]);
+        acc[j][7] = fmaf(pr[u], v7, acc[j][7]);
+      }
+    }
+  };
+
+  constexpr int STEP = NW * U;  // tokens between two tiles of one wave
+  int t = c0 + wave * U;        // first token of this wave's current tile
+  if (t < c1) {
+    lookup(t);
+    issue(kA, vA);
+    while (true) {
+      // stage A holds tile t
+      const int tn = t + STEP;
+      if (tn < c1) {
+        lookup(tn);
+        issue(kB, vB);
+      }
+      reduce(kA, vA, t);
+      if (tn >= c1) break;
+      const int tnn = tn + STEP;
+      if (tnn < c1) {
+        lookup(tnn);
+        issue(kA, vA);
+      }
+      reduce(kB, vB, tn);
+      if (tnn >= c1) break;
+      t = tnn;
+    }
+  }
+
+  // ---- merge the NW wave states of the workgroup through LDS ----
+  __shared__ float sm_o[NW][8][64];
+  __shared__ float sm_ml[NW][2][64];
+  __shared__ int sm_ticket;
+#pragma unroll
+  for (int j = 0; j < QPG; ++j) {
+    if (j > 0) __syncthreads();
+#pragma unroll
+    for (int d = 0; d < 8; ++d) sm_o[wave][d][lane] = acc[j][d];
+    sm_ml[wave][0][lane] = m[j];
+    sm_ml[wave][1][lane] = l[j];
+    __syncthreads();
+    if (wave == (j % NW)) {
+      float M = kNegBig;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) M = fmaxf(M, sm_ml[w][0][lane]);
+      float L = 0.f, r[8];
+#pragma unroll
+      for (int d = 0; d < 8; ++d) r[d] = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) {
+        const float f = fast_exp2(sm_ml[w][0][lane] - M);
+        L = fmaf(sm_ml[w][1][lane], f, L);
+#pragma unroll
+        for (int d = 0; d < 8; ++d) r[d] = fmaf(sm_o[w][d][lane], f, r[d]);
+      }
+      // result of query head qh0 + j now lives in wave (j % NW)
+      const int qh = qh0 + j;
+      if (head_ok) {
+        if (n_splits == 1) {
+          const float inv = L > 0.f ? 1.f / L : 0.f;
+          u32x4 out;
+          out.x = pack2<T>(r[0] * inv, r[1] * inv);
+          out.y = pack2<T>(r[2] * inv, r[3] * inv);
+          out.z = pack2<T>(r[4] * inv, r[5] * inv);
+          out.w = pack2<T>(r[6] * inv, r[7] * inv);
+          reinterpret_cast<u32x4*>(p.o)[((int64_t)b * p.num_qo_heads + qh) * LPR + li] = out;
+          if (p.lse && li == 0)
+            p.lse[(int64_t)b * p.num_qo_heads + qh] =
+                L > 0.f ? (M + fast_log2(L)) * kLn2 : -INFINITY;
+        } else {
+          const int64_t slot = ((int64_t)b * p.num_qo_heads + qh) * p.max_splits + split;
+          f32x4* dst = reinterpret_cast<f32x4*>(p.ws_o + slot * D + li * 8);
+          f32x4 a0 = {r[0], r[1], r[2], r[3]};
+          f32x4 a1 = {r[4], r[5], r[6], r[7]};
+          dst[0] = a0;
+          dst[1] = a1;
+          if (li == 0) {
+            p.ws_ml[slot * 2 + 0] = M;
+            p.ws_ml[slot * 2 + 1] = L;
+          }
+        }
+      }
+    }
+  }
+
+  if (n_splits == 1 || !p.fused_merge) return;
+
+  // ---- last-arriving workgroup of this (sequence, head group) reduces the partials ----
+  __threadfence();
+  __syncthreads();
+  if (tid == 0) sm_ticket = atomicAdd(p.ws_cnt + (int64_t)b * gridDim.x + hg, 1);
+  __syncthreads();
+  if (sm_ticket != n_splits - 1) return;
+  __threadfence();
+
+  constexpr int NQ = HPW * QPG;  // query heads of this head group
+  const int qh_base = hg * NQ;
+  for (int e = tid * 4; e < NQ * D; e += NW * 64 * 4) {
+    const int qh = qh_base + e / D;
+    const int d = e % D;
+    if (qh >= p.num_qo_heads) break;
+    const int64_t slot0 = ((int64_t)b * p.num_qo_heads + qh) * p.max_splits;
+    float M = kNegBig;
+    for (int sidx = 0; sidx < n_splits; ++sidx)
+      M = fmaxf(M, p.ws_ml[(slot0 + sidx) * 2]);
+    float L = 0.f;
+    f32x4 r = {0.f, 0.f, 0.f, 0.f};
+    for (int sidx = 0; sidx < n_splits; ++sidx) {
+      const float ms = p.ws_ml[(slot0 + sidx) * 2];
+      const float ls = p.ws_ml[(slot0 + sidx) * 2 + 1];
+      const float f = fast_exp2(ms - M);
+      L = fmaf(ls, f, L);
+      const f32x4 po = *reinterpret_cast<const f32x4*>(p.ws_o + (slot0 + sidx) * D + d);
+      r += po * f;
+    }
+    const float inv = L > 0.f ? 1.f / L : 0.f;
+    u32x2 out;
+    out.x = pack2<T>(r.x * inv, r.y * inv);
+    out.y = pack2<T>(r.z * inv, r.w * inv);
+    *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(p.o) +
+                              ((int64_t)b * p.num_qo_heads + qh) * D + d) = out;
+    if (p.lse && d == 0)
+      p.lse[(int64_t)b * p.num_qo_heads + qh] = L > 0.f ? (M + fast_log2(L)) * kLn2 : -INFINITY;
+  }
+  if (tid == 0) p.ws_cnt[(int64_t)b * gridDim.x + hg] = 0;
+}
+
+// Second-kernel merge: one workgroup of 64*... threads per (sequence, query head).
+template <typename T, int D>
+__global__ __launch_bounds__(D / 4) void merge_partials_kernel(const DecodeParams p) {
+  const int qh = blockIdx.x;
+  const int b = blockIdx.y;
+  const int d = threadIdx.x * 4;
+  int n_list;
+  if (p.indptr)
+    n_list = p.indptr[b + 1] - p.indptr[b];
+  else
+    n_list = p.n_list_host;
+  n_list = n_list < 0 ? 0 : (n_list > p.n_list_host ? p.n_list_host : n_list);
+  const int last_len = p.last_len_arr ? p.last_len_arr[b] : p.last_len;
+  const int n_items = (p.page_mode ? n_list * p.page_size : n_list) + last_len;
+  int n_splits = (n_items + p.chunk_tokens - 1) / p.chunk_tokens;
+  if (n_splits <= 1) return;  // the attention kernel already wrote the final result
+  const int64_t slot0 = ((int64_t)b * p.num_qo_heads + qh) * p.max_splits;
+  float M = kNegBig;
+  for (int sidx = 0; sidx < n_splits; ++sidx) M = fmaxf(M, p.ws_ml[(slot0 + sidx) * 2]);
+  float L = 0.f;
+  f32x4 r = {0.f, 0.f, 0.f, 0.f};
+  for (int sidx = 0; sidx < n_splits; ++sidx) {
+    const float f = fast_exp2(p.ws_ml[(slot0 + sidx) * 2] - M);
+    L = fmaf(p.ws_ml[(slot0 + sidx) * 2 + 1], f, L);
+    r += *reinterpret_cast<const f32x4*>(p.ws_o + (slot0 + sidx) * D + d) * f;
+  }
+  const float inv = L > 0.f ? 1.f / L : 0.f;
+  u32x2 out;
+  out.x = pack2<T>(r.x * inv, r.y * inv);
+  out.y = pack2<T>(r.z * inv, r.w * inv);
+  *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(p.o) +
+                            ((int64_t)b * p.num_qo_heads + qh) * D + d) = out;
+  if (p.lse && d == 0)
+    p.lse[(int64_t)b * p.num_qo_heads + qh] = L > 0.f ? (M + fast_log2(L)) * kLn2 : -INFINITY;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------------------------
+static int g_num_cus = 0;
+
+static int num_cus() {
+  if (g_num_cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess &&
+        n > 0)
+      g_num_cus = n;
+    else
+      g_num_cus = 256;  // MI355X
+  }
+  return g_num_cus;
+}
+
+constexpr int kTileTokens = 4;  // U
+
+static int qpg_for(int num_qo_heads, int num_kv_heads, int idx_rows) {
+  // KV rows are shared between the query heads of a group only when the group shares its list
+  const int group = num_qo_heads / num_kv_heads;
+  if (group > 1 && idx_rows != num_qo_heads) return group;
+  return 1;
+}
+
+template <typename T, int D, int QPG, int NW>
+static void launch_variant(const DecodeParams& p, bool page_mode, bool emit, dim3 grid,
+                           hipStream_t st) {
+  constexpr int U = kTileTokens;
+  if (page_mode) {
+    if (emit)
+      hipLaunchKernelGGL((decode_attn_kernel<T, D, QPG, U, NW, true, true>), grid, dim3(NW * 64), 0,
+                         st, p);
+    else
+      hipLaunchKernelGGL((decode_attn_kernel<T, D, QPG, U, NW, true, false>), grid, dim3(NW * 64),
+                         0, st, p);
+  } else {
+    if (emit)
+      hipLaunchKernelGGL((decode_attn_kernel<T, D, QPG, U, NW, false, true>), grid, dim3(NW * 64),
+                         0, st, p);
+    else
+      hipLaunchKernelGGL((decode_attn_kernel<T, D, QPG, U, NW, false, false>), grid, dim3(NW * 64),
+                         0, st, p);
+  }
+}
+
+// Instantiated shapes: one query head per lane group for head_dim 64/128/256 with 8 or 16
+// waves; 2, 4 or 8 query heads per lane group (shared KV rows under GQA) for head_dim 128 with
+// 8 waves.
+static bool shape_supported(int head_dim, int qpg, int nw) {
+  if (qpg == 1) return (head_dim == 64 || head_dim == 128 || head_dim == 256) && (nw == 8 || nw == 16);
+  return head_dim == 128 && (qpg == 2 || qpg == 4 || qpg == 8) && nw == 8;
+}
+
+template <typename T>
+static int launch_shape(const DecodeParams& p, int head_dim, int qpg, int nw, bool page_mode,
+                        bool emit, dim3 grid, hipStream_t st) {
+#define TD_CASE(D_, Q_, N_)                                                    \
+  if (head_dim == D_ && qpg == Q_ && nw == N_) {                               \
+    launch_variant<T, D_, Q_, N_>(p, page_mode, emit, grid, st);               \
+    return TD_OK;                                                              \
+  }
+  TD_CASE(64, 1, 8)
+  TD_CASE(64, 1, 16)
+  TD_CASE(128, 1, 8)
+  TD_CASE(128, 1, 16)
+  TD_CASE(256, 1, 8)
+  TD_CASE(256, 1, 16)
+  TD_CASE(128, 2, 8)
+  TD_CASE(128, 4, 8)
+  TD_CASE(128, 8, 8)
+#undef TD_CASE
+  return fail(TD_ERR_UNSUPPORTED,
+              "BatchDecodeWithPagedKVCache failed to dispatch: head_dim %d with %d query heads per "
+              "shared KV row and %d waves (supported: head_dim 64/128/256 with per-head lists; "
+              "head_dim 128 with shared lists and group size 2, 4 or 8)",
+              head_dim, qpg, nw);
+}
+
+template <typename T>
+static int launch_merge(const DecodeParams& p, int head_dim, dim3 grid, hipStream_t st) {
+  switch (head_dim) {
+    case 64: hipLaunchKernelGGL((merge_partials_kernel<T, 64>), grid, dim3(16), 0, st, p); break;
+    case 128: hipLaunchKernelGGL((merge_partials_kernel<T, 128>), grid, dim3(32), 0, st, p); break;
+    case 256: hipLaunchKernelGGL((merge_partials_kernel<T, 256>), grid, dim3(64), 0, st, p); break;
+  }
+  return TD_OK;
+}
+
+static int64_t align256(int64_t x) { return (x + 255) & ~(int64_t)255; }
+
+}  // namespace tidal
+
+using namespace tidal;
+
+extern "C" int td_num_cus(void) { return num_cus(); }
+
+extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t num_kv_heads,
+                              int32_t head_dim, int32_t idx_rows, int64_t max_items,
+                              td_decode_plan* plan) {
+  TD_REQUIRE(plan != nullptr, "td_decode_make_plan: plan is NULL");
+  TD_REQUIRE(batch >= 1, "td_decode_make_plan: batch %d < 1", batch);
+  TD_REQUIRE(num_kv_heads >= 1 && num_qo_heads >= num_kv_heads && num_qo_heads % num_kv_heads == 0,
+             "td_decode_make_plan: num_qo_heads %d must be a positive multiple of num_kv_heads %d",
+             num_qo_heads, num_kv_heads);
+  if (head_dim != 64 && head_dim != 128 && head_dim != 256)
+    return fail(TD_ERR_UNSUPPORTED, "td_decode_make_plan: head_dim %d (supported: 64, 128, 256)",
+                head_dim);
+  TD_REQUIRE(idx_rows == 1 || idx_rows == num_kv_heads || idx_rows == num_qo_heads,
+             "td_decode_make_plan: idx_rows %d must be 1, num_kv_heads (%d) or num_qo_heads (%d)",
+             idx_rows, num_kv_heads, num_qo_heads);
+  TD_REQUIRE(max_items >= 0 && max_items < ((int64_t)1 << 30), "td_decode_make_plan: max_items %lld",
+             (long long)max_items);
+
+  const int qpg = qpg_for(num_qo_heads, num_kv_heads, idx_rows);
+  const int hpw = 64 / (head_dim / 8);
+  const int n_hrows = num_qo_heads / qpg;
+  const int head_groups = (n_hrows + hpw - 1) / hpw;
+
+  int nw = plan->waves_per_block;
+  if (nw == 0) nw = 8;
+  if (!shape_supported(head_dim, qpg, nw))
+    return fail(TD_ERR_UNSUPPORTED,
+                "td_decode_make_plan: no kernel for head_dim %d, %d query heads per shared KV row, %d "
+                "waves per block",
+                head_dim, qpg, nw);
+  const int tile = nw * kTileTokens;  // tokens one pass of the workgroup covers
+
+  // Aim at ~2 workgroups of 8 waves per compute unit, never less than one tile per workgroup,
+  // never more than 64 partials per head.
+  const int64_t target_blocks = (int64_t)num_cus() * 2 * 8 / nw;
+  int64_t splits = target_blocks / ((int64_t)head_groups * batch);
+  if (splits < 1) splits = 1;
+  if (splits > 64) splits = 64;
+  int64_t chunk = max_items > 0 ? ceil_div64(max_items, splits) : tile;
+  if (plan->chunk_tokens > 0) chunk = plan->chunk_tokens;
+  chunk = ceil_div64(chunk, tile) * tile;
+  int64_t max_splits = max_items > 0 ? ceil_div64(max_items, chunk) : 1;
+  if (max_splits < 1) max_splits = 1;
+
+  plan->chunk_tokens = (int32_t)chunk;
+  plan->max_splits = (int32_t)max_splits;
+  plan->waves_per_block = nw;
+  if (plan->fused_merge < 0) plan->fused_merge = 1;
+  plan->fused_merge = plan->fused_merge ? 1 : 0;
+  const int64_t n_part = (int64_t)batch * num_qo_heads * max_splits;
+  plan->workspace_bytes = align256(n_part * head_dim * 4) + align256(n_part * 2 * 4) +
+                          align256((int64_t)batch * head_groups * 4);
+  return TD_OK;
+}
+
+extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
+                              const td_decode_plan* plan, const void* q, void* o, int32_t batch,
+                              int32_t num_qo_heads, float sm_scale, void* scores,
+                              int32_t scores_dtype, int64_t score_stride, float* lse,
+                              void* workspace, int64_t workspace_bytes, void* stream) {
+  TD_REQUIRE(kv && list && plan && q && o, "td_decode_attn: NULL argument");
+  TD_REQUIRE(kv->data != nullptr, "td_decode_attn: kv->data is NULL");
+  TD_REQUIRE(batch >= 1, "td_decode_attn: batch %d < 1", batch);
+  const int Hkv = kv->num_kv_heads, D = kv->head_dim, P = kv->page_size;
+  TD_REQUIRE(Hkv >= 1 && num_qo_heads >= Hkv && num_qo_heads % Hkv == 0,
+             "td_decode_attn: num_qo_heads %d must be a positive multiple of num_kv_heads %d",
+             num_qo_heads, Hkv);
+  TD_REQUIRE(P >= 1 && kv->max_pages >= 1, "td_decode_attn: page_size %d / max_pages %lld", P,
+             (long long)kv->max_pages);
+  TD_REQUIRE(kv->max_pages * P < ((int64_t)1 << 31), "td_decode_attn: pool too large for int32 slots");
+  TD_REQUIRE(kv->layout == TD_NHD || kv->layout == TD_HND, "td_decode_attn: layout %d", kv->layout);
+  if (kv->dtype != TD_F16 && kv->dtype != TD_BF16)
+    return fail(TD_ERR_UNSUPPORTED,
+                "BatchDecodeWithPagedKVCache failed to dispatch with dtype %d (supported: fp16, bf16)",
+                kv->dtype);
+  TD_REQUIRE(list->idx_rows == 1 || list->idx_rows == Hkv || list->idx_rows == num_qo_heads,
+             "td_decode_attn: idx_rows %d must be 1, %d or %d", list->idx_rows, Hkv, num_qo_heads);
+  TD_REQUIRE(list->kind == TD_IDX_PAGES || list->kind == TD_IDX_SLOTS, "td_decode_attn: kind %d",
+             list->kind);
+  TD_REQUIRE(list->n_list_host >= 0, "td_decode_attn: n_list_host %d", list->n_list_host);
+  TD_REQUIRE(list->idx != nullptr || list->n_list_host == 0,
+             "td_decode_attn: idx is NULL but n_list_host is %d", list->n_list_host);
+  TD_REQUIRE(list->idx_rows == 1 || list->idx_row_stride >= list->n_list_host,
+             "td_decode_attn: idx_row_stride %d < n_list_host %d", list->idx_row_stride,
+             list->n_list_host);
+  TD_REQUIRE(list->last_page_len >= 0 && list->last_page_len <= P,
+             "td_decode_attn: last_page_len %d not in [0, %d]", list->last_page_len, P);
+  TD_REQUIRE(list->last_page_idx >= 0 && list->last_page_idx < kv->max_pages,
+             "td_decode_attn: last_page_idx %d outside the pool of %lld pages", list->last_page_idx,
+             (long long)kv->max_pages);
+  TD_REQUIRE(plan->chunk_tokens > 0 && plan->max_splits >= 1 && plan->waves_per_block > 0 &&
+                 plan->chunk_tokens % (plan->waves_per_block * kTileTokens) == 0,
+             "td_decode_attn: plan not produced by td_decode_make_plan");
+  // the planned split must cover every token the list can describe
+  const int64_t max_items = (int64_t)list->n_list_host * (list->kind == TD_IDX_PAGES ? P : 1) +
+                            (list->last_page_len_arr ? P : list->last_page_len);
+  if (max_items > (int64_t)plan->chunk_tokens * plan->max_splits)
+    return fail(TD_ERR_STATE,
+                "td_decode_attn: the list describes up to %lld tokens but the plan covers %lld "
+                "(call td_decode_make_plan / begin_forward for this budget first)",
+                (long long)max_items, (long long)plan->chunk_tokens * plan->max_splits);
+  if (scores) {
+    TD_REQUIRE(scores_dtype == TD_F32 || scores_dtype == kv->dtype,
+               "td_decode_attn: scores dtype %d must be fp32 or the KV dtype", scores_dtype);
+    TD_REQUIRE(score_stride > 0, "td_decode_attn: score_stride %lld", (long long)score_stride);
+  }
+
+  const int qpg = qpg_for(num_qo_heads, Hkv, list->idx_rows);
+  const int hpw = 64 / (D / 8);
+  const int n_hrows = num_qo_heads / qpg;
+  const int head_groups = (n_hrows + hpw - 1) / hpw;
+
+  const int64_t n_part = (int64_t)batch * num_qo_heads * plan->max_splits;
+  const int64_t off_ml = align256(n_part * D * 4);
+  const int64_t off_cnt = off_ml + align256(n_part * 2 * 4);
+  const int64_t need = off_cnt + align256((int64_t)batch * head_groups * 4);
+  if (plan->max_splits > 1) {
+    if (workspace == nullptr || workspace_bytes < need)
+      return fail(TD_ERR_STATE,
+                  "td_decode_attn: workspace of %lld bytes is smaller than the %lld the plan needs "
+                  "(call td_decode_make_plan / begin_forward first)",
+                  (long long)workspace_bytes, (long long)need);
+  }
+
+  DecodeParams p;
+  p.q = q;
+  p.o = o;
+  p.kv = kv->data;
+  p.page_stride = (int64_t)2 * P * Hkv * D;
+  p.v_offset = (int64_t)P * Hkv * D;
+  if (kv->layout == TD_NHD) {
+    p.entry_stride = Hkv * D;
+    p.head_stride = D;
+  } else {
+    p.entry_stride = D;
+    p.head_stride = P * D;
+  }
+  p.page_size = P;
+  p.page_shift = -1;
+  for (int sft = 0; sft < 31; ++sft)
+    if ((1 << sft) == P) p.page_shift = sft;
+  p.max_slot = (uint32_t)(kv->max_pages * P - 1);
+  p.num_qo_heads = num_qo_heads;
+  p.n_hrows = n_hrows;
+  p.q_per_kv = num_qo_heads / Hkv;
+  p.idx = list->idx;
+  p.idx_row_stride = list->idx_rows == 1 ? 0 : list->idx_row_stride;
+  p.idx_per_kv = (qpg == 1 && list->idx_rows == Hkv && Hkv != num_qo_heads) ? 1 : 0;
+  p.page_mode = list->kind == TD_IDX_PAGES ? 1 : 0;
+  p.max_page = (uint32_t)(kv->max_pages - 1);
+  p.indptr = list->indptr;
+  p.n_list_host = list->n_list_host;
+  p.last_len_arr = list->last_page_len_arr;
+  p.last_idx_arr = list->last_page_idx_arr;
+  p.last_len = list->last_page_len;
+  p.last_idx = list->last_page_idx;
+  p.chunk_tokens = plan->chunk_tokens;
+  p.max_splits = plan->max_splits;
+  p.fused_merge = plan->fused_merge;
+  p.scale_log2 = sm_scale * kLog2e;
+  p.scores = scores;
+  p.scores_f32 = scores_dtype == TD_F32 ? 1 : 0;
+  p.score_stride = score_stride;
+  p.lse = lse;
+  char* ws = reinterpret_cast<char*>(workspace);
+  p.ws_o = reinterpret_cast<float*>(ws);
+  p.ws_ml = reinterpret_cast<float*>(ws ? ws + off_ml : nullptr);
+  p.ws_cnt = reinterpret_cast<int32_t*>(ws ? ws + off_cnt : nullptr);
+
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const bool page_mode = list->kind == TD_IDX_PAGES;
+  dim3 grid(head_groups, plan->max_splits, batch);
+  int rc;
+  if (kv->dtype == TD_F16)
+    rc = launch_shape<F16>(p, D, qpg, plan->waves_per_block, page_mode, scores != nullptr, grid, st);
+  else
+    rc = launch_shape<BF16>(p, D, qpg, plan->waves_per_block, page_mode, scores != nullptr, grid, st);
+  if (rc != TD_OK) return rc;
+  TD_HIP_CHECK(hipGetLastError());
+  if (plan->max_splits > 1 && !plan->fused_merge) {
+    dim3 mgrid(num_qo_heads, batch);
+    if (kv->dtype == TD_F16)
+      launch_merge<F16>(p, D, mgrid, st);
+    else
+      launch_merge<BF16>(p, D, mgrid, st);
+    TD_HIP_CHECK(hipGetLastError());
+  }
+  return TD_OK;
+}

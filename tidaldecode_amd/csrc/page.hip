@@ -1,0 +1,351 @@
+// Rotary embedding, paged KV append, their decode-step fusion, and RMSNorm for gfx950.
+//
+// RoPE is the rotate-half (Llama) form of kernels/include/decode/decode_page.cuh:639-687 of the
+// reference; angles are formed in double precision (position * theta^(-2j/D) / scale) and only
+// the sine / cosine are rounded to fp32, so positions of 1e5 and beyond lose nothing to the
+// fp32 product the reference forms.  Append follows AppendPagedKVCacheDecode/Prefill
+// (decode_page.cuh:387-557) including the per-page key max/min metadata.
+
+#include "common.cuh"
+
+namespace tidal {
+
+struct PoolGeom {
+  void* data;
+  int64_t page_stride;
+  int64_t v_offset;
+  int32_t entry_stride;
+  int32_t head_stride;
+  int32_t page_size;
+  int32_t num_heads;
+  uint32_t max_page;
+};
+
+static PoolGeom geom_of(const td_paged_kv* kv) {
+  PoolGeom g;
+  const int P = kv->page_size, H = kv->num_kv_heads, D = kv->head_dim;
+  g.data = kv->data;
+  g.page_stride = (int64_t)2 * P * H * D;
+  g.v_offset = (int64_t)P * H * D;
+  if (kv->layout == TD_NHD) {
+    g.entry_stride = H * D;
+    g.head_stride = D;
+  } else {
+    g.entry_stride = D;
+    g.head_stride = P * D;
+  }
+  g.page_size = P;
+  g.num_heads = H;
+  g.max_page = (uint32_t)(kv->max_pages - 1);
+  return g;
+}
+
+__device__ __forceinline__ int64_t k_offset(const PoolGeom& g, uint32_t page, int entry, int head) {
+  page = page > g.max_page ? g.max_page : page;
+  return (int64_t)page * g.page_stride + (int64_t)entry * g.entry_stride +
+         (int64_t)head * g.head_stride;
+}
+
+// sin / cos of position * theta^(-2j/D) / scale
+__device__ __forceinline__ void rope_sincos(double pos_over_scale, double log2_theta, int j, int D,
+                                            float& sn, float& cs) {
+  const double inv_freq = exp2(-log2_theta * (double)(2 * j) / (double)D);
+  double s, c;
+  sincos(pos_over_scale * inv_freq, &s, &c);
+  sn = (float)s;
+  cs = (float)c;
+}
+
+template <typename T>
+__device__ __forceinline__ void rotate_pair(uint16_t* row, int j, int half, float sn, float cs) {
+  const float lo = to_float<T>(row[j]);
+  const float hi = to_float<T>(row[j + half]);
+  row[j] = from_float<T>(lo * cs - hi * sn);
+  row[j + half] = from_float<T>(hi * cs + lo * sn);
+}
+
+// grid: n_tokens; block: 256 threads = (D/2 pair columns) x (512/D head slots)
+template <typename T>
+__global__ __launch_bounds__(256) void rope_kernel(uint16_t* q, uint16_t* k, int n_tokens, int Hq,
+                                                   int Hkv, int D, double past_len,
+                                                   double inv_scale, double log2_theta) {
+  const int tok = blockIdx.x;
+  const int half = D / 2;
+  const int j = threadIdx.x % half;
+  const int slot = threadIdx.x / half;
+  const int slots = 256 / half;
+  if (slot >= slots) return;
+  float sn, cs;
+  rope_sincos((past_len + (double)tok) * inv_scale, log2_theta, j, D, sn, cs);
+  for (int h = slot; h < Hq + Hkv; h += slots) {
+    uint16_t* row = h < Hq ? q + ((int64_t)tok * Hq + h) * D : k + ((int64_t)tok * Hkv + (h - Hq)) * D;
+    rotate_pair<T>(row, j, half, sn, cs);
+  }
+}
+
+// grid: batch; rotates q in place, rotates k into the cache slot, copies v into the cache slot
+template <typename T>
+__global__ __launch_bounds__(256) void rope_append_decode_kernel(
+    PoolGeom g, uint16_t* q, const uint16_t* k, const uint16_t* v, int Hq, int D,
+    const int32_t* positions, const int32_t* dst_slot, double inv_scale, double log2_theta) {
+  const int b = blockIdx.x;
+  const int Hkv = g.num_heads;
+  const int half = D / 2;
+  const int j = threadIdx.x % half;
+  const int slot = threadIdx.x / half;
+  const int slots = 256 / half;
+  if (slot >= slots) return;
+  const uint32_t dst = (uint32_t)dst_slot[b];
+  const uint32_t page = dst / (uint32_t)g.page_size;
+  const int entry = (int)(dst - page * (uint32_t)g.page_size);
+  float sn, cs;
+  rope_sincos((double)positions[b] * inv_scale, log2_theta, j, D, sn, cs);
+  uint16_t* pool = reinterpret_cast<uint16_t*>(g.data);
+  for (int h = slot; h < Hq + Hkv; h += slots) {
+    if (h < Hq) {
+      rotate_pair<T>(q + ((int64_t)b * Hq + h) * D, j, half, sn, cs);
+    } else {
+      const int hk = h - Hq;
+      const uint16_t* krow = k + ((int64_t)b * Hkv + hk) * D;
+      const uint16_t* vrow = v + ((int64_t)b * Hkv + hk) * D;
+      uint16_t* kdst = pool + k_offset(g, page, entry, hk);
+      const float lo = to_float<T>(krow[j]);
+      const float hi = to_float<T>(krow[j + half]);
+      kdst[j] = from_float<T>(lo * cs - hi * sn);
+      kdst[j + half] = from_float<T>(hi * cs + lo * sn);
+      kdst[g.v_offset + j] = vrow[j];
+      kdst[g.v_offset + j + half] = vrow[j + half];
+    }
+  }
+}
+
+// grid: n_tokens; copies one token's K and V rows (all heads) into its page slot, 16 B per lane
+__global__ __launch_bounds__(256) void append_copy_kernel(PoolGeom g, const uint16_t* k,
+                                                          const uint16_t* v, int n_tokens, int D,
+                                                          const int32_t* indices,
+                                                          const int32_t* indptr, int last_page_len) {
+  const int tok = blockIdx.x;
+  const int H = g.num_heads;
+  const int n_pages = indptr[1] - indptr[0];
+  const int seq_len = (n_pages - 1) * g.page_size + last_page_len;
+  const int pos = seq_len - n_tokens + tok;
+  if (pos < 0 || n_pages <= 0) return;
+  const int pg = pos / g.page_size;
+  const int entry = pos - pg * g.page_size;
+  const uint32_t page = (uint32_t)indices[indptr[0] + pg];
+  uint16_t* pool = reinterpret_cast<uint16_t*>(g.data);
+  const int vec_per_row = D / 8;
+  for (int x = threadIdx.x; x < H * vec_per_row; x += 256) {
+    const int h = x / vec_per_row;
+    const int c = (x - h * vec_per_row) * 8;
+    const int64_t src = ((int64_t)tok * H + h) * D + c;
+    uint16_t* dst = pool + k_offset(g, page, entry, h) + c;
+    *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(k + src);
+    *reinterpret_cast<u32x4*>(dst + g.v_offset) = *reinterpret_cast<const u32x4*>(v + src);
+  }
+}
+
+// Per KV page touched by the append: element-wise running max (K plane) / min (V plane) of the
+// page's keys, kept at entry (page ordinal) of the metadata pool.  grid: (touched pages, heads)
+template <typename T>
+__global__ void append_meta_kernel(PoolGeom kvg, PoolGeom mg, const uint16_t* k, int n_tokens,
+                                   int D, const int32_t* kv_indptr, int last_page_len,
+                                   const int32_t* meta_indices, const int32_t* meta_indptr,
+                                   float type_max) {
+  const int h = blockIdx.y;
+  const int d = threadIdx.x;  // one element per thread, D threads
+  const int H = kvg.num_heads;
+  const int P = kvg.page_size;
+  const int n_pages = kv_indptr[1] - kv_indptr[0];
+  const int seq_len = (n_pages - 1) * P + last_page_len;
+  const int start = seq_len - n_tokens;
+  if (start < 0 || n_pages <= 0) return;
+  const int pg = start / P + blockIdx.x;  // ordinal of the KV page inside the sequence
+  if (pg >= n_pages) return;
+  int e0 = start - pg * P;
+  e0 = e0 < 0 ? 0 : e0;
+  int e1 = seq_len - pg * P;
+  e1 = e1 > P ? P : e1;
+  const int mP = mg.page_size;
+  const uint32_t mpage = (uint32_t)meta_indices[meta_indptr[0] + pg / mP];
+  uint16_t* mrow = reinterpret_cast<uint16_t*>(mg.data) + k_offset(mg, mpage, pg % mP, h);
+  float mx = -type_max, mn = type_max;
+  if (e0 > 0) {
+    mx = to_float<T>(mrow[d]);
+    mn = to_float<T>(mrow[mg.v_offset + d]);
+  }
+  for (int e = e0; e < e1; ++e) {
+    const int tok = pg * P + e - start;
+    const float x = to_float<T>(k[((int64_t)tok * H + h) * D + d]);
+    mx = fmaxf(mx, x);
+    mn = fminf(mn, x);
+  }
+  mrow[d] = from_float<T>(mx);
+  mrow[mg.v_offset + d] = from_float<T>(mn);
+}
+
+// RMSNorm, one 256-thread workgroup per row, fp32 accumulation
+template <typename T>
+__global__ __launch_bounds__(256) void rms_norm_kernel(const uint16_t* x, const uint16_t* w,
+                                                       uint16_t* out, int cols, float eps) {
+  const int row = blockIdx.x;
+  const uint16_t* xr = x + (int64_t)row * cols;
+  uint16_t* orow = out + (int64_t)row * cols;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < cols; c += 256) {
+    const float f = to_float<T>(xr[c]);
+    ss = fmaf(f, f, ss);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+  __shared__ float part[4];
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  const float total = part[0] + part[1] + part[2] + part[3];
+  const float inv = rsqrtf(total / (float)cols + eps);
+  for (int c = threadIdx.x; c < cols; c += 256)
+    orow[c] = from_float<T>(to_float<T>(xr[c]) * inv * to_float<T>(w[c]));
+}
+
+static int check_pool(const td_paged_kv* kv, const char* who) {
+  TD_REQUIRE(kv && kv->data, "%s: pool is NULL", who);
+  TD_REQUIRE(kv->num_kv_heads >= 1 && kv->page_size >= 1 && kv->max_pages >= 1,
+             "%s: pool heads %d page_size %d max_pages %lld", who, kv->num_kv_heads, kv->page_size,
+             (long long)kv->max_pages);
+  TD_REQUIRE(kv->layout == TD_NHD || kv->layout == TD_HND, "%s: layout %d", who, kv->layout);
+  TD_REQUIRE(kv->max_pages * kv->page_size < ((int64_t)1 << 31), "%s: pool too large for int32 slots",
+             who);
+  return TD_OK;
+}
+
+}  // namespace tidal
+
+using namespace tidal;
+
+extern "C" int td_rope_in_place(void* q, void* k, int32_t n_tokens, int32_t num_qo_heads,
+                                int32_t num_kv_heads, int32_t head_dim, int64_t past_kv_len,
+                                float rope_scale, float rope_theta, int32_t dtype, void* stream) {
+  TD_REQUIRE(q && k, "apply_rope_in_place: NULL q or k");
+  TD_REQUIRE(n_tokens >= 0 && num_qo_heads >= 1 && num_kv_heads >= 1,
+             "apply_rope_in_place: n_tokens %d heads %d/%d", n_tokens, num_qo_heads, num_kv_heads);
+  if (head_dim != 64 && head_dim != 128 && head_dim != 256)
+    return fail(TD_ERR_UNSUPPORTED, "apply_rope_in_place: head_dim %d (supported: 64, 128, 256)",
+                head_dim);
+  TD_REQUIRE(rope_scale > 0.f && rope_theta > 0.f, "apply_rope_in_place: scale %g theta %g",
+             rope_scale, rope_theta);
+  TD_REQUIRE(past_kv_len >= 0, "apply_rope_in_place: past_kv_len %lld", (long long)past_kv_len);
+  if (n_tokens == 0) return TD_OK;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const double inv_scale = 1.0 / (double)rope_scale;
+  const double log2_theta = log2((double)rope_theta);
+  if (dtype == TD_F16)
+    hipLaunchKernelGGL(rope_kernel<F16>, dim3(n_tokens), dim3(256), 0, st, (uint16_t*)q,
+                       (uint16_t*)k, n_tokens, num_qo_heads, num_kv_heads, head_dim,
+                       (double)past_kv_len, inv_scale, log2_theta);
+  else if (dtype == TD_BF16)
+    hipLaunchKernelGGL(rope_kernel<BF16>, dim3(n_tokens), dim3(256), 0, st, (uint16_t*)q,
+                       (uint16_t*)k, n_tokens, num_qo_heads, num_kv_heads, head_dim,
+                       (double)past_kv_len, inv_scale, log2_theta);
+  else
+    return fail(TD_ERR_UNSUPPORTED, "apply_rope_in_place failed to dispatch with dtype %d", dtype);
+  TD_HIP_CHECK(hipGetLastError());
+  return TD_OK;
+}
+
+extern "C" int td_append_kv(const td_paged_kv* kv, const void* k, const void* v, int32_t n_tokens,
+                            const int32_t* kv_indices, const int32_t* kv_indptr,
+                            int32_t last_page_len, const td_paged_kv* meta,
+                            const int32_t* meta_indices, const int32_t* meta_indptr,
+                            int32_t meta_last_page_len, void* stream) {
+  (void)meta_last_page_len;
+  int rc = check_pool(kv, "append_kv_cache");
+  if (rc) return rc;
+  TD_REQUIRE(k && v && kv_indices && kv_indptr, "append_kv_cache: NULL argument");
+  TD_REQUIRE(n_tokens >= 0, "append_kv_cache: n_tokens %d", n_tokens);
+  TD_REQUIRE(last_page_len >= 1 && last_page_len <= kv->page_size,
+             "append_kv_cache: last_page_len %d not in [1, %d]", last_page_len, kv->page_size);
+  const int D = kv->head_dim;
+  if (D != 64 && D != 128 && D != 256)
+    return fail(TD_ERR_UNSUPPORTED, "append_kv_cache: head_dim %d (supported: 64, 128, 256)", D);
+  if (kv->dtype != TD_F16 && kv->dtype != TD_BF16)
+    return fail(TD_ERR_UNSUPPORTED, "Append_kv_cache failed to dispatch with dtype %d", kv->dtype);
+  if (n_tokens == 0) return TD_OK;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const PoolGeom g = geom_of(kv);
+  hipLaunchKernelGGL(append_copy_kernel, dim3(n_tokens), dim3(256), 0, st, g, (const uint16_t*)k,
+                     (const uint16_t*)v, n_tokens, D, kv_indices, kv_indptr, last_page_len);
+  TD_HIP_CHECK(hipGetLastError());
+  if (meta && meta->data) {
+    rc = check_pool(meta, "append_kv_cache(metadata)");
+    if (rc) return rc;
+    TD_REQUIRE(meta_indices && meta_indptr, "append_kv_cache: NULL metadata indices");
+    TD_REQUIRE(meta->num_kv_heads == kv->num_kv_heads && meta->head_dim == D &&
+                   meta->dtype == kv->dtype,
+               "append_kv_cache: metadata pool shape differs from the KV pool");
+    const PoolGeom mg = geom_of(meta);
+    // pages touched by n_tokens appended tokens: at most ceil(n/P) + 1
+    const int touched = (n_tokens + kv->page_size - 1) / kv->page_size + 1;
+    dim3 grid(touched, kv->num_kv_heads);
+    if (kv->dtype == TD_F16)
+      hipLaunchKernelGGL(append_meta_kernel<F16>, grid, dim3(D), 0, st, g, mg, (const uint16_t*)k,
+                         n_tokens, D, kv_indptr, last_page_len, meta_indices, meta_indptr, 65504.f);
+    else
+      hipLaunchKernelGGL(append_meta_kernel<BF16>, grid, dim3(D), 0, st, g, mg, (const uint16_t*)k,
+                         n_tokens, D, kv_indptr, last_page_len, meta_indices, meta_indptr,
+                         3.3895313892515355e38f);
+    TD_HIP_CHECK(hipGetLastError());
+  }
+  return TD_OK;
+}
+
+extern "C" int td_rope_append_decode(const td_paged_kv* kv, void* q, const void* k, const void* v,
+                                     int32_t batch, int32_t num_qo_heads, const int32_t* positions,
+                                     const int32_t* dst_slot, float rope_scale, float rope_theta,
+                                     void* stream) {
+  int rc = check_pool(kv, "td_rope_append_decode");
+  if (rc) return rc;
+  TD_REQUIRE(q && k && v && positions && dst_slot, "td_rope_append_decode: NULL argument");
+  TD_REQUIRE(batch >= 1 && num_qo_heads >= 1, "td_rope_append_decode: batch %d heads %d", batch,
+             num_qo_heads);
+  TD_REQUIRE(rope_scale > 0.f && rope_theta > 0.f, "td_rope_append_decode: scale %g theta %g",
+             rope_scale, rope_theta);
+  const int D = kv->head_dim;
+  if (D != 64 && D != 128 && D != 256)
+    return fail(TD_ERR_UNSUPPORTED, "td_rope_append_decode: head_dim %d (supported: 64, 128, 256)",
+                D);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const PoolGeom g = geom_of(kv);
+  const double inv_scale = 1.0 / (double)rope_scale;
+  const double log2_theta = log2((double)rope_theta);
+  if (kv->dtype == TD_F16)
+    hipLaunchKernelGGL(rope_append_decode_kernel<F16>, dim3(batch), dim3(256), 0, st, g,
+                       (uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, num_qo_heads, D,
+                       positions, dst_slot, inv_scale, log2_theta);
+  else if (kv->dtype == TD_BF16)
+    hipLaunchKernelGGL(rope_append_decode_kernel<BF16>, dim3(batch), dim3(256), 0, st, g,
+                       (uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, num_qo_heads, D,
+                       positions, dst_slot, inv_scale, log2_theta);
+  else
+    return fail(TD_ERR_UNSUPPORTED, "td_rope_append_decode failed to dispatch with dtype %d",
+                kv->dtype);
+  TD_HIP_CHECK(hipGetLastError());
+  return TD_OK;
+}
+
+extern "C" int td_rms_norm(const void* x, const void* weight, void* out, int32_t rows,
+                           int32_t cols, float eps, int32_t dtype, void* stream) {
+  TD_REQUIRE(x && weight && out, "rms_norm_forward: NULL argument");
+  TD_REQUIRE(rows >= 0 && cols >= 1, "rms_norm_forward: rows %d cols %d", rows, cols);
+  if (rows == 0) return TD_OK;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (dtype == TD_F16)
+    hipLaunchKernelGGL(rms_norm_kernel<F16>, dim3(rows), dim3(256), 0, st, (const uint16_t*)x,
+                       (const uint16_t*)weight, (uint16_t*)out, cols, eps);
+  else if (dtype == TD_BF16)
+    hipLaunchKernelGGL(rms_norm_kernel<BF16>, dim3(rows), dim3(256), 0, st, (const uint16_t*)x,
+                       (const uint16_t*)weight, (uint16_t*)out, cols, eps);
+  else
+    return fail(TD_ERR_UNSUPPORTED, "rms_norm_forward failed to dispatch with dtype %d", dtype);
+  TD_HIP_CHECK(hipGetLastError());
+  return TD_OK;
+}
