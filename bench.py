@@ -1,0 +1,308 @@
+#!/usr/bin/env python3
+"""Benchmark of the TidalDecode decode-attention path on one MI355X.
+
+Workload (BASELINE.json configs[1], Llama-2-7B shape): 32 layers, 32 query / 32 KV heads,
+head_dim 128, bf16 paged KV with page size 16 (pages scattered in the pool), context 32768
+tokens, top_k = 2048, token selection (full attention + logits + top-k) at layers 0 and 2, sparse
+attention over the persisted tokens in the other 30 layers.  One *step* is the attention path of
+one decode step over all 32 layers: fused RoPE + KV append, then selection or sparse attention.
+The cache holds synthetic N(0,1) data, already resident in HBM; every layer owns its 512 MiB
+pool, so a sparse layer reads cold data (the 30 layers touch ~1 GiB between two visits).
+
+Prints ONE JSON line.  `value` is the mean time of one sparse-layer attention launch (us/layer),
+measured with HIP events around a hipGraph that holds exactly the 30 sparse launches of a step.
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--ctx", type=int, default=32768)
+    ap.add_argument("--top-k", type=int, default=2048)
+    ap.add_argument("--layers", type=int, default=32)
+    ap.add_argument("--select-mode", default="per_head", choices=["per_head", "head_sum"])
+    ap.add_argument("--waves", type=int, default=0, help="waves per workgroup (0 = default)")
+    ap.add_argument("--chunk", type=int, default=0, help="tokens per workgroup (0 = default)")
+    ap.add_argument("--merge", type=int, default=-1, help="1 fused / 0 second kernel / -1 default")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of hipGraph")
+    ap.add_argument("--only-sparse", action="store_true",
+                    help="profile helper: run only the sparse-layer launches")
+    return ap.parse_args()
+
+
+class Workload:
+    """Controller + synthetic per-layer q/k/v for one decode step at a fixed context length."""
+
+    def __init__(self, args, select_mode):
+        import torch
+
+        from tidaldecode_amd.utils import InferenceController
+
+        self.torch = torch
+        self.dev = torch.device("cuda:0")
+        self.L, self.H, self.D, self.P = args.layers, 32, 128, 16
+        self.N, self.K = args.ctx, args.top_k
+        self.sel_layers = (0, 2)
+        self.dtype = torch.bfloat16
+        c = InferenceController(self.L, self.H, self.D, self.P, self.K, self.N + 64, self.dtype,
+                                self.dev, select_mode=select_mode, page_order_seed=0)
+        h = c._decode_handler._wrapper
+        h.waves_per_block, h.chunk_tokens, h.fused_merge = args.waves, args.chunk, args.merge
+        c.kv_cache.pool.buf.normal_()      # synthetic prefilled cache, resident in HBM
+        c.prepare_metadata(self.N)         # the prompt
+        c.prepare_metadata(1)              # the token being decoded
+        c.begin_forward(1)
+        self.c = c
+        g = torch.Generator(device=self.dev).manual_seed(0)
+        shape = (self.L, 1, self.H, self.D)
+        self.q = torch.randn(shape, generator=g, device=self.dev).to(self.dtype)
+        self.k = torch.randn(shape, generator=g, device=self.dev).to(self.dtype)
+        self.v = torch.randn(shape, generator=g, device=self.dev).to(self.dtype)
+        pos = c.kv_cache.seqlen - 1
+        self.positions = torch.tensor([pos], dtype=torch.int32, device=self.dev)
+        page = c.kv_cache.indicies[pos // self.P]
+        self.dst_slot = torch.tensor([page * self.P + pos % self.P], dtype=torch.int32,
+                                     device=self.dev)
+
+    # --- pieces of the step ---------------------------------------------------------------
+    def rope_append(self, layer):
+        from tidaldecode_amd import utils as ops
+
+        ops.rope_append_kv(self.q[layer], self.k[layer], self.v[layer], self.c, layer,
+                           self.positions, self.dst_slot)
+
+    def select_attn(self, layer):
+        from tidaldecode_amd import utils as ops
+
+        return ops.decode_sparse_attn(self.q[layer], self.c, layer,
+                                      self.c.kv_indices_without_last, True)
+
+    def topk(self):
+        from tidaldecode_amd import utils as ops
+
+        ops.decode_topk(self.c)
+
+    def sparse_attn(self, layer):
+        from tidaldecode_amd import utils as ops
+
+        return ops.decode_sparse_attn(self.q[layer], self.c, layer,
+                                      self.c.topk_dindices_buffer, False)
+
+    def step(self):
+        for layer in range(self.L):
+            self.rope_append(layer)
+            if layer in self.sel_layers:
+                self.select_attn(layer)
+                self.topk()
+            else:
+                self.sparse_attn(layer)
+
+    def sparse_layers(self):
+        return [l for l in range(self.L) if l not in self.sel_layers]
+
+
+def capture(torch, fn, use_graph):
+    """Returns a callable that replays fn (hipGraph unless disabled or capture fails)."""
+    if not use_graph:
+        return fn, "eager"
+    try:
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            fn()  # warm-up on the side stream: scratch buffers, plans
+        torch.cuda.current_stream().wait_stream(s)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            fn()
+        return g.replay, "hipGraph"
+    except Exception as e:  # pragma: no cover - depends on the runtime
+        print(f"[bench] graph capture failed ({e}); launching eagerly", file=sys.stderr)
+        torch.cuda.synchronize()
+        return fn, "eager"
+
+
+def time_events(torch, run, reps, warm=3):
+    """mean milliseconds of run() over reps, HIP events on the current stream"""
+    for _ in range(warm):
+        run()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        run()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / reps
+
+
+def cpu_baseline(args, budget_s=20.0):
+    """The CPU port of the reference's PyTorch path (dense logits -> mask -> fp32 softmax -> PV)
+    on this host: one selection layer and one sparse layer of the same workload."""
+    import torch
+
+    from oracle import tidal_oracle as orc
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    n, h, d, k = args.ctx, 32, 128, args.top_k
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn((h, d), generator=g)
+    kk = torch.randn((n, h, d), generator=g)
+    vv = torch.randn((n, h, d), generator=g)
+    t0 = time.perf_counter()
+    sel_t, sp_t = [], []
+    idx = None
+    while True:
+        t = time.perf_counter()
+        _, idx, _ = orc.select_layer(q, kk, vv, k, "per_head")
+        sel_t.append(time.perf_counter() - t)
+        mask = orc.mask_from_indices(idx, h, n)
+        t = time.perf_counter()
+        orc.sparse_layer(q, kk, vv, mask)
+        sp_t.append(time.perf_counter() - t)
+        if time.perf_counter() - t0 > budget_s or len(sp_t) >= 30:
+            break
+    return {
+        "value": round(statistics.median(sp_t) * 1e6, 1),
+        "unit": "us/layer",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"{len(sp_t)} runs of 1 selection + 1 sparse layer at ctx {n}, top_k {k}, "
+                  f"32 heads x 128, fp32, torch-CPU; median; selection layer "
+                  f"{statistics.median(sel_t) * 1e6:.0f} us",
+        "selection_us_per_layer": round(statistics.median(sel_t) * 1e6, 1),
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the decode-attention path of this build is "
+              "single-GPU (no collectives); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (libtidal_hip.so has no CPU path)", file=sys.stderr)
+        sys.exit(1)
+
+    use_graph = not args.no_graph
+    results = {}
+    for mode in ([args.select_mode] if args.only_sparse else
+                 [args.select_mode] + [m for m in ("per_head", "head_sum") if m != args.select_mode]):
+        w = Workload(args, mode)
+        # selection must run once so that the sparse layers have their token lists
+        w.step()
+        torch.cuda.synchronize()
+        sparse = w.sparse_layers()
+
+        def run_sparse():
+            for layer in sparse:
+                w.sparse_attn(layer)
+
+        r_sparse, how = capture(torch, run_sparse, use_graph)
+        sparse_ms = time_events(torch, r_sparse, max(args.steps, 20))
+        entry = {"sparse_us_per_layer": sparse_ms * 1e3 / len(sparse), "launch": how}
+        if not args.only_sparse:
+            def run_select():
+                for layer in w.sel_layers:
+                    w.select_attn(layer)
+
+            def run_topk():
+                for _ in w.sel_layers:
+                    w.topk()
+
+            def run_rope():
+                for layer in range(w.L):
+                    w.rope_append(layer)
+
+            r, _ = capture(torch, run_select, use_graph)
+            entry["selection_attn_us_per_layer"] = time_events(torch, r, 20) * 1e3 / len(w.sel_layers)
+            r, _ = capture(torch, run_topk, use_graph)
+            entry["topk_us_per_layer"] = time_events(torch, r, 20) * 1e3 / len(w.sel_layers)
+            r, _ = capture(torch, run_rope, use_graph)
+            entry["rope_append_us_per_layer"] = time_events(torch, r, 20) * 1e3 / w.L
+            # the contract's timed region: W warm-up steps, then exactly K steps
+            r_step, _ = capture(torch, w.step, use_graph)
+            for _ in range(args.warmup):
+                r_step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                r_step()
+            torch.cuda.synchronize()
+            entry["ms_per_step"] = (time.perf_counter() - t0) * 1e3 / args.steps
+        rows = w.c.index_rows
+        algo = (w.K * w.H * w.D * 2 * 2      # K and V rows of the attended tokens
+                + w.K * rows * 4             # the token list(s)
+                + 2 * w.H * w.D * 2)         # q in, o out
+        entry["algorithmic_bytes"] = algo
+        entry["achieved_gbs"] = algo / (entry["sparse_us_per_layer"] * 1e-6) / 1e9
+        sel_bytes = (w.c.kv_cache.seqlen * w.H * w.D * 2 * 2 + w.H * w.c.kv_cache.seqlen * 4
+                     + 2 * w.H * w.D * 2)
+        if "selection_attn_us_per_layer" in entry:
+            entry["selection_achieved_gbs"] = sel_bytes / (entry["selection_attn_us_per_layer"] * 1e-6) / 1e9
+        results[mode] = entry
+        del w
+        torch.cuda.empty_cache()
+
+    main_mode = args.select_mode
+    e = results[main_mode]
+    line = {
+        "metric": "sparse_decode_attn_us_per_layer",
+        "value": round(e["sparse_us_per_layer"], 3),
+        "unit": "us/layer",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(e.get("ms_per_step", float("nan")), 4),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"llama2-7b-shape decode attention path: {args.layers} layers, 32/32 heads, "
+                        f"head_dim 128, paged bf16 KV page 16, ctx {args.ctx}, top_k {args.top_k}, "
+                        f"selection at layers 0 and 2 ({main_mode} lists), batch 1",
+            "select_mode": main_mode,
+            "launch": e["launch"],
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(e["achieved_gbs"], 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(e["achieved_gbs"] / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "kernel": "decode_attn_kernel (sparse layer, token-slot lists)",
+            "algorithmic_bytes_per_launch": e["algorithmic_bytes"],
+        },
+        "detail": {m: {k: (round(v, 3) if isinstance(v, float) else v) for k, v in r.items()}
+                   for m, r in results.items()},
+    }
+    if "ms_per_step" in e:
+        line["attention_path_tokens_per_s"] = round(1e3 / e["ms_per_step"], 1)
+    if not args.no_cpu and not args.only_sparse:
+        line["cpu_baseline"] = cpu_baseline(args)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -173,9 +173,10 @@ int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t num_kv_head
  *   scores     optional [batch, num_qo_heads, score_stride]: element i = q . k_i / sqrt(D) of the
  *              i-th attended token in list order (td_dtype scores_dtype); NULL to skip
  *   lse        optional float [batch, num_qo_heads]: natural-log sum of exp of the logits
- *   workspace  device scratch of plan->workspace_bytes, zero-filled once before first use; the
- *              call leaves its ticket counters zero again.  Calls that share a workspace must
- *              be ordered on one stream.
+ *   workspace  device scratch of at least plan->workspace_bytes whose first 64 KiB (ticket
+ *              counters) were zero-filled once before first use; every call leaves them zero
+ *              again, so one workspace serves plans of any shape.  Calls that share a
+ *              workspace must be ordered on one stream.
  * Replaces BatchDecodeWithPagedKVCachePyTorchWrapper::Forward (bsk_ops.h:104-113,
  * tidal/ops/csrc/approx_attn.cu:68-151), BatchDecodeWithPagedKVCacheKernel
  * (kernels/include/decode/decode_attn.cuh:432-658) including its score output

@@ -33,7 +33,8 @@ def _check(values, k, cuda):
     assert torch.equal(got.long(), want), "index set differs from the stable oracle"
     want_c = cref.stable_topk(values.float().numpy(), k)
     assert np.array_equal(got.numpy(), want_c)
-    assert torch.equal(vals, torch.gather(values, 1, want))  # values travel with their index
+    expect = torch.gather(values, 1, want)  # values travel with their index (NaN == NaN here)
+    assert torch.equal(torch.nan_to_num(vals.float(), nan=1e38), torch.nan_to_num(expect.float(), nan=1e38))
     return got
 
 

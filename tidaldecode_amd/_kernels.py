@@ -39,6 +39,16 @@ def _check_input(x: torch.Tensor, name: str) -> None:
         raise RuntimeError(f"{name} must be contiguous")
 
 
+def _check_rows(x: torch.Tensor, name: str) -> None:
+    """2-D device tensor whose rows are dense (a column slice of a wider buffer is fine)."""
+    if not x.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if x.dim() != 2:
+        raise RuntimeError(f"{name} must be a 2D tensor")
+    if x.numel() > 0 and x.stride(1) != 1:
+        raise RuntimeError(f"{name} must have dense rows")
+
+
 def _check_dim(d: int, x: torch.Tensor, name: str) -> None:
     if x.dim() != d:
         raise RuntimeError(f"{name} must be a {d}D tensor")
@@ -120,8 +130,7 @@ def topk_filtering(estimated_value: torch.Tensor, estimated_indices: Optional[to
     Extensions: ``estimated_indices=None`` returns positions, or physical token slots when a
     ``page_table`` ``[n_pages]`` is given; fp32 values.
     """
-    _check_input(estimated_value, "estimated_value")
-    _check_dim(2, estimated_value, "estimated_value")
+    _check_rows(estimated_value, "estimated_value")
     rows, length = estimated_value.shape
     in_ptr, in_stride = None, 0
     if estimated_indices is not None:
@@ -132,15 +141,16 @@ def topk_filtering(estimated_value: torch.Tensor, estimated_indices: Optional[to
             raise RuntimeError("estimated_value and estimated_indices differ in rows")
         length = min(length, estimated_indices.size(1))
         in_ptr, in_stride = estimated_indices.data_ptr(), estimated_indices.size(1)
-    _check_input(indices_out, "indices_out")
+    _check_rows(indices_out, "indices_out")
     _check_i32(indices_out, "indices_out")
     k = int(page_budget)
     if indices_out.dim() != 2 or indices_out.size(0) != rows or indices_out.size(1) != k:
         raise RuntimeError(f"indices_out must be [{rows}, {k}]")
     out_vals = None
     if d_out is not None and d_out.numel() > 0:
-        _check_input(d_out, "d_out")
-        if d_out.shape != indices_out.shape or d_out.dtype != estimated_value.dtype:
+        _check_rows(d_out, "d_out")
+        if d_out.shape != indices_out.shape or d_out.dtype != estimated_value.dtype or \
+                d_out.stride(0) != indices_out.stride(0):
             raise RuntimeError("d_out must match indices_out in shape and estimated_value in dtype")
         out_vals = d_out.data_ptr()
     if k > length:
@@ -343,9 +353,8 @@ class BatchDecodeWithPagedKVCachePyTorchWrapper:
                                "BatchDecodeWithPagedKVCacheWrapper()")
         _check_input(q, "q")
         _check_input(o, "o")
-        _check_input(paged_kv_indices, "paged_kv_indices")
+        _check_rows(paged_kv_indices, "paged_kv_indices")
         _check_dim(3, q, "q")
-        _check_dim(2, paged_kv_indices, "paged_kv_indices")
         _check_i32(paged_kv_indices, "paged_kv_indices")
         pool = _pool(paged_kv_data, self._layout, "paged_kv_data")
         hq, hkv, d, page, dtype = self._geom

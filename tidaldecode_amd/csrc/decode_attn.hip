@@ -510,6 +510,11 @@ static int launch_merge(const DecodeParams& p, int head_dim, dim3 grid, hipStrea
 
 static int64_t align256(int64_t x) { return (x + 255) & ~(int64_t)255; }
 
+// Workspace layout: [ticket counters, fixed size | partial o | partial (m, l)].  The counters sit
+// at a fixed place so that plans of different shapes sharing one workspace never find another
+// plan's partial results where they expect zeroed tickets.
+constexpr int64_t kTicketBytes = 65536;
+
 }  // namespace tidal
 
 using namespace tidal;
@@ -564,9 +569,11 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
   plan->waves_per_block = nw;
   if (plan->fused_merge < 0) plan->fused_merge = 1;
   plan->fused_merge = plan->fused_merge ? 1 : 0;
+  TD_REQUIRE((int64_t)batch * head_groups * 4 <= kTicketBytes,
+             "td_decode_make_plan: batch %d x %d head groups exceeds the %lld ticket counters", batch,
+             head_groups, (long long)(kTicketBytes / 4));
   const int64_t n_part = (int64_t)batch * num_qo_heads * max_splits;
-  plan->workspace_bytes = align256(n_part * head_dim * 4) + align256(n_part * 2 * 4) +
-                          align256((int64_t)batch * head_groups * 4);
+  plan->workspace_bytes = kTicketBytes + align256(n_part * head_dim * 4) + align256(n_part * 2 * 4);
   return TD_OK;
 }
 
@@ -628,9 +635,12 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
   const int head_groups = (n_hrows + hpw - 1) / hpw;
 
   const int64_t n_part = (int64_t)batch * num_qo_heads * plan->max_splits;
-  const int64_t off_ml = align256(n_part * D * 4);
-  const int64_t off_cnt = off_ml + align256(n_part * 2 * 4);
-  const int64_t need = off_cnt + align256((int64_t)batch * head_groups * 4);
+  const int64_t off_o = kTicketBytes;
+  const int64_t off_ml = off_o + align256(n_part * D * 4);
+  const int64_t need = off_ml + align256(n_part * 2 * 4);
+  TD_REQUIRE((int64_t)batch * head_groups * 4 <= kTicketBytes,
+             "td_decode_attn: batch %d x %d head groups exceeds the ticket counters", batch,
+             head_groups);
   if (plan->max_splits > 1) {
     if (workspace == nullptr || workspace_bytes < need)
       return fail(TD_ERR_STATE,
@@ -680,9 +690,9 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
   p.score_stride = score_stride;
   p.lse = lse;
   char* ws = reinterpret_cast<char*>(workspace);
-  p.ws_o = reinterpret_cast<float*>(ws);
+  p.ws_cnt = reinterpret_cast<int32_t*>(ws);
+  p.ws_o = reinterpret_cast<float*>(ws ? ws + off_o : nullptr);
   p.ws_ml = reinterpret_cast<float*>(ws ? ws + off_ml : nullptr);
-  p.ws_cnt = reinterpret_cast<int32_t*>(ws ? ws + off_cnt : nullptr);
 
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const bool page_mode = list->kind == TD_IDX_PAGES;

@@ -198,8 +198,8 @@ __global__ __launch_bounds__(kTopkThreads) void topk_kernel(const TopkParams p) 
     const uint32_t eq_rank = eq_run + (uint32_t)__popcll(eq_mask & lt_mask);
     const bool sel = gt || (eq && eq_rank < r);
     const uint64_t sel_mask = __ballot(sel);
-    if (sel) {
-      const uint32_t pos = out_run + (uint32_t)__popcll(sel_mask & lt_mask);
+    const uint32_t pos = out_run + (uint32_t)__popcll(sel_mask & lt_mask);
+    if (sel && pos < (uint32_t)k) {
       int32_t payload;
       if (p.in_idx)
         payload = p.in_idx[(int64_t)row * p.in_idx_stride + i];
