@@ -60,7 +60,7 @@ struct DecodeParams {
   float* lse;
   float* ws_o;      // [batch * H_q * max_splits, D]
   float* ws_ml;     // [batch * H_q * max_splits, 2]
-  int32_t* ws_cnt;  // [batch * head_groups]
+  int32_t* ws_cnt;  // [batch * head rows] ticket counters
 };
 
 __device__ __forceinline__ void divmod_page(const DecodeParams& p, uint32_t x, uint32_t& page,
@@ -83,21 +83,36 @@ struct SeqList {
   int32_t last_idx;
 };
 
-// Element offset of the K row of item i (slot clamped into the pool); items past the end map
-// to slot 0, a valid address whose contribution is masked out.
+// Physical (page, entry) of item i as one packed word; items past the end map to slot 0, a valid
+// address whose contribution is masked out.  `raw` is what had to be fetched from the list.
+template <bool PAGE_MODE>
+__device__ __forceinline__ bool item_needs_load(const SeqList& s, const DecodeParams& p, int32_t i,
+                                                uint32_t& list_pos) {
+  if (i >= s.n_items) return false;
+  if constexpr (PAGE_MODE) {
+    uint32_t pg, e;
+    divmod_page(p, (uint32_t)i, pg, e);
+    list_pos = pg;
+    return (int32_t)pg < s.n_list;
+  } else {
+    list_pos = (uint32_t)i;
+    return i < s.n_list;
+  }
+}
+
 template <bool PAGE_MODE>
 __device__ __forceinline__ int64_t item_offset(const DecodeParams& p, const SeqList& s, int32_t i,
-                                               int32_t kv_head_off) {
+                                               int32_t raw, int32_t kv_head_off) {
   uint32_t page = 0, entry = 0;
   if (i < s.n_items) {
     if constexpr (PAGE_MODE) {
-      uint32_t li, e;
-      divmod_page(p, (uint32_t)i, li, e);
-      page = ((int32_t)li < s.n_list) ? (uint32_t)s.row[li] : (uint32_t)s.last_idx;
+      uint32_t pg, e;
+      divmod_page(p, (uint32_t)i, pg, e);
+      page = ((int32_t)pg < s.n_list) ? (uint32_t)raw : (uint32_t)s.last_idx;
       entry = e;
       page = page > p.max_page ? p.max_page : page;
     } else {
-      uint32_t slot = (i < s.n_list) ? (uint32_t)s.row[i]
+      uint32_t slot = (i < s.n_list) ? (uint32_t)raw
                                      : (uint32_t)s.last_idx * (uint32_t)p.page_size +
                                            (uint32_t)(i - s.n_list);
       slot = slot > p.max_slot ? p.max_slot : slot;
@@ -107,28 +122,102 @@ __device__ __forceinline__ int64_t item_offset(const DecodeParams& p, const SeqL
   return (int64_t)page * p.page_stride + (int64_t)entry * p.entry_stride + kv_head_off;
 }
 
-template <typename T, int D, int QPG, int U, int NW, bool PAGE_MODE, bool EMIT>
-__global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams p) {
-  constexpr int LPR = D / 8;     // lanes per row
-  constexpr int HPW = 64 / LPR;  // head rows per wave
+// 8-byte device-coherent accesses for the split partials: they are written by one workgroup and
+// read by another that may sit on a different XCD (own L2), so they go to memory (sc1) instead
+// of relying on an L2-wide write-back fence.
+__device__ __forceinline__ void store_coherent(float* dst, float a, float b) {
+  const uint64_t v = (uint64_t)__builtin_bit_cast(uint32_t, a) |
+                     ((uint64_t)__builtin_bit_cast(uint32_t, b) << 32);
+  __hip_atomic_store(reinterpret_cast<uint64_t*>(dst), v, __ATOMIC_RELAXED,
+                     __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void load_coherent(const float* src, float& a, float& b) {
+  const uint64_t v = __hip_atomic_load(reinterpret_cast<const uint64_t*>(src), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+  a = __builtin_bit_cast(float, (uint32_t)v);
+  b = __builtin_bit_cast(float, (uint32_t)(v >> 32));
+}
+
+// Reduce the n_splits partial results of the QPG query heads of one head row and write o (and
+// lse).  Runs in one workgroup of NT threads: NT / (QPG * D / 2) "slots" of threads each own a
+// float2 column and a subset of the splits; slots are combined through LDS.
+template <typename T, int D, int QPG, int NT>
+__device__ __forceinline__ void merge_splits(const DecodeParams& p, int b, int qh0, int n_splits) {
+  constexpr int COLS = QPG * D / 2;
+  constexpr int SLOTS = NT / COLS;
+  constexpr int PRE = 4;  // partial loads kept in flight per thread
+  static_assert(SLOTS >= 1, "workgroup too small for the merge");
+  __shared__ float mg_m[QPG][64], mg_l[QPG][64];
+  __shared__ float mg_part[SLOTS][COLS][2];
   const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int g = lane / LPR;   // lane group = head row inside the wave
-  const int li = lane % LPR;  // 16-byte column of the row
-  const int hg = blockIdx.x;
-  const int split = blockIdx.y;
-  const int b = blockIdx.z;
+  const int c = tid % COLS, slot = tid / COLS;
+  const int j = c / (D / 2), d2 = c % (D / 2);
+  const int64_t part0 = ((int64_t)b * p.num_qo_heads + qh0 + j) * p.max_splits;
 
-  const int hrow_raw = hg * HPW + g;
-  const bool head_ok = hrow_raw < p.n_hrows;
-  const int hrow = head_ok ? hrow_raw : p.n_hrows - 1;
-  const int kv_head = (QPG > 1) ? hrow : hrow / p.q_per_kv;
-  const int qh0 = hrow * QPG;  // first query head of this lane group
+  float ml_m = kNegBig, ml_l = 0.f;
+  const bool has_ml = tid < n_splits * QPG;
+  if (has_ml) {
+    const int jj = tid / n_splits, ss = tid % n_splits;
+    load_coherent(p.ws_ml + (((int64_t)b * p.num_qo_heads + qh0 + jj) * p.max_splits + ss) * 2,
+                  ml_m, ml_l);
+  }
+  float pa[PRE], pb[PRE];
+#pragma unroll
+  for (int u = 0; u < PRE; ++u) {
+    const int sidx = slot + u * SLOTS;
+    pa[u] = pb[u] = 0.f;
+    if (slot < SLOTS && sidx < n_splits) load_coherent(p.ws_o + (part0 + sidx) * D + d2 * 2, pa[u], pb[u]);
+  }
+  if (has_ml) {
+    mg_m[tid / n_splits][tid % n_splits] = ml_m;
+    mg_l[tid / n_splits][tid % n_splits] = ml_l;
+  }
+  __syncthreads();
+  float M = kNegBig;
+  for (int sidx = 0; sidx < n_splits; ++sidx) M = fmaxf(M, mg_m[j][sidx]);
+  float ra = 0.f, rb = 0.f;
+  if (slot < SLOTS) {
+#pragma unroll
+    for (int u = 0; u < PRE; ++u) {
+      const int sidx = slot + u * SLOTS;
+      if (sidx < n_splits) {
+        const float f = fast_exp2(mg_m[j][sidx] - M);
+        ra = fmaf(pa[u], f, ra);
+        rb = fmaf(pb[u], f, rb);
+      }
+    }
+    for (int sidx = slot + PRE * SLOTS; sidx < n_splits; sidx += SLOTS) {
+      float xa, xb;
+      load_coherent(p.ws_o + (part0 + sidx) * D + d2 * 2, xa, xb);
+      const float f = fast_exp2(mg_m[j][sidx] - M);
+      ra = fmaf(xa, f, ra);
+      rb = fmaf(xb, f, rb);
+    }
+    mg_part[slot][c][0] = ra;
+    mg_part[slot][c][1] = rb;
+  }
+  __syncthreads();
+  if (tid < COLS) {
+    float L = 0.f;
+    for (int sidx = 0; sidx < n_splits; ++sidx)
+      L = fmaf(mg_l[j][sidx], fast_exp2(mg_m[j][sidx] - M), L);
+    float oa = 0.f, ob = 0.f;
+#pragma unroll
+    for (int sl = 0; sl < SLOTS; ++sl) {
+      oa += mg_part[sl][c][0];
+      ob += mg_part[sl][c][1];
+    }
+    const float inv = L > 0.f ? 1.f / L : 0.f;
+    const int qh = qh0 + j;
+    reinterpret_cast<uint32_t*>(p.o)[((int64_t)b * p.num_qo_heads + qh) * (D / 2) + d2] =
+        pack2<T>(oa * inv, ob * inv);
+    if (p.lse && d2 == 0)
+      p.lse[(int64_t)b * p.num_qo_heads + qh] = L > 0.f ? (M + fast_log2(L)) * kLn2 : -INFINITY;
+  }
+}
 
-  // sequence descriptor
-  SeqList s;
-  int list_beg = 0;
+__device__ __forceinline__ int seq_items(const DecodeParams& p, int b, SeqList& s, int& list_beg) {
+  list_beg = 0;
   if (p.indptr) {
     list_beg = p.indptr[b];
     s.n_list = p.indptr[b + 1] - list_beg;
@@ -138,13 +227,33 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
   s.n_list = s.n_list < 0 ? 0 : (s.n_list > p.n_list_host ? p.n_list_host : s.n_list);
   s.last_len = p.last_len_arr ? p.last_len_arr[b] : p.last_len;
   s.last_idx = p.last_idx_arr ? p.last_idx_arr[b] : p.last_idx;
-  s.n_items = (PAGE_MODE ? s.n_list * p.page_size : s.n_list) + s.last_len;
+  s.n_items = (p.page_mode ? s.n_list * p.page_size : s.n_list) + s.last_len;
+  int n_splits = (s.n_items + p.chunk_tokens - 1) / p.chunk_tokens;
+  return n_splits < 1 ? 1 : n_splits;
+}
+
+template <typename T, int D, int QPG, int U, int NW, bool PAGE_MODE, bool EMIT>
+__global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams p) {
+  constexpr int LPR = D / 8;     // lanes per K/V row
+  constexpr int TPI = 64 / LPR;  // tokens one wave instruction covers
+  constexpr int TILE = U * TPI;  // tokens per wave tile
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int g = lane / LPR;   // lane group = token slot inside the instruction
+  const int li = lane % LPR;  // 16-byte column of the row
+  const int hrow = blockIdx.x;
+  const int split = blockIdx.y;
+  const int b = blockIdx.z;
+  const int kv_head = (QPG > 1) ? hrow : hrow / p.q_per_kv;
+  const int qh0 = hrow * QPG;  // first query head of this head row
+
+  SeqList s;
+  int list_beg;
+  const int n_splits = seq_items(p, b, s, list_beg);
+  if (split >= n_splits) return;  // uniform for the whole workgroup
   const int idx_row = (QPG == 1 && p.idx_per_kv) ? kv_head : hrow;
   s.row = p.idx + (int64_t)idx_row * p.idx_row_stride + list_beg;
-
-  int n_splits = (s.n_items + p.chunk_tokens - 1) / p.chunk_tokens;
-  n_splits = n_splits < 1 ? 1 : n_splits;
-  if (split >= n_splits) return;  // uniform for the whole workgroup
 
   const int c0 = split * p.chunk_tokens;
   int c1 = c0 + p.chunk_tokens;
@@ -157,7 +266,7 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
         reinterpret_cast<const u32x4*>(p.q) + ((int64_t)b * p.num_qo_heads + qh0) * LPR + li;
 #pragma unroll
     for (int j = 0; j < QPG; ++j) {
-      u32x4 v = qptr[j * LPR];
+      const u32x4 v = qptr[j * LPR];
       qp[j][0] = v.x;
       qp[j][1] = v.y;
       qp[j][2] = v.z;
@@ -177,29 +286,37 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
   const int kv_head_off = kv_head * p.head_stride + li * 8;
   const uint16_t* kv16 = reinterpret_cast<const uint16_t*>(p.kv);
 
-  // ---- tile pipeline: loads of tile t+1 are in flight while tile t is reduced ----
+  // ---- software pipeline over this wave's tiles ------------------------------------------------
+  // program order per iteration: list entries of tile t+2, K/V rows of tile t+1, arithmetic of
+  // tile t.  Waiting for older list entries never waits for younger K/V loads, so two tiles of
+  // K/V stay in flight per wave.
   u32x4 kA[U], vA[U], kB[U], vB[U];
-  int64_t offN[U];  // element offsets of the tile whose loads are issued next
+  int32_t rawA[U], rawB[U];
 
-  auto lookup = [&](int base) {
+  auto fetch_list = [&](int base, int32_t(&raw)[U]) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      int i = base + u;
-      offN[u] = item_offset<PAGE_MODE>(p, s, i < c1 ? i : s.n_items, kv_head_off);
+      const int i = base + u * TPI + g;
+      uint32_t pos = 0;
+      raw[u] = 0;
+      if (i < c1 && item_needs_load<PAGE_MODE>(s, p, i, pos)) raw[u] = s.row[pos];
     }
   };
-  auto issue = [&](u32x4(&kb)[U], u32x4(&vb)[U]) {
+  auto issue = [&](int base, const int32_t(&raw)[U], u32x4(&kb)[U], u32x4(&vb)[U]) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      kb[u] = *reinterpret_cast<const u32x4*>(kv16 + offN[u]);
-      vb[u] = *reinterpret_cast<const u32x4*>(kv16 + offN[u] + p.v_offset);
+      const int i = base + u * TPI + g;
+      const int64_t off = item_offset<PAGE_MODE>(p, s, i < c1 ? i : s.n_items, raw[u], kv_head_off);
+      kb[u] = *reinterpret_cast<const u32x4*>(kv16 + off);
+      vb[u] = *reinterpret_cast<const u32x4*>(kv16 + off + p.v_offset);
     }
   };
   auto reduce = [&](const u32x4(&kb)[U], const u32x4(&vb)[U], int base) {
     float sc[QPG][U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const bool valid = base + u < c1;
+      const int i = base + u * TPI + g;
+      const bool valid = i < c1;
 #pragma unroll
       for (int j = 0; j < QPG; ++j) {
         float a = dot2<T>(qp[j][0], kb[u].x, 0.f);
@@ -209,9 +326,8 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
         a = group_sum<LPR>(a) * p.scale_log2;
         sc[j][u] = valid ? a : kNegBig;
         if constexpr (EMIT) {
-          if (valid && head_ok && li == 0) {
-            const int64_t at =
-                ((int64_t)b * p.num_qo_heads + qh0 + j) * p.score_stride + (base + u);
+          if (valid && li == 0) {
+            const int64_t at = ((int64_t)b * p.num_qo_heads + qh0 + j) * p.score_stride + i;
             const float nat = a * kLn2;
             if (p.scores_f32)
               reinterpret_cast<float*>(p.scores)[at] = nat;
@@ -233,7 +349,7 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
       float ps = 0.f;
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        pr[u] = (base + u < c1) ? fast_exp2(sc[j][u] - m_new) : 0.f;
+        pr[u] = (base + u * TPI + g < c1) ? fast_exp2(sc[j][u] - m_new) : 0.f;
         ps += pr[u];
       }
       l[j] = l[j] * alpha + ps;
@@ -258,163 +374,125 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
     }
   };
 
-  constexpr int STEP = NW * U;  // tokens between two tiles of one wave
-  int t = c0 + wave * U;        // first token of this wave's current tile
+  constexpr int STEP = NW * TILE;  // tokens between two tiles of one wave
+  int t = c0 + wave * TILE;        // first token of this wave's current tile
   if (t < c1) {
-    lookup(t);
-    issue(kA, vA);
+    fetch_list(t, rawA);
+    if (t + STEP < c1) fetch_list(t + STEP, rawB);
+    issue(t, rawA, kA, vA);
     while (true) {
-      // stage A holds tile t
+      // A: K/V of tile t in flight; rawB: list entries of tile t+STEP in flight
       const int tn = t + STEP;
-      if (tn < c1) {
-        lookup(tn);
-        issue(kB, vB);
-      }
+      const int tnn = tn + STEP;
+      if (tnn < c1) fetch_list(tnn, rawA);
+      if (tn < c1) issue(tn, rawB, kB, vB);
       reduce(kA, vA, t);
       if (tn >= c1) break;
-      const int tnn = tn + STEP;
-      if (tnn < c1) {
-        lookup(tnn);
-        issue(kA, vA);
-      }
+      const int tnnn = tnn + STEP;
+      if (tnnn < c1) fetch_list(tnnn, rawB);
+      if (tnn < c1) issue(tnn, rawA, kA, vA);
       reduce(kB, vB, tn);
       if (tnn >= c1) break;
       t = tnn;
     }
   }
 
-  // ---- merge the NW wave states of the workgroup through LDS ----
-  __shared__ float sm_o[NW][8][64];
-  __shared__ float sm_ml[NW][2][64];
+  // ---- combine the TPI token slots of the wave (butterfly over lane groups) ---------------------
+#pragma unroll
+  for (int j = 0; j < QPG; ++j) {
+    float mw = m[j];
+#pragma unroll
+    for (int off = LPR; off < 64; off <<= 1) mw = fmaxf(mw, __shfl_xor(mw, off, 64));
+    const float f = fast_exp2(m[j] - mw);
+    m[j] = mw;
+    l[j] *= f;
+#pragma unroll
+    for (int d = 0; d < 8; ++d) acc[j][d] *= f;
+#pragma unroll
+    for (int off = LPR; off < 64; off <<= 1) {
+      l[j] += __shfl_xor(l[j], off, 64);
+#pragma unroll
+      for (int d = 0; d < 8; ++d) acc[j][d] += __shfl_xor(acc[j][d], off, 64);
+    }
+  }
+
+  // ---- merge the NW wave states of the workgroup through LDS ------------------------------------
+  __shared__ float sm_o[NW][8][LPR];
+  __shared__ float sm_ml[NW][2];
   __shared__ int sm_ticket;
 #pragma unroll
   for (int j = 0; j < QPG; ++j) {
     if (j > 0) __syncthreads();
+    if (lane < LPR) {
 #pragma unroll
-    for (int d = 0; d < 8; ++d) sm_o[wave][d][lane] = acc[j][d];
-    sm_ml[wave][0][lane] = m[j];
-    sm_ml[wave][1][lane] = l[j];
+      for (int d = 0; d < 8; ++d) sm_o[wave][d][lane] = acc[j][d];
+      if (lane == 0) {
+        sm_ml[wave][0] = m[j];
+        sm_ml[wave][1] = l[j];
+      }
+    }
     __syncthreads();
-    if (wave == (j % NW)) {
+    if (wave == (j % NW) && lane < LPR) {
       float M = kNegBig;
 #pragma unroll
-      for (int w = 0; w < NW; ++w) M = fmaxf(M, sm_ml[w][0][lane]);
+      for (int w = 0; w < NW; ++w) M = fmaxf(M, sm_ml[w][0]);
       float L = 0.f, r[8];
 #pragma unroll
       for (int d = 0; d < 8; ++d) r[d] = 0.f;
 #pragma unroll
       for (int w = 0; w < NW; ++w) {
-        const float f = fast_exp2(sm_ml[w][0][lane] - M);
-        L = fmaf(sm_ml[w][1][lane], f, L);
+        const float f = fast_exp2(sm_ml[w][0] - M);
+        L = fmaf(sm_ml[w][1], f, L);
 #pragma unroll
         for (int d = 0; d < 8; ++d) r[d] = fmaf(sm_o[w][d][lane], f, r[d]);
       }
-      // result of query head qh0 + j now lives in wave (j % NW)
       const int qh = qh0 + j;
-      if (head_ok) {
-        if (n_splits == 1) {
-          const float inv = L > 0.f ? 1.f / L : 0.f;
-          u32x4 out;
-          out.x = pack2<T>(r[0] * inv, r[1] * inv);
-          out.y = pack2<T>(r[2] * inv, r[3] * inv);
-          out.z = pack2<T>(r[4] * inv, r[5] * inv);
-          out.w = pack2<T>(r[6] * inv, r[7] * inv);
-          reinterpret_cast<u32x4*>(p.o)[((int64_t)b * p.num_qo_heads + qh) * LPR + li] = out;
-          if (p.lse && li == 0)
-            p.lse[(int64_t)b * p.num_qo_heads + qh] =
-                L > 0.f ? (M + fast_log2(L)) * kLn2 : -INFINITY;
-        } else {
-          const int64_t slot = ((int64_t)b * p.num_qo_heads + qh) * p.max_splits + split;
-          f32x4* dst = reinterpret_cast<f32x4*>(p.ws_o + slot * D + li * 8);
-          f32x4 a0 = {r[0], r[1], r[2], r[3]};
-          f32x4 a1 = {r[4], r[5], r[6], r[7]};
-          dst[0] = a0;
-          dst[1] = a1;
-          if (li == 0) {
-            p.ws_ml[slot * 2 + 0] = M;
-            p.ws_ml[slot * 2 + 1] = L;
-          }
-        }
+      if (n_splits == 1) {
+        const float inv = L > 0.f ? 1.f / L : 0.f;
+        u32x4 out;
+        out.x = pack2<T>(r[0] * inv, r[1] * inv);
+        out.y = pack2<T>(r[2] * inv, r[3] * inv);
+        out.z = pack2<T>(r[4] * inv, r[5] * inv);
+        out.w = pack2<T>(r[6] * inv, r[7] * inv);
+        reinterpret_cast<u32x4*>(p.o)[((int64_t)b * p.num_qo_heads + qh) * LPR + lane] = out;
+        if (p.lse && lane == 0)
+          p.lse[(int64_t)b * p.num_qo_heads + qh] = L > 0.f ? (M + fast_log2(L)) * kLn2 : -INFINITY;
+      } else {
+        const int64_t part = ((int64_t)b * p.num_qo_heads + qh) * p.max_splits + split;
+        float* dst = p.ws_o + part * D + lane * 8;
+        store_coherent(dst + 0, r[0], r[1]);
+        store_coherent(dst + 2, r[2], r[3]);
+        store_coherent(dst + 4, r[4], r[5]);
+        store_coherent(dst + 6, r[6], r[7]);
+        if (lane == 0) store_coherent(p.ws_ml + part * 2, M, L);
       }
     }
   }
 
   if (n_splits == 1 || !p.fused_merge) return;
 
-  // ---- last-arriving workgroup of this (sequence, head group) reduces the partials ----
-  __threadfence();
+  // ---- the last workgroup of this (sequence, head row) to arrive reduces the partials ----------
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // partial stores have left this CU
   __syncthreads();
-  if (tid == 0) sm_ticket = atomicAdd(p.ws_cnt + (int64_t)b * gridDim.x + hg, 1);
+  int32_t* ticket = p.ws_cnt + (int64_t)b * gridDim.x + hrow;
+  if (tid == 0)
+    sm_ticket = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
   if (sm_ticket != n_splits - 1) return;
-  __threadfence();
-
-  constexpr int NQ = HPW * QPG;  // query heads of this head group
-  const int qh_base = hg * NQ;
-  for (int e = tid * 4; e < NQ * D; e += NW * 64 * 4) {
-    const int qh = qh_base + e / D;
-    const int d = e % D;
-    if (qh >= p.num_qo_heads) break;
-    const int64_t slot0 = ((int64_t)b * p.num_qo_heads + qh) * p.max_splits;
-    float M = kNegBig;
-    for (int sidx = 0; sidx < n_splits; ++sidx)
-      M = fmaxf(M, p.ws_ml[(slot0 + sidx) * 2]);
-    float L = 0.f;
-    f32x4 r = {0.f, 0.f, 0.f, 0.f};
-    for (int sidx = 0; sidx < n_splits; ++sidx) {
-      const float ms = p.ws_ml[(slot0 + sidx) * 2];
-      const float ls = p.ws_ml[(slot0 + sidx) * 2 + 1];
-      const float f = fast_exp2(ms - M);
-      L = fmaf(ls, f, L);
-      const f32x4 po = *reinterpret_cast<const f32x4*>(p.ws_o + (slot0 + sidx) * D + d);
-      r += po * f;
-    }
-    const float inv = L > 0.f ? 1.f / L : 0.f;
-    u32x2 out;
-    out.x = pack2<T>(r.x * inv, r.y * inv);
-    out.y = pack2<T>(r.z * inv, r.w * inv);
-    *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(p.o) +
-                              ((int64_t)b * p.num_qo_heads + qh) * D + d) = out;
-    if (p.lse && d == 0)
-      p.lse[(int64_t)b * p.num_qo_heads + qh] = L > 0.f ? (M + fast_log2(L)) * kLn2 : -INFINITY;
-  }
-  if (tid == 0) p.ws_cnt[(int64_t)b * gridDim.x + hg] = 0;
+  merge_splits<T, D, QPG, NW * 64>(p, b, qh0, n_splits);
+  if (tid == 0) __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Second-kernel merge: one workgroup of 64*... threads per (sequence, query head).
-template <typename T, int D>
-__global__ __launch_bounds__(D / 4) void merge_partials_kernel(const DecodeParams p) {
-  const int qh = blockIdx.x;
+// Second-kernel merge (plan.fused_merge == 0): one workgroup per (head row, sequence).
+template <typename T, int D, int QPG, int NT>
+__global__ __launch_bounds__(NT) void merge_partials_kernel(const DecodeParams p) {
+  const int hrow = blockIdx.x;
   const int b = blockIdx.y;
-  const int d = threadIdx.x * 4;
-  int n_list;
-  if (p.indptr)
-    n_list = p.indptr[b + 1] - p.indptr[b];
-  else
-    n_list = p.n_list_host;
-  n_list = n_list < 0 ? 0 : (n_list > p.n_list_host ? p.n_list_host : n_list);
-  const int last_len = p.last_len_arr ? p.last_len_arr[b] : p.last_len;
-  const int n_items = (p.page_mode ? n_list * p.page_size : n_list) + last_len;
-  int n_splits = (n_items + p.chunk_tokens - 1) / p.chunk_tokens;
+  SeqList s;
+  int list_beg;
+  const int n_splits = seq_items(p, b, s, list_beg);
   if (n_splits <= 1) return;  // the attention kernel already wrote the final result
-  const int64_t slot0 = ((int64_t)b * p.num_qo_heads + qh) * p.max_splits;
-  float M = kNegBig;
-  for (int sidx = 0; sidx < n_splits; ++sidx) M = fmaxf(M, p.ws_ml[(slot0 + sidx) * 2]);
-  float L = 0.f;
-  f32x4 r = {0.f, 0.f, 0.f, 0.f};
-  for (int sidx = 0; sidx < n_splits; ++sidx) {
-    const float f = fast_exp2(p.ws_ml[(slot0 + sidx) * 2] - M);
-    L = fmaf(p.ws_ml[(slot0 + sidx) * 2 + 1], f, L);
-    r += *reinterpret_cast<const f32x4*>(p.ws_o + (slot0 + sidx) * D + d) * f;
-  }
-  const float inv = L > 0.f ? 1.f / L : 0.f;
-  u32x2 out;
-  out.x = pack2<T>(r.x * inv, r.y * inv);
-  out.y = pack2<T>(r.z * inv, r.w * inv);
-  *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(p.o) +
-                            ((int64_t)b * p.num_qo_heads + qh) * D + d) = out;
-  if (p.lse && d == 0)
-    p.lse[(int64_t)b * p.num_qo_heads + qh] = L > 0.f ? (M + fast_log2(L)) * kLn2 : -INFINITY;
+  merge_splits<T, D, QPG, NT>(p, b, hrow * QPG, n_splits);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -435,7 +513,7 @@ static int num_cus() {
   return g_num_cus;
 }
 
-constexpr int kTileTokens = 4;  // U
+constexpr int kTileInstr = 4;  // U: K/V load instructions per wave tile and stream
 
 static int qpg_for(int num_qo_heads, int num_kv_heads, int idx_rows) {
   // KV rows are shared between the query heads of a group only when the group shares its list
@@ -445,9 +523,9 @@ static int qpg_for(int num_qo_heads, int num_kv_heads, int idx_rows) {
 }
 
 template <typename T, int D, int QPG, int NW>
-static void launch_variant(const DecodeParams& p, bool page_mode, bool emit, dim3 grid,
-                           hipStream_t st) {
-  constexpr int U = kTileTokens;
+static void launch_variant(const DecodeParams& p, bool page_mode, bool emit, bool merge_kernel,
+                           dim3 grid, hipStream_t st) {
+  constexpr int U = kTileInstr;
   if (page_mode) {
     if (emit)
       hipLaunchKernelGGL((decode_attn_kernel<T, D, QPG, U, NW, true, true>), grid, dim3(NW * 64), 0,
@@ -463,10 +541,13 @@ static void launch_variant(const DecodeParams& p, bool page_mode, bool emit, dim
       hipLaunchKernelGGL((decode_attn_kernel<T, D, QPG, U, NW, false, false>), grid, dim3(NW * 64),
                          0, st, p);
   }
+  if (merge_kernel)
+    hipLaunchKernelGGL((merge_partials_kernel<T, D, QPG, 512>), dim3(grid.x, grid.z), dim3(512), 0,
+                       st, p);
 }
 
-// Instantiated shapes: one query head per lane group for head_dim 64/128/256 with 8 or 16
-// waves; 2, 4 or 8 query heads per lane group (shared KV rows under GQA) for head_dim 128 with
+// Instantiated shapes: one query head per head row for head_dim 64/128/256 with 8 or 16 waves;
+// 2, 4 or 8 query heads per head row (KV rows shared inside a GQA group) for head_dim 128 with
 // 8 waves.
 static bool shape_supported(int head_dim, int qpg, int nw) {
   if (qpg == 1) return (head_dim == 64 || head_dim == 128 || head_dim == 256) && (nw == 8 || nw == 16);
@@ -475,10 +556,10 @@ static bool shape_supported(int head_dim, int qpg, int nw) {
 
 template <typename T>
 static int launch_shape(const DecodeParams& p, int head_dim, int qpg, int nw, bool page_mode,
-                        bool emit, dim3 grid, hipStream_t st) {
+                        bool emit, bool merge_kernel, dim3 grid, hipStream_t st) {
 #define TD_CASE(D_, Q_, N_)                                                    \
   if (head_dim == D_ && qpg == Q_ && nw == N_) {                               \
-    launch_variant<T, D_, Q_, N_>(p, page_mode, emit, grid, st);               \
+    launch_variant<T, D_, Q_, N_>(p, page_mode, emit, merge_kernel, grid, st); \
     return TD_OK;                                                              \
   }
   TD_CASE(64, 1, 8)
@@ -496,16 +577,6 @@ static int launch_shape(const DecodeParams& p, int head_dim, int qpg, int nw, bo
               "shared KV row and %d waves (supported: head_dim 64/128/256 with per-head lists; "
               "head_dim 128 with shared lists and group size 2, 4 or 8)",
               head_dim, qpg, nw);
-}
-
-template <typename T>
-static int launch_merge(const DecodeParams& p, int head_dim, dim3 grid, hipStream_t st) {
-  switch (head_dim) {
-    case 64: hipLaunchKernelGGL((merge_partials_kernel<T, 64>), grid, dim3(16), 0, st, p); break;
-    case 128: hipLaunchKernelGGL((merge_partials_kernel<T, 128>), grid, dim3(32), 0, st, p); break;
-    case 256: hipLaunchKernelGGL((merge_partials_kernel<T, 256>), grid, dim3(64), 0, st, p); break;
-  }
-  return TD_OK;
 }
 
 static int64_t align256(int64_t x) { return (x + 255) & ~(int64_t)255; }
@@ -539,9 +610,7 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
              (long long)max_items);
 
   const int qpg = qpg_for(num_qo_heads, num_kv_heads, idx_rows);
-  const int hpw = 64 / (head_dim / 8);
   const int n_hrows = num_qo_heads / qpg;
-  const int head_groups = (n_hrows + hpw - 1) / hpw;
 
   int nw = plan->waves_per_block;
   if (nw == 0) nw = 8;
@@ -550,18 +619,23 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
                 "td_decode_make_plan: no kernel for head_dim %d, %d query heads per shared KV row, %d "
                 "waves per block",
                 head_dim, qpg, nw);
-  const int tile = nw * kTileTokens;  // tokens one pass of the workgroup covers
+  // tokens one pass of the workgroup covers: waves x instructions x rows per instruction
+  const int tile = nw * kTileInstr * (64 / (head_dim / 8));
 
-  // Aim at ~2 workgroups of 8 waves per compute unit, never less than one tile per workgroup,
-  // never more than 64 partials per head.
-  const int64_t target_blocks = (int64_t)num_cus() * 2 * 8 / nw;
-  int64_t splits = target_blocks / ((int64_t)head_groups * batch);
+  // Aim at ~2 workgroups per compute unit, never less than one pass per workgroup, never more
+  // than 64 partials per head.
+  const int64_t target_blocks = (int64_t)num_cus() * 2;
+  int64_t splits = target_blocks / ((int64_t)n_hrows * batch);
   if (splits < 1) splits = 1;
   if (splits > 64) splits = 64;
   int64_t chunk = max_items > 0 ? ceil_div64(max_items, splits) : tile;
   if (plan->chunk_tokens > 0) chunk = plan->chunk_tokens;
   chunk = ceil_div64(chunk, tile) * tile;
   int64_t max_splits = max_items > 0 ? ceil_div64(max_items, chunk) : 1;
+  if (max_splits > 64) {  // keep the merge bounded: widen the chunks
+    chunk = ceil_div64(ceil_div64(max_items, 64), tile) * tile;
+    max_splits = ceil_div64(max_items, chunk);
+  }
   if (max_splits < 1) max_splits = 1;
 
   plan->chunk_tokens = (int32_t)chunk;
@@ -569,9 +643,9 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
   plan->waves_per_block = nw;
   if (plan->fused_merge < 0) plan->fused_merge = 1;
   plan->fused_merge = plan->fused_merge ? 1 : 0;
-  TD_REQUIRE((int64_t)batch * head_groups * 4 <= kTicketBytes,
-             "td_decode_make_plan: batch %d x %d head groups exceeds the %lld ticket counters", batch,
-             head_groups, (long long)(kTicketBytes / 4));
+  TD_REQUIRE((int64_t)batch * n_hrows * 4 <= kTicketBytes,
+             "td_decode_make_plan: batch %d x %d head rows exceeds the %lld ticket counters", batch,
+             n_hrows, (long long)(kTicketBytes / 4));
   const int64_t n_part = (int64_t)batch * num_qo_heads * max_splits;
   plan->workspace_bytes = kTicketBytes + align256(n_part * head_dim * 4) + align256(n_part * 2 * 4);
   return TD_OK;
@@ -586,6 +660,10 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
   TD_REQUIRE(kv->data != nullptr, "td_decode_attn: kv->data is NULL");
   TD_REQUIRE(batch >= 1, "td_decode_attn: batch %d < 1", batch);
   const int Hkv = kv->num_kv_heads, D = kv->head_dim, P = kv->page_size;
+  if (D != 64 && D != 128 && D != 256)
+    return fail(TD_ERR_UNSUPPORTED,
+                "BatchDecodeWithPagedKVCache failed to dispatch: head_dim %d (supported: 64, 128, 256)",
+                D);
   TD_REQUIRE(Hkv >= 1 && num_qo_heads >= Hkv && num_qo_heads % Hkv == 0,
              "td_decode_attn: num_qo_heads %d must be a positive multiple of num_kv_heads %d",
              num_qo_heads, Hkv);
@@ -613,7 +691,7 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
              "td_decode_attn: last_page_idx %d outside the pool of %lld pages", list->last_page_idx,
              (long long)kv->max_pages);
   TD_REQUIRE(plan->chunk_tokens > 0 && plan->max_splits >= 1 && plan->waves_per_block > 0 &&
-                 plan->chunk_tokens % (plan->waves_per_block * kTileTokens) == 0,
+                 plan->chunk_tokens % (plan->waves_per_block * kTileInstr * (64 / (D / 8))) == 0,
              "td_decode_attn: plan not produced by td_decode_make_plan");
   // the planned split must cover every token the list can describe
   const int64_t max_items = (int64_t)list->n_list_host * (list->kind == TD_IDX_PAGES ? P : 1) +
@@ -630,17 +708,16 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
   }
 
   const int qpg = qpg_for(num_qo_heads, Hkv, list->idx_rows);
-  const int hpw = 64 / (D / 8);
   const int n_hrows = num_qo_heads / qpg;
-  const int head_groups = (n_hrows + hpw - 1) / hpw;
 
   const int64_t n_part = (int64_t)batch * num_qo_heads * plan->max_splits;
   const int64_t off_o = kTicketBytes;
   const int64_t off_ml = off_o + align256(n_part * D * 4);
   const int64_t need = off_ml + align256(n_part * 2 * 4);
-  TD_REQUIRE((int64_t)batch * head_groups * 4 <= kTicketBytes,
-             "td_decode_attn: batch %d x %d head groups exceeds the ticket counters", batch,
-             head_groups);
+  TD_REQUIRE((int64_t)batch * n_hrows * 4 <= kTicketBytes,
+             "td_decode_attn: batch %d x %d head rows exceeds the ticket counters", batch, n_hrows);
+  TD_REQUIRE(plan->max_splits <= 64, "td_decode_attn: plan has %d splits (limit 64)",
+             plan->max_splits);
   if (plan->max_splits > 1) {
     if (workspace == nullptr || workspace_bytes < need)
       return fail(TD_ERR_STATE,
@@ -696,21 +773,16 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
 
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const bool page_mode = list->kind == TD_IDX_PAGES;
-  dim3 grid(head_groups, plan->max_splits, batch);
+  dim3 grid(n_hrows, plan->max_splits, batch);
+  const bool merge_kernel = plan->max_splits > 1 && !plan->fused_merge;
   int rc;
   if (kv->dtype == TD_F16)
-    rc = launch_shape<F16>(p, D, qpg, plan->waves_per_block, page_mode, scores != nullptr, grid, st);
+    rc = launch_shape<F16>(p, D, qpg, plan->waves_per_block, page_mode, scores != nullptr,
+                           merge_kernel, grid, st);
   else
-    rc = launch_shape<BF16>(p, D, qpg, plan->waves_per_block, page_mode, scores != nullptr, grid, st);
+    rc = launch_shape<BF16>(p, D, qpg, plan->waves_per_block, page_mode, scores != nullptr,
+                            merge_kernel, grid, st);
   if (rc != TD_OK) return rc;
   TD_HIP_CHECK(hipGetLastError());
-  if (plan->max_splits > 1 && !plan->fused_merge) {
-    dim3 mgrid(num_qo_heads, batch);
-    if (kv->dtype == TD_F16)
-      launch_merge<F16>(p, D, mgrid, st);
-    else
-      launch_merge<BF16>(p, D, mgrid, st);
-    TD_HIP_CHECK(hipGetLastError());
-  }
   return TD_OK;
 }
