@@ -102,7 +102,7 @@ typedef struct {
 typedef struct {
   int32_t chunk_tokens;    /* tokens per workgroup and head group */
   int32_t max_splits;      /* upper bound of partial results per head */
-  int32_t waves_per_block; /* 4, 8 or 16 */
+  int32_t waves_per_block; /* 8 or 16 */
   int32_t fused_merge;     /* 1: last workgroup merges in-kernel; 0: second kernel */
   int64_t workspace_bytes; /* device scratch the call needs (partials + tickets) */
 } td_decode_plan;
@@ -158,9 +158,12 @@ int td_rope_append_decode(const td_paged_kv* kv, void* q, const void* k, const v
 
 /*
  * Choose the split of a decode-attention call.  max_items is an upper bound of the tokens any
- * sequence attends to; idx_rows as in td_index_list.  waves_per_block / fused_merge may be
- * preset to non-zero / non-negative values in *plan to override the heuristics (pass a
- * zero-initialised struct with fused_merge = -1 for defaults).
+ * sequence attends to; idx_rows as in td_index_list.  chunk_tokens / waves_per_block (non-zero)
+ * and fused_merge (non-negative) may be preset in *plan to override the heuristics; pass a
+ * zero-initialised struct with fused_merge = -1 for defaults.  Host arithmetic only.
+ * Replaces BatchDecodeWithPagedKVCacheWorkEstimation and PartitionPagedKVCacheComputeAuxiliaryInfo
+ * (kernels/include/decode/decode_attn.cuh:815-906, :687-748), reached through
+ * BatchDecodeHandler::BeginForward (decode_handler.cuh:39-121, binding approx_attn.cu:27-62).
  */
 int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t num_kv_heads, int32_t head_dim,
                    int32_t idx_rows, int64_t max_items, td_decode_plan* plan);

@@ -8,7 +8,8 @@ import os
 from ctypes import POINTER, Structure, c_char_p, c_float, c_int32, c_int64, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libtidal_hip.so")
+# TIDAL_HIP_LIB selects another build of the same ABI (kernel experiments); default: in-tree build
+LIB_PATH = os.environ.get("TIDAL_HIP_LIB") or os.path.join(_HERE, "libtidal_hip.so")
 
 TD_OK, TD_ERR_INVALID_ARG, TD_ERR_UNSUPPORTED, TD_ERR_STATE, TD_ERR_HIP = range(5)
 TD_F16, TD_BF16, TD_F32 = 0, 1, 2

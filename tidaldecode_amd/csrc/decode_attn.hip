@@ -303,13 +303,17 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
     }
   };
   auto issue = [&](int base, const int32_t(&raw)[U], u32x4(&kb)[U], u32x4(&vb)[U]) {
+    int64_t offs[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int i = base + u * TPI + g;
       const int64_t off = item_offset<PAGE_MODE>(p, s, i < c1 ? i : s.n_items, raw[u], kv_head_off);
+      offs[u] = off;
       kb[u] = *reinterpret_cast<const u32x4*>(kv16 + off);
-      vb[u] = *reinterpret_cast<const u32x4*>(kv16 + off + p.v_offset);
     }
+    // V after all K: the q.k arithmetic of a tile starts while its V rows are still in flight
+#pragma unroll
+    for (int u = 0; u < U; ++u) vb[u] = *reinterpret_cast<const u32x4*>(kv16 + offs[u] + p.v_offset);
   };
   auto reduce = [&](const u32x4(&kb)[U], const u32x4(&vb)[U], int base) {
     float sc[QPG][U];
@@ -515,10 +519,20 @@ static int num_cus() {
 
 constexpr int kTileInstr = 4;  // U: K/V load instructions per wave tile and stream
 
-static int qpg_for(int num_qo_heads, int num_kv_heads, int idx_rows) {
-  // KV rows are shared between the query heads of a group only when the group shares its list
+// Instantiated shapes: one query head per head row for head_dim 64/128/256 with 8 or 16 waves;
+// 2, 4 or 8 query heads per head row (KV rows shared inside a GQA group) for head_dim 128 with
+// 8 waves.
+static bool shape_supported(int head_dim, int qpg, int nw) {
+  if (qpg == 1) return (head_dim == 64 || head_dim == 128 || head_dim == 256) && (nw == 8 || nw == 16);
+  return head_dim == 128 && (qpg == 2 || qpg == 4 || qpg == 8) && nw == 8;
+}
+
+// Query heads scored per loaded KV row.  KV rows are shared between the query heads of a GQA
+// group only when the group shares its list and a kernel for that shape exists; otherwise every
+// query head walks the list on its own (same result, the KV rows are read once per query head).
+static int qpg_for(int num_qo_heads, int num_kv_heads, int idx_rows, int head_dim) {
   const int group = num_qo_heads / num_kv_heads;
-  if (group > 1 && idx_rows != num_qo_heads) return group;
+  if (group > 1 && idx_rows != num_qo_heads && shape_supported(head_dim, group, 8)) return group;
   return 1;
 }
 
@@ -544,14 +558,6 @@ static void launch_variant(const DecodeParams& p, bool page_mode, bool emit, boo
   if (merge_kernel)
     hipLaunchKernelGGL((merge_partials_kernel<T, D, QPG, 512>), dim3(grid.x, grid.z), dim3(512), 0,
                        st, p);
-}
-
-// Instantiated shapes: one query head per head row for head_dim 64/128/256 with 8 or 16 waves;
-// 2, 4 or 8 query heads per head row (KV rows shared inside a GQA group) for head_dim 128 with
-// 8 waves.
-static bool shape_supported(int head_dim, int qpg, int nw) {
-  if (qpg == 1) return (head_dim == 64 || head_dim == 128 || head_dim == 256) && (nw == 8 || nw == 16);
-  return head_dim == 128 && (qpg == 2 || qpg == 4 || qpg == 8) && nw == 8;
 }
 
 template <typename T>
@@ -609,11 +615,12 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
   TD_REQUIRE(max_items >= 0 && max_items < ((int64_t)1 << 30), "td_decode_make_plan: max_items %lld",
              (long long)max_items);
 
-  const int qpg = qpg_for(num_qo_heads, num_kv_heads, idx_rows);
+  const int qpg = qpg_for(num_qo_heads, num_kv_heads, idx_rows, head_dim);
   const int n_hrows = num_qo_heads / qpg;
 
   int nw = plan->waves_per_block;
   if (nw == 0) nw = 8;
+  if (qpg > 1) nw = 8;  // the shared-row kernels exist for 8 waves only
   if (!shape_supported(head_dim, qpg, nw))
     return fail(TD_ERR_UNSUPPORTED,
                 "td_decode_make_plan: no kernel for head_dim %d, %d query heads per shared KV row, %d "
@@ -707,7 +714,7 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
     TD_REQUIRE(score_stride > 0, "td_decode_attn: score_stride %lld", (long long)score_stride);
   }
 
-  const int qpg = qpg_for(num_qo_heads, Hkv, list->idx_rows);
+  const int qpg = qpg_for(num_qo_heads, Hkv, list->idx_rows, D);
   const int n_hrows = num_qo_heads / qpg;
 
   const int64_t n_part = (int64_t)batch * num_qo_heads * plan->max_splits;

@@ -46,14 +46,15 @@ __device__ __forceinline__ int64_t k_offset(const PoolGeom& g, uint32_t page, in
          (int64_t)head * g.head_stride;
 }
 
-// sin / cos of position * theta^(-2j/D) / scale
+// sin / cos of position * theta^(-2j/D) / scale.  The angle is formed and reduced to a fraction
+// of a turn in double precision (exact to ~1e-10 rad at positions of 1e6); only the reduced
+// argument, |x| <= 1, goes through the fp32 sincospi.
 __device__ __forceinline__ void rope_sincos(double pos_over_scale, double log2_theta, int j, int D,
                                             float& sn, float& cs) {
   const double inv_freq = exp2(-log2_theta * (double)(2 * j) / (double)D);
-  double s, c;
-  sincos(pos_over_scale * inv_freq, &s, &c);
-  sn = (float)s;
-  cs = (float)c;
+  double turns = pos_over_scale * inv_freq * 0.15915494309189535;  // / (2 pi)
+  turns -= rint(turns);                                            // [-0.5, 0.5]
+  sincospif((float)(2.0 * turns), &sn, &cs);
 }
 
 template <typename T>
