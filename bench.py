@@ -24,6 +24,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+# HBM bytes one sparse-layer launch of the default workload moves, from rocprofv3 FETCH_SIZE /
+# WRITE_SIZE scaled by a plain 256 MiB copy (profiles/decode_attn_sparse_llama2-7b_ctx32k_top2048.md)
+TRAFFIC_DEFAULT_WORKLOAD = 35372816
 
 
 def parse():
@@ -42,6 +45,9 @@ def parse():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of hipGraph")
     ap.add_argument("--only-sparse", action="store_true",
                     help="profile helper: run only the sparse-layer launches")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="profile helper: also run 10 plain elementwise copies of 256 MiB "
+                         "(reads 256 MiB, writes 256 MiB) to scale rocprofv3 byte counters")
     return ap.parse_args()
 
 
@@ -203,6 +209,13 @@ def main():
         sys.exit(1)
 
     use_graph = not args.no_graph
+    if args.calibrate_copy:
+        src = torch.ones(64 << 20, dtype=torch.float32, device="cuda:0")  # 256 MiB
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            torch.add(src, 0.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
     results = {}
     for mode in ([args.select_mode] if args.only_sparse else
                  [args.select_mode] + [m for m in ("per_head", "head_sum") if m != args.select_mode]):
@@ -290,7 +303,9 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(e["achieved_gbs"] / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": (TRAFFIC_DEFAULT_WORKLOAD
+                        if (args.ctx, args.top_k, args.layers, main_mode) == (32768, 2048, 32, "per_head")
+                        else None),
             "kernel": "decode_attn_kernel (sparse layer, token-slot lists)",
             "algorithmic_bytes_per_launch": e["algorithmic_bytes"],
         },
