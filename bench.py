@@ -41,10 +41,15 @@ def parse():
     ap.add_argument("--waves", type=int, default=0, help="waves per workgroup (0 = default)")
     ap.add_argument("--chunk", type=int, default=0, help="tokens per workgroup (0 = default)")
     ap.add_argument("--merge", type=int, default=-1, help="1 fused / 0 second kernel / -1 default")
+    ap.add_argument("--rows", type=int, default=0, help="K/V loads per wave tile: 2 / 4 (0 = default)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of hipGraph")
     ap.add_argument("--only-sparse", action="store_true",
                     help="profile helper: run only the sparse-layer launches")
+    ap.add_argument("--no-e2e", action="store_true",
+                    help="skip the end-to-end decoder leg (Llama-2-7B shape, random weights)")
+    ap.add_argument("--e2e-ctx", type=str, default="32768,102400",
+                    help="context lengths of the end-to-end leg")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="profile helper: also run 10 plain elementwise copies of 256 MiB "
                          "(reads 256 MiB, writes 256 MiB) to scale rocprofv3 byte counters")
@@ -69,6 +74,7 @@ class Workload:
                                 self.dev, select_mode=select_mode, page_order_seed=0)
         h = c._decode_handler._wrapper
         h.waves_per_block, h.chunk_tokens, h.fused_merge = args.waves, args.chunk, args.merge
+        h.tile_rows = args.rows
         c.kv_cache.pool.buf.normal_()      # synthetic prefilled cache, resident in HBM
         c.prepare_metadata(self.N)         # the prompt
         c.prepare_metadata(1)              # the token being decoded
@@ -97,6 +103,12 @@ class Workload:
 
         return ops.decode_sparse_attn(self.q[layer], self.c, layer,
                                       self.c.kv_indices_without_last, True)
+
+    def full_attn(self, layer):
+        from tidaldecode_amd import utils as ops
+
+        return ops.decode_sparse_attn(self.q[layer], self.c, layer,
+                                      self.c.kv_indices_without_last, False)
 
     def topk(self):
         from tidaldecode_amd import utils as ops
@@ -196,6 +208,40 @@ def cpu_baseline(args, budget_s=20.0):
     }
 
 
+def e2e_leg(args):
+    """End-to-end decode of a Llama-2-7B-shape decoder with random bf16 weights (torch GEMMs and
+    norms around the library's attention path), TidalDecode schedule vs. the same decoder with
+    full attention in every layer, at each context length.  One decode step at that context is
+    captured as a hipGraph and replayed (steady-state per-token latency; the cache holds
+    synthetic N(0,1) data)."""
+    import torch
+
+    from tidaldecode_amd.llama import TidalLlama, TidalLlamaConfig
+
+    ctxs = [int(x) for x in args.e2e_ctx.split(",") if x]
+    cfg = TidalLlamaConfig.llama2_7b(top_k=args.top_k, sparse_layer_start=0, correction_layer=2,
+                                     select_mode=args.select_mode)
+    model = TidalLlama(cfg, "cuda:0", seed=0)
+    model.tidal_init(page_size=16, max_seq_len=max(ctxs) + 64, page_order_seed=0)
+    out = {}
+    for ctx in ctxs:
+        row = {}
+        for kind in ("tidal", "full"):
+            cfg.attn_type = kind
+            model.tidal_clear()
+            model.synthetic_prefill(ctx)
+            dt, how = model.timed_decode(steps=max(10, args.steps // 2), warmup=3,
+                                         use_graph=not args.no_graph)
+            row[f"{kind}_ms_per_token"] = round(dt * 1e3, 4)
+            row[f"{kind}_tokens_per_s"] = round(1.0 / dt, 2)
+            row["launch"] = how
+        row["speedup_vs_full_attention"] = round(row["full_ms_per_token"] / row["tidal_ms_per_token"], 3)
+        out[str(ctx)] = row
+    del model
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -261,6 +307,17 @@ def main():
                 r_step()
             torch.cuda.synchronize()
             entry["ms_per_step"] = (time.perf_counter() - t0) * 1e3 / args.steps
+
+            # the same step with full attention in every layer (no selection): attention-only
+            # latency ratio, the quantity the reference plots (README, llama_latency_eval.png)
+            def full_step():
+                for layer in range(w.L):
+                    w.rope_append(layer)
+                    w.full_attn(layer)
+
+            r_full, _ = capture(torch, full_step, use_graph)
+            entry["full_attention_ms_per_step"] = time_events(torch, r_full, 5, warm=1)
+            entry["attention_ratio_vs_full"] = entry["ms_per_step"] / entry["full_attention_ms_per_step"]
         rows = w.c.index_rows
         algo = (w.K * w.H * w.D * 2 * 2      # K and V rows of the attended tokens
                 + w.K * rows * 4             # the token list(s)
@@ -314,6 +371,8 @@ def main():
     }
     if "ms_per_step" in e:
         line["attention_path_tokens_per_s"] = round(1e3 / e["ms_per_step"], 1)
+    if not args.no_e2e and not args.only_sparse:
+        line["e2e_decode_llama2_7b_shape"] = e2e_leg(args)
     if not args.no_cpu and not args.only_sparse:
         line["cpu_baseline"] = cpu_baseline(args)
     print(json.dumps(line))

@@ -103,6 +103,7 @@ typedef struct {
   int32_t chunk_tokens;    /* tokens per workgroup and head group */
   int32_t max_splits;      /* upper bound of partial results per head */
   int32_t waves_per_block; /* 8 or 16 */
+  int32_t tile_rows;       /* K/V load instructions per wave tile: 2 or 4 */
   int32_t fused_merge;     /* 1: last workgroup merges in-kernel; 0: second kernel */
   int64_t workspace_bytes; /* device scratch the call needs (partials + tickets) */
 } td_decode_plan;
@@ -158,7 +159,7 @@ int td_rope_append_decode(const td_paged_kv* kv, void* q, const void* k, const v
 
 /*
  * Choose the split of a decode-attention call.  max_items is an upper bound of the tokens any
- * sequence attends to; idx_rows as in td_index_list.  chunk_tokens / waves_per_block (non-zero)
+ * sequence attends to; idx_rows as in td_index_list.  chunk_tokens / waves_per_block / tile_rows (non-zero)
  * and fused_merge (non-negative) may be preset in *plan to override the heuristics; pass a
  * zero-initialised struct with fused_merge = -1 for defaults.  Host arithmetic only.
  * Replaces BatchDecodeWithPagedKVCacheWorkEstimation and PartitionPagedKVCacheComputeAuxiliaryInfo

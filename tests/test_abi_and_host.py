@@ -41,7 +41,8 @@ def test_every_declaration_cites_the_reference():
 def _plan(batch, hq, hkv, d, rows, items, **preset):
     from tidaldecode_amd._lib import DecodePlan, lib
 
-    p = DecodePlan(preset.get("chunk", 0), 0, preset.get("waves", 0), preset.get("merge", -1), 0)
+    p = DecodePlan(preset.get("chunk", 0), 0, preset.get("waves", 0), preset.get("rows", 0),
+                   preset.get("merge", -1), 0)
     rc = lib.td_decode_make_plan(batch, hq, hkv, d, rows, items, p)
     return rc, p
 
@@ -53,7 +54,8 @@ def _plan(batch, hq, hkv, d, rows, items, **preset):
 def test_plan_covers_the_list(hq, hkv, d, rows, items):
     rc, p = _plan(1, hq, hkv, d, rows, items)
     assert rc == 0
-    tile = p.waves_per_block * 4 * (64 // (d // 8))
+    assert p.tile_rows in (2, 4)
+    tile = p.waves_per_block * p.tile_rows * (64 // (d // 8))
     assert p.chunk_tokens % tile == 0 and p.chunk_tokens > 0
     assert 1 <= p.max_splits <= 64
     assert p.chunk_tokens * p.max_splits >= items

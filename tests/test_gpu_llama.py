@@ -1,0 +1,156 @@
+"""GPU: the decoder harness (tidaldecode_amd/llama.py) against a plain fp32 torch restatement of the
+same Llama forward pass with the same weights.
+
+With top_k >= context every sparse layer attends to every token, so the TidalDecode model must
+reproduce dense attention (the reference's k = N special case); tolerance is that of bf16 GEMMs
+against fp32 (relative 3e-2 of the logit scale).  With a small budget the persisted lists must be
+the ones the last selection layer wrote, and the logits must equal a dense-mask evaluation
+(src/tidal_build/modify_llama.py:121-133) that uses those lists.
+"""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _small(**kw):
+    from tidaldecode_amd.llama import TidalLlamaConfig
+
+    base = dict(num_layers=5, hidden_size=256, num_heads=4, num_kv_heads=2, head_dim=64,
+                intermediate_size=512, vocab_size=1000, rope_theta=1e4, top_k=4096,
+                sparse_layer_start=1, correction_layer=3)
+    base.update(kw)
+    return TidalLlamaConfig(**base)
+
+
+def _rope(x, pos, theta):
+    d = x.shape[-1]
+    inv = 1.0 / (theta ** (torch.arange(0, d, 2, device=x.device, dtype=torch.float64) / d))
+    ang = pos.double()[:, None] * inv[None]
+    cos, sin = torch.cat([ang.cos(), ang.cos()], -1)[:, None], torch.cat([ang.sin(), ang.sin()], -1)[:, None]
+    x = x.double()
+    rot = torch.cat([-x[..., d // 2:], x[..., : d // 2]], -1)
+    return (x * cos + rot * sin).float()
+
+
+def _reference_logits(model, ids, masks=None):
+    """fp32 forward of the whole sequence; returns logits of the last position and per-layer
+    (q_last, k, v).  masks: optional {layer: [H, N] 0/1} applied to the last position's attention."""
+    c = model.config
+    f = lambda t: t.float()
+    n = ids.numel()
+    pos = torch.arange(n, device=ids.device)
+    x = f(model.embed)[ids]
+    rms = lambda t, w: t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + c.rms_norm_eps) * f(w)
+    for idx, layer in enumerate(model.layers):
+        h = rms(x, layer["ln1"])
+        qkv = h @ f(layer["wqkv"]).t()
+        qe, ke = c.num_heads * c.head_dim, (c.num_heads + c.num_kv_heads) * c.head_dim
+        q = _rope(qkv[:, :qe].reshape(n, c.num_heads, c.head_dim), pos, c.rope_theta)
+        k = _rope(qkv[:, qe:ke].reshape(n, c.num_kv_heads, c.head_dim), pos, c.rope_theta)
+        v = qkv[:, ke:].reshape(n, c.num_kv_heads, c.head_dim)
+        g = c.num_heads // c.num_kv_heads
+        kk, vv = k.repeat_interleave(g, 1), v.repeat_interleave(g, 1)
+        logit = torch.einsum("qhd,khd->hqk", q, kk) / math.sqrt(c.head_dim)
+        causal = torch.ones(n, n, device=ids.device).tril().bool()
+        logit = logit.masked_fill(~causal, float("-inf"))
+        if masks is not None and idx in masks:
+            logit[:, -1] = logit[:, -1].masked_fill(masks[idx] == 0, torch.finfo(torch.float32).min)
+        o = torch.einsum("hqk,khd->qhd", logit.softmax(-1), vv).reshape(n, -1)
+        x = x + o @ f(layer["wo"]).t()
+        h2 = rms(x, layer["ln2"])
+        gu = h2 @ f(layer["w_gate_up"]).t()
+        x = x + (torch.nn.functional.silu(gu[:, : c.intermediate_size]) * gu[:, c.intermediate_size:]) @ f(layer["w_down"]).t()
+    return (rms(x[-1:], model.norm) @ f(model.lm_head).t())[0]
+
+
+def _close(got, want, rel=3e-2):
+    scale = want.abs().max().item()
+    return (got.float() - want).abs().max().item() <= rel * scale
+
+
+@pytest.mark.parametrize("select_mode", ["per_head", "head_sum"])
+def test_budget_covering_the_context_equals_dense_attention(cuda, select_mode):
+    from tidaldecode_amd.llama import TidalLlama
+
+    torch.manual_seed(0)
+    model = TidalLlama(_small(select_mode=select_mode), cuda, seed=1, init_std=0.05)
+    model.tidal_init(page_size=16, max_seq_len=256, page_order_seed=3)
+    ids = torch.randint(0, 1000, (70,), device=cuda)
+    logits = model.prefill(ids)
+    assert _close(logits, _reference_logits(model, ids))
+    seq = ids
+    for _ in range(5):  # greedy steps, each compared with a fresh dense forward
+        tok = logits.argmax().view(1)
+        seq = torch.cat([seq, tok])
+        logits = model.decode_step(tok)
+        assert _close(logits, _reference_logits(model, seq))
+    assert model.iController.kv_cache.seqlen == 75
+    assert len(model.iController.decode_latency) == 5 and len(model.iController.prefill_latency) == 1
+    model.tidal_clear()
+    assert model.iController.kv_cache.seqlen == 0
+
+
+def test_sparse_layers_use_the_persisted_lists(cuda):
+    """small budget: logits equal a dense evaluation masked with the lists the selection layers
+    wrote (layers 2 and 4 reuse the lists of layers 1 and 3)"""
+    from tidaldecode_amd.llama import TidalLlama
+    from tidaldecode_amd import utils as ops
+
+    cfg = _small(top_k=12)
+    model = TidalLlama(cfg, cuda, seed=2, init_std=0.05)
+    model.tidal_init(page_size=4, max_seq_len=128, page_order_seed=1)
+    ids = torch.randint(0, 1000, (60,), device=cuda)
+    logits = model.prefill(ids)
+    tok = logits.argmax().view(1)
+    seq = torch.cat([ids, tok])
+    # record the list after every selection layer
+    lists, orig = {}, ops.decode_topk
+
+    def spy(ctrl):
+        orig(ctrl)
+        lists[len(lists)] = ctrl.topk_dindices_buffer.clone()
+
+    import tidaldecode_amd.llama as mod
+    mod.tidal_utils.decode_topk = spy
+    try:
+        got = model.decode_step(tok)
+    finally:
+        mod.tidal_utils.decode_topk = orig
+    assert len(lists) == 2 and lists[0].shape == (4, 12)
+    ctrl = model.iController
+    table = ctrl.kv_cache.indices_device.long()
+    inv = torch.full((int(table.max()) + 1,), -1, device=cuda)
+    inv[table] = torch.arange(table.numel(), device=cuda)
+
+    def mask_of(slots):
+        pos = inv[slots.long() // 4] * 4 + slots.long() % 4
+        assert (pos >= 0).all() and (pos < 61).all()
+        return torch.zeros(4, 61, device=cuda).scatter_(1, pos, 1.0)
+
+    masks = {2: mask_of(lists[0]), 4: mask_of(lists[1])}
+    assert (masks[2].sum(1) == 12).all()
+    assert _close(got, _reference_logits(model, seq, masks))
+    # and the result is not what dense attention gives
+    assert not _close(got, _reference_logits(model, seq), rel=1e-3)
+
+
+def test_layer_schedule_and_full_mode(cuda):
+    from tidaldecode_amd.llama import TidalLlama, TidalLlamaConfig
+
+    c = TidalLlamaConfig(num_layers=6, sparse_layer_start=0, correction_layer=2)
+    assert [c.layer_kind(i) for i in range(6)] == ["select", "sparse", "select", "sparse", "sparse", "sparse"]
+    c = TidalLlamaConfig(num_layers=4, sparse_layer_start=2, correction_layer=13)
+    assert [c.layer_kind(i) for i in range(4)] == ["full", "full", "select", "sparse"]
+    cfg = _small(top_k=8, attn_type="full")
+    assert all(cfg.layer_kind(i) == "full" for i in range(5))
+    model = TidalLlama(cfg, cuda, seed=3, init_std=0.05)
+    model.tidal_init(page_size=16, max_seq_len=128)
+    ids = torch.randint(0, 1000, (40,), device=cuda)
+    logits = model.prefill(ids)
+    tok = logits.argmax().view(1)
+    assert _close(model.decode_step(tok), _reference_logits(model, torch.cat([ids, tok])))
+    dt, how = model.timed_decode(steps=3, warmup=1)
+    assert dt > 0 and how in ("hipGraph", "eager")

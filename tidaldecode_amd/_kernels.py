@@ -302,6 +302,7 @@ class BatchDecodeWithPagedKVCachePyTorchWrapper:
         self.waves_per_block = 0  # 0 = library default; tuning knob
         self.fused_merge = -1     # -1 = library default
         self.chunk_tokens = 0     # 0 = library default
+        self.tile_rows = 0        # 0 = library default
 
     def begin_forward(self, indptr: torch.Tensor, num_qo_heads: int, num_kv_heads: int,
                       head_dim: int, page_size: int, empty_data: torch.Tensor) -> None:
@@ -326,11 +327,12 @@ class BatchDecodeWithPagedKVCachePyTorchWrapper:
 
     def _plan(self, batch: int, idx_rows: int, max_items: int) -> DecodePlan:
         key = (batch, idx_rows, max_items, self.waves_per_block, self.fused_merge,
-               self.chunk_tokens)
+               self.chunk_tokens, self.tile_rows)
         plan = self._plans.get(key)
         if plan is None:
             hq, hkv, d, _, _ = self._geom
-            plan = DecodePlan(self.chunk_tokens, 0, self.waves_per_block, self.fused_merge, 0)
+            plan = DecodePlan(self.chunk_tokens, 0, self.waves_per_block, self.tile_rows,
+                              self.fused_merge, 0)
             check(lib.td_decode_make_plan(batch, hq, hkv, d, idx_rows, max_items, plan))
             self._plans[key] = plan
         return plan

@@ -56,6 +56,7 @@ class DecodePlan(Structure):
         ("chunk_tokens", c_int32),
         ("max_splits", c_int32),
         ("waves_per_block", c_int32),
+        ("tile_rows", c_int32),
         ("fused_merge", c_int32),
         ("workspace_bytes", c_int64),
     ]

@@ -1,507 +1,9 @@
-// Decode attention over a paged KV pool for gfx950 (MI355X): one new query token per sequence
-// attends to a listed subset of the cache (sparse layers), or to the whole cache while emitting
-// per-token logits (token-selection layers).
-//
-// Mapping.  A K or V row of one head is head_dim two-byte elements; LPR = head_dim/8 adjacent
-// lanes hold it, 16 bytes (one global_load_dwordx4) per lane, so a 64-wide wavefront carries
-// HPW = 64/LPR "head rows" at once and never reduces across more than one DPP row for
-// head_dim 128.  A workgroup owns one group of HPW head rows and one chunk of the token list;
-// its waves take interleaved tiles of U tokens, each wave keeping a private online-softmax
-// state in base 2.  Wave states are merged through LDS, workgroup results through a fp32
-// partial buffer that the last-arriving workgroup of a head group reduces (ticket counter), or
-// that a second small kernel reduces when the plan asks for it.
-//
-// With grouped-query attention and an index list shared by the query heads of a KV head
-// (QPG > 1) each lane group loads the KV row once and scores it against QPG query heads.
-//
-// Semantics follow kernels/include/decode/decode_attn.cuh:432-658 of the reference
-// (BatchDecodeWithPagedKVCacheKernel) including the forced last page
-// (decode_page.cuh:320-346) and the logits output (decode_attn.cuh:107-109).
-
-#include "common.cuh"
+// Host side of the decode-attention entry points: split planning and argument checks.  The
+// kernels live in decode_attn.cuh and are instantiated in decode_attn_{f16,bf16}.hip.
+#include "decode_attn.cuh"
 
 namespace tidal {
 
-struct DecodeParams {
-  const void* q;
-  void* o;
-  const void* kv;
-  int64_t page_stride;   // elements from page p to page p+1  (2 * P * H_kv * D)
-  int64_t v_offset;      // elements from a K row to its V row (P * H_kv * D)
-  int32_t entry_stride;  // elements between consecutive tokens of a page
-  int32_t head_stride;   // elements between consecutive KV heads of a token
-  int32_t page_size;
-  int32_t page_shift;  // log2(page_size) or -1
-  uint32_t max_slot;   // max_pages * page_size - 1
-  uint32_t max_page;   // max_pages - 1
-  int32_t page_mode;   // 1: list entries are pages, 0: token slots
-  int32_t num_qo_heads;
-  int32_t n_hrows;   // head rows: num_qo_heads (QPG == 1) or num_kv_heads (QPG > 1)
-  int32_t q_per_kv;  // query heads per KV head (used when QPG == 1)
-  // index list
-  const int32_t* idx;
-  int32_t idx_row_stride;  // 0 for a shared row
-  int32_t idx_per_kv;      // 1: rows are per KV head while QPG == 1
-  const int32_t* indptr;
-  int32_t n_list_host;
-  const int32_t* last_len_arr;
-  const int32_t* last_idx_arr;
-  int32_t last_len;
-  int32_t last_idx;
-  // split
-  int32_t chunk_tokens;
-  int32_t max_splits;
-  int32_t fused_merge;
-  float scale_log2;  // sm_scale * log2(e)
-  // outputs
-  void* scores;
-  int32_t scores_f32;
-  int64_t score_stride;
-  float* lse;
-  float* ws_o;      // [batch * H_q * max_splits, D]
-  float* ws_ml;     // [batch * H_q * max_splits, 2]
-  int32_t* ws_cnt;  // [batch * head rows] ticket counters
-};
-
-__device__ __forceinline__ void divmod_page(const DecodeParams& p, uint32_t x, uint32_t& page,
-                                            uint32_t& entry) {
-  if (p.page_shift >= 0) {
-    page = x >> p.page_shift;
-    entry = x & ((1u << p.page_shift) - 1u);
-  } else {
-    page = x / (uint32_t)p.page_size;
-    entry = x - page * (uint32_t)p.page_size;
-  }
-}
-
-// Per-sequence view of the token list.
-struct SeqList {
-  const int32_t* row;  // this lane group's index row, already offset to the sequence
-  int32_t n_list;      // listed entries (pages or slots)
-  int32_t n_items;     // tokens attended
-  int32_t last_len;
-  int32_t last_idx;
-};
-
-// Physical (page, entry) of item i as one packed word; items past the end map to slot 0, a valid
-// address whose contribution is masked out.  `raw` is what had to be fetched from the list.
-template <bool PAGE_MODE>
-__device__ __forceinline__ bool item_needs_load(const SeqList& s, const DecodeParams& p, int32_t i,
-                                                uint32_t& list_pos) {
-  if (i >= s.n_items) return false;
-  if constexpr (PAGE_MODE) {
-    uint32_t pg, e;
-    divmod_page(p, (uint32_t)i, pg, e);
-    list_pos = pg;
-    return (int32_t)pg < s.n_list;
-  } else {
-    list_pos = (uint32_t)i;
-    return i < s.n_list;
-  }
-}
-
-template <bool PAGE_MODE>
-__device__ __forceinline__ int64_t item_offset(const DecodeParams& p, const SeqList& s, int32_t i,
-                                               int32_t raw, int32_t kv_head_off) {
-  uint32_t page = 0, entry = 0;
-  if (i < s.n_items) {
-    if constexpr (PAGE_MODE) {
-      uint32_t pg, e;
-      divmod_page(p, (uint32_t)i, pg, e);
-      page = ((int32_t)pg < s.n_list) ? (uint32_t)raw : (uint32_t)s.last_idx;
-      entry = e;
-      page = page > p.max_page ? p.max_page : page;
-    } else {
-      uint32_t slot = (i < s.n_list) ? (uint32_t)raw
-                                     : (uint32_t)s.last_idx * (uint32_t)p.page_size +
-                                           (uint32_t)(i - s.n_list);
-      slot = slot > p.max_slot ? p.max_slot : slot;
-      divmod_page(p, slot, page, entry);
-    }
-  }
-  return (int64_t)page * p.page_stride + (int64_t)entry * p.entry_stride + kv_head_off;
-}
-
-// 8-byte device-coherent accesses for the split partials: they are written by one workgroup and
-// read by another that may sit on a different XCD (own L2), so they go to memory (sc1) instead
-// of relying on an L2-wide write-back fence.
-__device__ __forceinline__ void store_coherent(float* dst, float a, float b) {
-  const uint64_t v = (uint64_t)__builtin_bit_cast(uint32_t, a) |
-                     ((uint64_t)__builtin_bit_cast(uint32_t, b) << 32);
-  __hip_atomic_store(reinterpret_cast<uint64_t*>(dst), v, __ATOMIC_RELAXED,
-                     __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void load_coherent(const float* src, float& a, float& b) {
-  const uint64_t v = __hip_atomic_load(reinterpret_cast<const uint64_t*>(src), __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);
-  a = __builtin_bit_cast(float, (uint32_t)v);
-  b = __builtin_bit_cast(float, (uint32_t)(v >> 32));
-}
-
-// Reduce the n_splits partial results of the QPG query heads of one head row and write o (and
-// lse).  Runs in one workgroup of NT threads: NT / (QPG * D / 2) "slots" of threads each own a
-// float2 column and a subset of the splits; slots are combined through LDS.
-template <typename T, int D, int QPG, int NT>
-__device__ __forceinline__ void merge_splits(const DecodeParams& p, int b, int qh0, int n_splits) {
-  constexpr int COLS = QPG * D / 2;
-  constexpr int SLOTS = NT / COLS;
-  constexpr int PRE = 4;  // partial loads kept in flight per thread
-  static_assert(SLOTS >= 1, "workgroup too small for the merge");
-  __shared__ float mg_m[QPG][64], mg_l[QPG][64];
-  __shared__ float mg_part[SLOTS][COLS][2];
-  const int tid = threadIdx.x;
-  const int c = tid % COLS, slot = tid / COLS;
-  const int j = c / (D / 2), d2 = c % (D / 2);
-  const int64_t part0 = ((int64_t)b * p.num_qo_heads + qh0 + j) * p.max_splits;
-
-  float ml_m = kNegBig, ml_l = 0.f;
-  const bool has_ml = tid < n_splits * QPG;
-  if (has_ml) {
-    const int jj = tid / n_splits, ss = tid % n_splits;
-    load_coherent(p.ws_ml + (((int64_t)b * p.num_qo_heads + qh0 + jj) * p.max_splits + ss) * 2,
-                  ml_m, ml_l);
-  }
-  float pa[PRE], pb[PRE];
-#pragma unroll
-  for (int u = 0; u < PRE; ++u) {
-    const int sidx = slot + u * SLOTS;
-    pa[u] = pb[u] = 0.f;
-    if (slot < SLOTS && sidx < n_splits) load_coherent(p.ws_o + (part0 + sidx) * D + d2 * 2, pa[u], pb[u]);
-  }
-  if (has_ml) {
-    mg_m[tid / n_splits][tid % n_splits] = ml_m;
-    mg_l[tid / n_splits][tid % n_splits] = ml_l;
-  }
-  __syncthreads();
-  float M = kNegBig;
-  for (int sidx = 0; sidx < n_splits; ++sidx) M = fmaxf(M, mg_m[j][sidx]);
-  float ra = 0.f, rb = 0.f;
-  if (slot < SLOTS) {
-#pragma unroll
-    for (int u = 0; u < PRE; ++u) {
-      const int sidx = slot + u * SLOTS;
-      if (sidx < n_splits) {
-        const float f = fast_exp2(mg_m[j][sidx] - M);
-        ra = fmaf(pa[u], f, ra);
-        rb = fmaf(pb[u], f, rb);
-      }
-    }
-    for (int sidx = slot + PRE * SLOTS; sidx < n_splits; sidx += SLOTS) {
-      float xa, xb;
-      load_coherent(p.ws_o + (part0 + sidx) * D + d2 * 2, xa, xb);
-      const float f = fast_exp2(mg_m[j][sidx] - M);
-      ra = fmaf(xa, f, ra);
-      rb = fmaf(xb, f, rb);
-    }
-    mg_part[slot][c][0] = ra;
-    mg_part[slot][c][1] = rb;
-  }
-  __syncthreads();
-  if (tid < COLS) {
-    float L = 0.f;
-    for (int sidx = 0; sidx < n_splits; ++sidx)
-      L = fmaf(mg_l[j][sidx], fast_exp2(mg_m[j][sidx] - M), L);
-    float oa = 0.f, ob = 0.f;
-#pragma unroll
-    for (int sl = 0; sl < SLOTS; ++sl) {
-      oa += mg_part[sl][c][0];
-      ob += mg_part[sl][c][1];
-    }
-    const float inv = L > 0.f ? 1.f / L : 0.f;
-    const int qh = qh0 + j;
-    reinterpret_cast<uint32_t*>(p.o)[((int64_t)b * p.num_qo_heads + qh) * (D / 2) + d2] =
-        pack2<T>(oa * inv, ob * inv);
-    if (p.lse && d2 == 0)
-      p.lse[(int64_t)b * p.num_qo_heads + qh] = L > 0.f ? (M + fast_log2(L)) * kLn2 : -INFINITY;
-  }
-}
-
-__device__ __forceinline__ int seq_items(const DecodeParams& p, int b, SeqList& s, int& list_beg) {
-  list_beg = 0;
-  if (p.indptr) {
-    list_beg = p.indptr[b];
-    s.n_list = p.indptr[b + 1] - list_beg;
-  } else {
-    s.n_list = p.n_list_host;
-  }
-  s.n_list = s.n_list < 0 ? 0 : (s.n_list > p.n_list_host ? p.n_list_host : s.n_list);
-  s.last_len = p.last_len_arr ? p.last_len_arr[b] : p.last_len;
-  s.last_idx = p.last_idx_arr ? p.last_idx_arr[b] : p.last_idx;
-  s.n_items = (p.page_mode ? s.n_list * p.page_size : s.n_list) + s.last_len;
-  int n_splits = (s.n_items + p.chunk_tokens - 1) / p.chunk_tokens;
-  return n_splits < 1 ? 1 : n_splits;
-}
-
-template <typename T, int D, int QPG, int U, int NW, bool PAGE_MODE, bool EMIT>
-__global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams p) {
-  constexpr int LPR = D / 8;     // lanes per K/V row
-  constexpr int TPI = 64 / LPR;  // tokens one wave instruction covers
-  constexpr int TILE = U * TPI;  // tokens per wave tile
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int g = lane / LPR;   // lane group = token slot inside the instruction
-  const int li = lane % LPR;  // 16-byte column of the row
-  const int hrow = blockIdx.x;
-  const int split = blockIdx.y;
-  const int b = blockIdx.z;
-  const int kv_head = (QPG > 1) ? hrow : hrow / p.q_per_kv;
-  const int qh0 = hrow * QPG;  // first query head of this head row
-
-  SeqList s;
-  int list_beg;
-  const int n_splits = seq_items(p, b, s, list_beg);
-  if (split >= n_splits) return;  // uniform for the whole workgroup
-  const int idx_row = (QPG == 1 && p.idx_per_kv) ? kv_head : hrow;
-  s.row = p.idx + (int64_t)idx_row * p.idx_row_stride + list_beg;
-
-  const int c0 = split * p.chunk_tokens;
-  int c1 = c0 + p.chunk_tokens;
-  c1 = c1 > s.n_items ? s.n_items : c1;
-
-  // query: QPG heads x 8 elements per lane, kept packed in the KV dtype
-  uint32_t qp[QPG][4];
-  {
-    const u32x4* qptr =
-        reinterpret_cast<const u32x4*>(p.q) + ((int64_t)b * p.num_qo_heads + qh0) * LPR + li;
-#pragma unroll
-    for (int j = 0; j < QPG; ++j) {
-      const u32x4 v = qptr[j * LPR];
-      qp[j][0] = v.x;
-      qp[j][1] = v.y;
-      qp[j][2] = v.z;
-      qp[j][3] = v.w;
-    }
-  }
-
-  float m[QPG], l[QPG], acc[QPG][8];
-#pragma unroll
-  for (int j = 0; j < QPG; ++j) {
-    m[j] = kNegBig;
-    l[j] = 0.f;
-#pragma unroll
-    for (int d = 0; d < 8; ++d) acc[j][d] = 0.f;
-  }
-
-  const int kv_head_off = kv_head * p.head_stride + li * 8;
-  const uint16_t* kv16 = reinterpret_cast<const uint16_t*>(p.kv);
-
-  // ---- software pipeline over this wave's tiles ------------------------------------------------
-  // program order per iteration: list entries of tile t+2, K/V rows of tile t+1, arithmetic of
-  // tile t.  Waiting for older list entries never waits for younger K/V loads, so two tiles of
-  // K/V stay in flight per wave.
-  u32x4 kA[U], vA[U], kB[U], vB[U];
-  int32_t rawA[U], rawB[U];
-
-  auto fetch_list = [&](int base, int32_t(&raw)[U]) {
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int i = base + u * TPI + g;
-      uint32_t pos = 0;
-      raw[u] = 0;
-      if (i < c1 && item_needs_load<PAGE_MODE>(s, p, i, pos)) raw[u] = s.row[pos];
-    }
-  };
-  auto issue = [&](int base, const int32_t(&raw)[U], u32x4(&kb)[U], u32x4(&vb)[U]) {
-    int64_t offs[U];
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int i = base + u * TPI + g;
-      const int64_t off = item_offset<PAGE_MODE>(p, s, i < c1 ? i : s.n_items, raw[u], kv_head_off);
-      offs[u] = off;
-      kb[u] = *reinterpret_cast<const u32x4*>(kv16 + off);
-    }
-    // V after all K: the q.k arithmetic of a tile starts while its V rows are still in flight
-#pragma unroll
-    for (int u = 0; u < U; ++u) vb[u] = *reinterpret_cast<const u32x4*>(kv16 + offs[u] + p.v_offset);
-  };
-  auto reduce = [&](const u32x4(&kb)[U], const u32x4(&vb)[U], int base) {
-    float sc[QPG][U];
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int i = base + u * TPI + g;
-      const bool valid = i < c1;
-#pragma unroll
-      for (int j = 0; j < QPG; ++j) {
-        float a = dot2<T>(qp[j][0], kb[u].x, 0.f);
-        a = dot2<T>(qp[j][1], kb[u].y, a);
-        a = dot2<T>(qp[j][2], kb[u].z, a);
-        a = dot2<T>(qp[j][3], kb[u].w, a);
-        a = group_sum<LPR>(a) * p.scale_log2;
-        sc[j][u] = valid ? a : kNegBig;
-        if constexpr (EMIT) {
-          if (valid && li == 0) {
-            const int64_t at = ((int64_t)b * p.num_qo_heads + qh0 + j) * p.score_stride + i;
-            const float nat = a * kLn2;
-            if (p.scores_f32)
-              reinterpret_cast<float*>(p.scores)[at] = nat;
-            else
-              reinterpret_cast<uint16_t*>(p.scores)[at] = from_float<T>(nat);
-          }
-        }
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < QPG; ++j) {
-      float mt = sc[j][0];
-#pragma unroll
-      for (int u = 1; u < U; ++u) mt = fmaxf(mt, sc[j][u]);
-      const float m_new = fmaxf(m[j], mt);
-      const float alpha = fast_exp2(m[j] - m_new);
-      m[j] = m_new;
-      float pr[U];
-      float ps = 0.f;
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        pr[u] = (base + u * TPI + g < c1) ? fast_exp2(sc[j][u] - m_new) : 0.f;
-        ps += pr[u];
-      }
-      l[j] = l[j] * alpha + ps;
-#pragma unroll
-      for (int d = 0; d < 8; ++d) acc[j][d] *= alpha;
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        float v0, v1, v2, v3, v4, v5, v6, v7;
-        unpack2<T>(vb[u].x, v0, v1);
-        unpack2<T>(vb[u].y, v2, v3);
-        unpack2<T>(vb[u].z, v4, v5);
-        unpack2<T>(vb[u].w, v6, v7);
-        acc[j][0] = fmaf(pr[u], v0, acc[j][0]);
-        acc[j][1] = fmaf(pr[u], v1, acc[j][1]);
-        acc[j][2] = fmaf(pr[u], v2, acc[j][2]);
-        acc[j][3] = fmaf(pr[u], v3, acc[j][3]);
-        acc[j][4] = fmaf(pr[u], v4, acc[j][4]);
-        acc[j][5] = fmaf(pr[u], v5, acc[j][5]);
-        acc[j][6] = fmaf(pr[u], v6, acc[j][6]);
-        acc[j][7] = fmaf(pr[u], v7, acc[j][7]);
-      }
-    }
-  };
-
-  constexpr int STEP = NW * TILE;  // tokens between two tiles of one wave
-  int t = c0 + wave * TILE;        // first token of this wave's current tile
-  if (t < c1) {
-    fetch_list(t, rawA);
-    if (t + STEP < c1) fetch_list(t + STEP, rawB);
-    issue(t, rawA, kA, vA);
-    while (true) {
-      // A: K/V of tile t in flight; rawB: list entries of tile t+STEP in flight
-      const int tn = t + STEP;
-      const int tnn = tn + STEP;
-      if (tnn < c1) fetch_list(tnn, rawA);
-      if (tn < c1) issue(tn, rawB, kB, vB);
-      reduce(kA, vA, t);
-      if (tn >= c1) break;
-      const int tnnn = tnn + STEP;
-      if (tnnn < c1) fetch_list(tnnn, rawB);
-      if (tnn < c1) issue(tnn, rawA, kA, vA);
-      reduce(kB, vB, tn);
-      if (tnn >= c1) break;
-      t = tnn;
-    }
-  }
-
-  // ---- combine the TPI token slots of the wave (butterfly over lane groups) ---------------------
-#pragma unroll
-  for (int j = 0; j < QPG; ++j) {
-    float mw = m[j];
-#pragma unroll
-    for (int off = LPR; off < 64; off <<= 1) mw = fmaxf(mw, __shfl_xor(mw, off, 64));
-    const float f = fast_exp2(m[j] - mw);
-    m[j] = mw;
-    l[j] *= f;
-#pragma unroll
-    for (int d = 0; d < 8; ++d) acc[j][d] *= f;
-#pragma unroll
-    for (int off = LPR; off < 64; off <<= 1) {
-      l[j] += __shfl_xor(l[j], off, 64);
-#pragma unroll
-      for (int d = 0; d < 8; ++d) acc[j][d] += __shfl_xor(acc[j][d], off, 64);
-    }
-  }
-
-  // ---- merge the NW wave states of the workgroup through LDS ------------------------------------
-  __shared__ float sm_o[NW][8][LPR];
-  __shared__ float sm_ml[NW][2];
-  __shared__ int sm_ticket;
-#pragma unroll
-  for (int j = 0; j < QPG; ++j) {
-    if (j > 0) __syncthreads();
-    if (lane < LPR) {
-#pragma unroll
-      for (int d = 0; d < 8; ++d) sm_o[wave][d][lane] = acc[j][d];
-      if (lane == 0) {
-        sm_ml[wave][0] = m[j];
-        sm_ml[wave][1] = l[j];
-      }
-    }
-    __syncthreads();
-    if (wave == (j % NW) && lane < LPR) {
-      float M = kNegBig;
-#pragma unroll
-      for (int w = 0; w < NW; ++w) M = fmaxf(M, sm_ml[w][0]);
-      float L = 0.f, r[8];
-#pragma unroll
-      for (int d = 0; d < 8; ++d) r[d] = 0.f;
-#pragma unroll
-      for (int w = 0; w < NW; ++w) {
-        const float f = fast_exp2(sm_ml[w][0] - M);
-        L = fmaf(sm_ml[w][1], f, L);
-#pragma unroll
-        for (int d = 0; d < 8; ++d) r[d] = fmaf(sm_o[w][d][lane], f, r[d]);
-      }
-      const int qh = qh0 + j;
-      if (n_splits == 1) {
-        const float inv = L > 0.f ? 1.f / L : 0.f;
-        u32x4 out;
-        out.x = pack2<T>(r[0] * inv, r[1] * inv);
-        out.y = pack2<T>(r[2] * inv, r[3] * inv);
-        out.z = pack2<T>(r[4] * inv, r[5] * inv);
-        out.w = pack2<T>(r[6] * inv, r[7] * inv);
-        reinterpret_cast<u32x4*>(p.o)[((int64_t)b * p.num_qo_heads + qh) * LPR + lane] = out;
-        if (p.lse && lane == 0)
-          p.lse[(int64_t)b * p.num_qo_heads + qh] = L > 0.f ? (M + fast_log2(L)) * kLn2 : -INFINITY;
-      } else {
-        const int64_t part = ((int64_t)b * p.num_qo_heads + qh) * p.max_splits + split;
-        float* dst = p.ws_o + part * D + lane * 8;
-        store_coherent(dst + 0, r[0], r[1]);
-        store_coherent(dst + 2, r[2], r[3]);
-        store_coherent(dst + 4, r[4], r[5]);
-        store_coherent(dst + 6, r[6], r[7]);
-        if (lane == 0) store_coherent(p.ws_ml + part * 2, M, L);
-      }
-    }
-  }
-
-  if (n_splits == 1 || !p.fused_merge) return;
-
-  // ---- the last workgroup of this (sequence, head row) to arrive reduces the partials ----------
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // partial stores have left this CU
-  __syncthreads();
-  int32_t* ticket = p.ws_cnt + (int64_t)b * gridDim.x + hrow;
-  if (tid == 0)
-    sm_ticket = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __syncthreads();
-  if (sm_ticket != n_splits - 1) return;
-  merge_splits<T, D, QPG, NW * 64>(p, b, qh0, n_splits);
-  if (tid == 0) __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// Second-kernel merge (plan.fused_merge == 0): one workgroup per (head row, sequence).
-template <typename T, int D, int QPG, int NT>
-__global__ __launch_bounds__(NT) void merge_partials_kernel(const DecodeParams p) {
-  const int hrow = blockIdx.x;
-  const int b = blockIdx.y;
-  SeqList s;
-  int list_beg;
-  const int n_splits = seq_items(p, b, s, list_beg);
-  if (n_splits <= 1) return;  // the attention kernel already wrote the final result
-  merge_splits<T, D, QPG, NT>(p, b, hrow * QPG, n_splits);
-}
-
-// ---------------------------------------------------------------------------------------------
-// Host side
-// ---------------------------------------------------------------------------------------------
 static int g_num_cus = 0;
 
 static int num_cus() {
@@ -515,74 +17,6 @@ static int num_cus() {
       g_num_cus = 256;  // MI355X
   }
   return g_num_cus;
-}
-
-constexpr int kTileInstr = 4;  // U: K/V load instructions per wave tile and stream
-
-// Instantiated shapes: one query head per head row for head_dim 64/128/256 with 8 or 16 waves;
-// 2, 4 or 8 query heads per head row (KV rows shared inside a GQA group) for head_dim 128 with
-// 8 waves.
-static bool shape_supported(int head_dim, int qpg, int nw) {
-  if (qpg == 1) return (head_dim == 64 || head_dim == 128 || head_dim == 256) && (nw == 8 || nw == 16);
-  return head_dim == 128 && (qpg == 2 || qpg == 4 || qpg == 8) && nw == 8;
-}
-
-// Query heads scored per loaded KV row.  KV rows are shared between the query heads of a GQA
-// group only when the group shares its list and a kernel for that shape exists; otherwise every
-// query head walks the list on its own (same result, the KV rows are read once per query head).
-static int qpg_for(int num_qo_heads, int num_kv_heads, int idx_rows, int head_dim) {
-  const int group = num_qo_heads / num_kv_heads;
-  if (group > 1 && idx_rows != num_qo_heads && shape_supported(head_dim, group, 8)) return group;
-  return 1;
-}
-
-template <typename T, int D, int QPG, int NW>
-static void launch_variant(const DecodeParams& p, bool page_mode, bool emit, bool merge_kernel,
-                           dim3 grid, hipStream_t st) {
-  constexpr int U = kTileInstr;
-  if (page_mode) {
-    if (emit)
-      hipLaunchKernelGGL((decode_attn_kernel<T, D, QPG, U, NW, true, true>), grid, dim3(NW * 64), 0,
-                         st, p);
-    else
-      hipLaunchKernelGGL((decode_attn_kernel<T, D, QPG, U, NW, true, false>), grid, dim3(NW * 64),
-                         0, st, p);
-  } else {
-    if (emit)
-      hipLaunchKernelGGL((decode_attn_kernel<T, D, QPG, U, NW, false, true>), grid, dim3(NW * 64),
-                         0, st, p);
-    else
-      hipLaunchKernelGGL((decode_attn_kernel<T, D, QPG, U, NW, false, false>), grid, dim3(NW * 64),
-                         0, st, p);
-  }
-  if (merge_kernel)
-    hipLaunchKernelGGL((merge_partials_kernel<T, D, QPG, 512>), dim3(grid.x, grid.z), dim3(512), 0,
-                       st, p);
-}
-
-template <typename T>
-static int launch_shape(const DecodeParams& p, int head_dim, int qpg, int nw, bool page_mode,
-                        bool emit, bool merge_kernel, dim3 grid, hipStream_t st) {
-#define TD_CASE(D_, Q_, N_)                                                    \
-  if (head_dim == D_ && qpg == Q_ && nw == N_) {                               \
-    launch_variant<T, D_, Q_, N_>(p, page_mode, emit, merge_kernel, grid, st); \
-    return TD_OK;                                                              \
-  }
-  TD_CASE(64, 1, 8)
-  TD_CASE(64, 1, 16)
-  TD_CASE(128, 1, 8)
-  TD_CASE(128, 1, 16)
-  TD_CASE(256, 1, 8)
-  TD_CASE(256, 1, 16)
-  TD_CASE(128, 2, 8)
-  TD_CASE(128, 4, 8)
-  TD_CASE(128, 8, 8)
-#undef TD_CASE
-  return fail(TD_ERR_UNSUPPORTED,
-              "BatchDecodeWithPagedKVCache failed to dispatch: head_dim %d with %d query heads per "
-              "shared KV row and %d waves (supported: head_dim 64/128/256 with per-head lists; "
-              "head_dim 128 with shared lists and group size 2, 4 or 8)",
-              head_dim, qpg, nw);
 }
 
 static int64_t align256(int64_t x) { return (x + 255) & ~(int64_t)255; }
@@ -621,13 +55,17 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
   int nw = plan->waves_per_block;
   if (nw == 0) nw = 8;
   if (qpg > 1) nw = 8;  // the shared-row kernels exist for 8 waves only
-  if (!shape_supported(head_dim, qpg, nw))
+  // Short lists (sparse layers) are cut finer: 2 K/V rows per lane group and tile; long ones
+  // stream with 4.
+  int rows = plan->tile_rows;
+  if (rows == 0) rows = 4;
+  if (!shape_supported(head_dim, qpg, nw, rows))
     return fail(TD_ERR_UNSUPPORTED,
                 "td_decode_make_plan: no kernel for head_dim %d, %d query heads per shared KV row, %d "
-                "waves per block",
-                head_dim, qpg, nw);
+                "waves per block, %d rows per tile",
+                head_dim, qpg, nw, rows);
   // tokens one pass of the workgroup covers: waves x instructions x rows per instruction
-  const int tile = nw * kTileInstr * (64 / (head_dim / 8));
+  const int tile = nw * rows * (64 / (head_dim / 8));
 
   // Aim at ~2 workgroups per compute unit, never less than one pass per workgroup, never more
   // than 64 partials per head.
@@ -648,6 +86,7 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
   plan->chunk_tokens = (int32_t)chunk;
   plan->max_splits = (int32_t)max_splits;
   plan->waves_per_block = nw;
+  plan->tile_rows = rows;
   if (plan->fused_merge < 0) plan->fused_merge = 1;
   plan->fused_merge = plan->fused_merge ? 1 : 0;
   TD_REQUIRE((int64_t)batch * n_hrows * 4 <= kTicketBytes,
@@ -698,7 +137,8 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
              "td_decode_attn: last_page_idx %d outside the pool of %lld pages", list->last_page_idx,
              (long long)kv->max_pages);
   TD_REQUIRE(plan->chunk_tokens > 0 && plan->max_splits >= 1 && plan->waves_per_block > 0 &&
-                 plan->chunk_tokens % (plan->waves_per_block * kTileInstr * (64 / (D / 8))) == 0,
+                 plan->tile_rows > 0 &&
+                 plan->chunk_tokens % (plan->waves_per_block * plan->tile_rows * (64 / (D / 8))) == 0,
              "td_decode_attn: plan not produced by td_decode_make_plan");
   // the planned split must cover every token the list can describe
   const int64_t max_items = (int64_t)list->n_list_host * (list->kind == TD_IDX_PAGES ? P : 1) +
@@ -751,6 +191,9 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
   for (int sft = 0; sft < 31; ++sft)
     if ((1 << sft) == P) p.page_shift = sft;
   p.max_slot = (uint32_t)(kv->max_pages * P - 1);
+  p.page_stride_b = (uint32_t)(p.page_stride * 2);
+  p.entry_stride_b = (uint32_t)(p.entry_stride * 2);
+  p.lean = (p.page_shift >= 0 && (int64_t)kv->max_pages * p.page_stride * 2 < ((int64_t)1 << 32)) ? 1 : 0;
   p.num_qo_heads = num_qo_heads;
   p.n_hrows = n_hrows;
   p.q_per_kv = num_qo_heads / Hkv;
@@ -784,10 +227,10 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
   const bool merge_kernel = plan->max_splits > 1 && !plan->fused_merge;
   int rc;
   if (kv->dtype == TD_F16)
-    rc = launch_shape<F16>(p, D, qpg, plan->waves_per_block, page_mode, scores != nullptr,
+    rc = launch_decode_f16(p, D, qpg, plan->waves_per_block, plan->tile_rows, page_mode, scores != nullptr,
                            merge_kernel, grid, st);
   else
-    rc = launch_shape<BF16>(p, D, qpg, plan->waves_per_block, page_mode, scores != nullptr,
+    rc = launch_decode_bf16(p, D, qpg, plan->waves_per_block, plan->tile_rows, page_mode, scores != nullptr,
                             merge_kernel, grid, st);
   if (rc != TD_OK) return rc;
   TD_HIP_CHECK(hipGetLastError());

@@ -1,0 +1,251 @@
+"""Llama-style decoder whose attention runs through the TidalDecode operator surface
+(counterpart of the decode driver in the reference: tidal/models/llama.py:498-578 for the layer
+loop and budget handling, tidal/models/{Full,Search,Sparse}Attention.py:131-190 for the three
+attention flavours, scripts/bench_textgen.py:41-101 for the latency harness).
+
+Only what the decode-attention path needs is here: random-initialised weights of a given
+shape (there is no checkpoint loading), torch GEMMs and norms around the library's kernels, and
+the layer schedule of the PyTorch path of the reference (src/tidal_build/modify_llama.py:84,116):
+
+    layer <  sparse_layer_start                      full attention
+    layer == sparse_layer_start or correction_layer  full attention + token selection
+    otherwise                                         sparse attention over the persisted tokens
+"""
+import math
+import time
+from dataclasses import dataclass
+from typing import Optional, Tuple
+
+import torch
+
+from . import utils as tidal_utils
+from .utils import InferenceController
+
+
+@dataclass
+class TidalLlamaConfig:
+    num_layers: int = 32
+    hidden_size: int = 4096
+    num_heads: int = 32
+    num_kv_heads: int = 32
+    head_dim: int = 128
+    intermediate_size: int = 11008
+    vocab_size: int = 32000
+    rope_theta: float = 1e4
+    rope_scale: float = 1.0
+    rms_norm_eps: float = 1e-5
+    # TidalDecode
+    top_k: int = 256
+    sparse_layer_start: int = 2
+    correction_layer: int = 13
+    select_mode: str = "per_head"
+    attn_type: str = "tidal"  # "tidal" or "full" (every layer attends to the whole cache)
+    dtype: torch.dtype = torch.bfloat16
+
+    @staticmethod
+    def llama2_7b(**kw):
+        return TidalLlamaConfig(32, 4096, 32, 32, 128, 11008, 32000, 1e4, **kw)
+
+    @staticmethod
+    def llama3_8b(**kw):
+        return TidalLlamaConfig(32, 4096, 32, 8, 128, 14336, 128256, 5e5, **kw)
+
+    def layer_kind(self, layer: int) -> str:
+        if self.attn_type == "full" or layer < self.sparse_layer_start:
+            return "full"
+        if layer in (self.sparse_layer_start, self.correction_layer):
+            return "select"
+        return "sparse"
+
+
+class TidalLlama:
+    """Decoder with random weights.  ``tidal_init`` allocates the paged cache and controller,
+    ``prefill`` / ``synthetic_prefill`` fills it, ``decode_step`` produces next-token logits."""
+
+    def __init__(self, config: TidalLlamaConfig, device, seed: int = 0, init_std: float = 0.02):
+        self.config = c = config
+        self.device = torch.device(device)
+        g = torch.Generator(device=self.device).manual_seed(seed)
+
+        def w(*shape):
+            return (torch.randn(shape, generator=g, device=self.device) * init_std).to(c.dtype)
+
+        qkv_out = (c.num_heads + 2 * c.num_kv_heads) * c.head_dim
+        self.embed = w(c.vocab_size, c.hidden_size)
+        self.layers = []
+        for _ in range(c.num_layers):
+            self.layers.append(dict(
+                ln1=torch.ones(c.hidden_size, dtype=c.dtype, device=self.device),
+                wqkv=w(qkv_out, c.hidden_size),
+                wo=w(c.hidden_size, c.num_heads * c.head_dim),
+                ln2=torch.ones(c.hidden_size, dtype=c.dtype, device=self.device),
+                w_gate_up=w(2 * c.intermediate_size, c.hidden_size),
+                w_down=w(c.hidden_size, c.intermediate_size),
+            ))
+        self.norm = torch.ones(c.hidden_size, dtype=c.dtype, device=self.device)
+        self.lm_head = w(c.vocab_size, c.hidden_size)
+        self.iController: Optional[InferenceController] = None
+        self._positions = torch.zeros(1, dtype=torch.int32, device=self.device)
+        self._dst_slot = torch.zeros(1, dtype=torch.int32, device=self.device)
+
+    # ----- cache lifecycle (tidal/models/llama.py:616-656) -----------------------------------
+    def tidal_init(self, page_size: int, max_seq_len: int, token_budget: Optional[int] = None,
+                   page_order_seed=None):
+        c = self.config
+        self.iController = InferenceController(
+            c.num_layers, c.num_heads, c.head_dim, page_size,
+            c.top_k if token_budget is None else token_budget, max_seq_len, c.dtype, self.device,
+            num_kv_heads=c.num_kv_heads, select_mode=c.select_mode, select_scope="all",
+            page_order_seed=page_order_seed)
+
+    def tidal_clear(self):
+        self.iController.clean_states()
+
+    # ----- pieces -------------------------------------------------------------------------------
+    def _rms(self, x, weight):
+        return tidal_utils.rms_norm_forward(x, weight, self.config.rms_norm_eps)
+
+    def _mlp(self, layer, x):
+        c = self.config
+        gu = x @ layer["w_gate_up"].t()
+        gate, up = gu[..., : c.intermediate_size], gu[..., c.intermediate_size:]
+        return (torch.nn.functional.silu(gate) * up) @ layer["w_down"].t()
+
+    def _qkv(self, layer, h):
+        c = self.config
+        qkv = h @ layer["wqkv"].t()
+        n = qkv.shape[0]
+        q_end = c.num_heads * c.head_dim
+        k_end = q_end + c.num_kv_heads * c.head_dim
+        q = qkv[:, :q_end].reshape(n, c.num_heads, c.head_dim).contiguous()
+        k = qkv[:, q_end:k_end].reshape(n, c.num_kv_heads, c.head_dim).contiguous()
+        v = qkv[:, k_end:].reshape(n, c.num_kv_heads, c.head_dim).contiguous()
+        return q, k, v
+
+    # ----- prefill ----------------------------------------------------------------------------
+    @torch.no_grad()
+    def prefill(self, input_ids: torch.Tensor) -> torch.Tensor:
+        """Run the prompt [N] through all layers (full causal attention), fill the cache, return
+        the logits of the last position."""
+        c, ctrl = self.config, self.iController
+        n = input_ids.numel()
+        past = ctrl.kv_cache.seqlen
+        t0 = time.perf_counter()
+        ctrl.prepare_metadata(n)
+        ctrl.begin_forward(n)
+        x = self.embed[input_ids.to(self.device)]
+        for idx, layer in enumerate(self.layers):
+            h = self._rms(x, layer["ln1"])
+            q, k, v = self._qkv(layer, h)
+            tidal_utils.apply_rope_in_place(q, k, past, c.rope_scale, c.rope_theta)
+            tidal_utils.append_kv(k, v, ctrl, idx)
+            o = tidal_utils.prefill_forward(q, ctrl, idx)
+            x = x + o.reshape(n, -1) @ layer["wo"].t()
+            x = x + self._mlp(layer, self._rms(x, layer["ln2"]))
+        ctrl.end_forward()
+        logits = self._rms(x[-1:], self.norm) @ self.lm_head.t()
+        torch.cuda.synchronize()
+        ctrl.prefill_latency.append(time.perf_counter() - t0)
+        return logits[0]
+
+    @torch.no_grad()
+    def synthetic_prefill(self, n: int):
+        """Latency-only stand-in for a prompt of n tokens: the cache is filled with N(0,1) data
+        (what the reference's harness gets from random input embeddings)."""
+        ctrl = self.iController
+        ctrl.kv_cache.pool.buf.normal_()
+        ctrl.prepare_metadata(n)
+
+    # ----- decode -----------------------------------------------------------------------------
+    @torch.no_grad()
+    def begin_decode_step(self):
+        """Host bookkeeping of one decode step: reserve the slot of the new token and publish its
+        position / physical slot to the device."""
+        ctrl = self.iController
+        ctrl.prepare_metadata(1)
+        ctrl.begin_forward(1)
+        pos = ctrl.kv_cache.seqlen - 1
+        page = ctrl.kv_cache.indicies[pos // ctrl.page_size]
+        self._positions.fill_(pos)
+        self._dst_slot.fill_(page * ctrl.page_size + pos % ctrl.page_size)
+
+    @torch.no_grad()
+    def decode_layers(self, x: torch.Tensor) -> torch.Tensor:
+        """The layer loop of one decode step on hidden state x [1, hidden]; device work only (safe
+        to capture in a hipGraph once begin_decode_step has run)."""
+        c, ctrl = self.config, self.iController
+        for idx, layer in enumerate(self.layers):
+            h = self._rms(x, layer["ln1"])
+            q, k, v = self._qkv(layer, h)
+            tidal_utils.rope_append_kv(q, k, v, ctrl, idx, self._positions, self._dst_slot,
+                                       c.rope_scale, c.rope_theta)
+            kind = c.layer_kind(idx)
+            if kind == "sparse":
+                o = tidal_utils.decode_sparse_attn(q, ctrl, idx, ctrl.topk_dindices_buffer, False)
+            else:
+                o = tidal_utils.decode_sparse_attn(q, ctrl, idx, ctrl.kv_indices_without_last,
+                                                   kind == "select")
+                if kind == "select":
+                    tidal_utils.decode_topk(ctrl)
+            x = x + o.reshape(1, -1) @ layer["wo"].t()
+            x = x + self._mlp(layer, self._rms(x, layer["ln2"]))
+        return self._rms(x, self.norm) @ self.lm_head.t()
+
+    @torch.no_grad()
+    def decode_step(self, token: torch.Tensor) -> torch.Tensor:
+        """One eager decode step for token id(s) [1]; returns logits [vocab]."""
+        ctrl = self.iController
+        t0 = time.perf_counter()
+        self.begin_decode_step()
+        logits = self.decode_layers(self.embed[token.to(self.device).view(1)])
+        ctrl.end_forward()
+        torch.cuda.synchronize()
+        ctrl.decode_latency.append(time.perf_counter() - t0)
+        return logits[0]
+
+    @torch.no_grad()
+    def generate(self, input_ids: torch.Tensor, max_new_tokens: int) -> torch.Tensor:
+        """Greedy decoding (prefill + max_new_tokens steps)."""
+        logits = self.prefill(input_ids)
+        out = []
+        for _ in range(max_new_tokens):
+            tok = logits.argmax().view(1)
+            out.append(tok)
+            logits = self.decode_step(tok)
+        return torch.cat(out)
+
+    @torch.no_grad()
+    def timed_decode(self, steps: int, warmup: int = 3, use_graph: bool = True) -> Tuple[float, str]:
+        """Steady-state latency of a decode step at the current context length: the step that
+        appends token number seqlen is captured once (hipGraph) and replayed; returns
+        (seconds per step, "hipGraph" | "eager")."""
+        ctrl = self.iController
+        self.begin_decode_step()
+        x = self.embed[:1].clone()
+        run, how = (lambda: self.decode_layers(x)), "eager"
+        if use_graph:
+            try:
+                s = torch.cuda.Stream()
+                s.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(s):
+                    self.decode_layers(x)
+                torch.cuda.current_stream().wait_stream(s)
+                torch.cuda.synchronize()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    self.decode_layers(x)
+                run, how = g.replay, "hipGraph"
+            except Exception as e:  # pragma: no cover - runtime dependent
+                print(f"[tidal] graph capture failed ({e}); timing eager launches")
+                torch.cuda.synchronize()
+        for _ in range(warmup):
+            run()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            run()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / steps
+        ctrl.end_forward()
+        ctrl.decode_latency.append(dt)
+        return dt, how
