@@ -42,6 +42,7 @@ def parse():
     ap.add_argument("--chunk", type=int, default=0, help="tokens per workgroup (0 = default)")
     ap.add_argument("--merge", type=int, default=-1, help="1 fused / 0 second kernel / -1 default")
     ap.add_argument("--rows", type=int, default=0, help="K/V loads per wave tile: 2 / 4 (0 = default)")
+    ap.add_argument("--layout", default="NHD", choices=["NHD", "HND"], help="page layout")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of hipGraph")
     ap.add_argument("--only-sparse", action="store_true",
@@ -71,7 +72,8 @@ class Workload:
         self.sel_layers = (0, 2)
         self.dtype = torch.bfloat16
         c = InferenceController(self.L, self.H, self.D, self.P, self.K, self.N + 64, self.dtype,
-                                self.dev, select_mode=select_mode, page_order_seed=0)
+                                self.dev, select_mode=select_mode, page_order_seed=0,
+                                kv_layout=args.layout)
         h = c._decode_handler._wrapper
         h.waves_per_block, h.chunk_tokens, h.fused_merge = args.waves, args.chunk, args.merge
         h.tile_rows = args.rows

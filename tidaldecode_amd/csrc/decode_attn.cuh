@@ -223,9 +223,10 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
   const int idx_row = (QPG == 1 && p.idx_per_kv) ? kv_head : hrow;
   s.row = p.idx + (int64_t)idx_row * p.idx_row_stride + list_beg;
 
-  const int c0 = split * p.chunk_tokens;
-  int c1 = c0 + p.chunk_tokens;
-  c1 = c1 > s.n_items ? s.n_items : c1;
+  // The splits of a head row interleave: split s takes the workgroup-wide tiles s, s + n_splits,
+  // s + 2 n_splits, ... so that all workgroups sweep the sequence together as one moving window
+  // (DRAM row locality of a streaming read) instead of as n_splits distant streams.
+  const int c1 = s.n_items;
 
   // query: QPG heads x 8 elements per lane, kept packed in the KV dtype
   uint32_t qp[QPG][4];
@@ -310,21 +311,25 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         offs[u] = page[u] * p.page_stride_b + entry[u] * p.entry_stride_b + head_byte_off;
-        kb[u] = *reinterpret_cast<const u32x4*>(kbase + offs[u]);
+        kb[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kbase + offs[u]));
       }
-      // V after all K: the q.k arithmetic of a tile starts while its V rows are still in flight
+      // V after all K: the q.k arithmetic of a tile starts while its V rows are still in flight.
+      // K/V rows are read once per launch: non-temporal loads keep them from displacing the lists,
+      // q and the split partials in L2 / Infinity Cache (measured: +15 % on the streaming layer).
 #pragma unroll
-      for (int u = 0; u < U; ++u) vb[u] = *reinterpret_cast<const u32x4*>(vbase + offs[u]);
+      for (int u = 0; u < U; ++u)
+        vb[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vbase + offs[u]));
     } else {
       int64_t offs[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         offs[u] = (int64_t)page[u] * p.page_stride + (int64_t)entry[u] * p.entry_stride + kv_head_off;
-        kb[u] = *reinterpret_cast<const u32x4*>(kv16 + offs[u]);
+        kb[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kv16 + offs[u]));
       }
 #pragma unroll
       for (int u = 0; u < U; ++u)
-        vb[u] = *reinterpret_cast<const u32x4*>(kv16 + offs[u] + p.v_offset);
+        vb[u] = __builtin_nontemporal_load(
+            reinterpret_cast<const u32x4*>(kv16 + offs[u] + p.v_offset));
     }
   };
   auto reduce = [&](const u32x4(&kb)[U], const u32x4(&vb)[U], int base) {
@@ -390,8 +395,8 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
     }
   };
 
-  constexpr int STEP = NW * TILE;  // tokens between two tiles of one wave
-  int t = c0 + wave * TILE;        // first token of this wave's current tile
+  const int STEP = n_splits * NW * TILE;  // tokens between two tiles of one wave
+  int t = (split * NW + wave) * TILE;     // first token of this wave's current tile
   if (t < c1) {
     fetch_list(t, rawA);
     if (t + STEP < c1) fetch_list(t + STEP, rawB);
