@@ -43,6 +43,8 @@ def parse():
     ap.add_argument("--merge", type=int, default=-1, help="1 fused / 0 second kernel / -1 default")
     ap.add_argument("--rows", type=int, default=0, help="K/V loads per wave tile: 2 / 4 (0 = default)")
     ap.add_argument("--layout", default="NHD", choices=["NHD", "HND"], help="page layout")
+    ap.add_argument("--no-fuse", action="store_true",
+                    help="run RoPE + append as their own launch instead of inside attention")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of hipGraph")
     ap.add_argument("--only-sparse", action="store_true",
@@ -92,6 +94,9 @@ class Workload:
         page = c.kv_cache.indicies[pos // self.P]
         self.dst_slot = torch.tensor([page * self.P + pos % self.P], dtype=torch.int32,
                                      device=self.dev)
+        self.fuse = (not args.no_fuse) and c.fused_step_ok
+        from tidaldecode_amd import _kernels
+        self.cos, self.sin = _kernels.rope_table(self.positions, self.D)
 
     # --- pieces of the step ---------------------------------------------------------------
     def rope_append(self, layer):
@@ -100,37 +105,51 @@ class Workload:
         ops.rope_append_kv(self.q[layer], self.k[layer], self.v[layer], self.c, layer,
                            self.positions, self.dst_slot)
 
-    def select_attn(self, layer):
+    def fresh(self, layer):
+        return (self.k[layer], self.v[layer], self.cos, self.sin, self.dst_slot)
+
+    def rope_table(self):
+        from tidaldecode_amd import _kernels
+
+        _kernels.rope_table(self.positions, self.D, 1.0, 1e4, self.cos, self.sin)
+
+    def select_attn(self, layer, fresh=None):
         from tidaldecode_amd import utils as ops
 
         return ops.decode_sparse_attn(self.q[layer], self.c, layer,
-                                      self.c.kv_indices_without_last, True)
+                                      self.c.kv_indices_without_last, True, fresh=fresh)
 
-    def full_attn(self, layer):
+    def full_attn(self, layer, fresh=None):
         from tidaldecode_amd import utils as ops
 
         return ops.decode_sparse_attn(self.q[layer], self.c, layer,
-                                      self.c.kv_indices_without_last, False)
+                                      self.c.kv_indices_without_last, False, fresh=fresh)
 
     def topk(self):
         from tidaldecode_amd import utils as ops
 
         ops.decode_topk(self.c)
 
-    def sparse_attn(self, layer):
+    def sparse_attn(self, layer, fresh=None):
         from tidaldecode_amd import utils as ops
 
         return ops.decode_sparse_attn(self.q[layer], self.c, layer,
-                                      self.c.topk_dindices_buffer, False)
+                                      self.c.topk_dindices_buffer, False, fresh=fresh)
 
     def step(self):
+        """attention path of one decode step; with fusion RoPE + append ride inside the attention
+        launches and only the cos/sin table is a launch of its own (once per step)"""
+        if self.fuse:
+            self.rope_table()
         for layer in range(self.L):
-            self.rope_append(layer)
+            fresh = self.fresh(layer) if self.fuse else None
+            if not self.fuse:
+                self.rope_append(layer)
             if layer in self.sel_layers:
-                self.select_attn(layer)
+                self.select_attn(layer, fresh)
                 self.topk()
             else:
-                self.sparse_attn(layer)
+                self.sparse_attn(layer, fresh)
 
     def sparse_layers(self):
         return [l for l in range(self.L) if l not in self.sel_layers]
@@ -275,15 +294,16 @@ def main():
 
         def run_sparse():
             for layer in sparse:
-                w.sparse_attn(layer)
+                w.sparse_attn(layer, w.fresh(layer) if w.fuse else None)
 
         r_sparse, how = capture(torch, run_sparse, use_graph)
         sparse_ms = time_events(torch, r_sparse, max(args.steps, 20))
-        entry = {"sparse_us_per_layer": sparse_ms * 1e3 / len(sparse), "launch": how}
+        entry = {"sparse_us_per_layer": sparse_ms * 1e3 / len(sparse), "launch": how,
+                 "fused_rope_append": bool(w.fuse)}
         if not args.only_sparse:
             def run_select():
                 for layer in w.sel_layers:
-                    w.select_attn(layer)
+                    w.select_attn(layer, w.fresh(layer) if w.fuse else None)
 
             def run_topk():
                 for _ in w.sel_layers:
@@ -313,9 +333,12 @@ def main():
             # the same step with full attention in every layer (no selection): attention-only
             # latency ratio, the quantity the reference plots (README, llama_latency_eval.png)
             def full_step():
+                if w.fuse:
+                    w.rope_table()
                 for layer in range(w.L):
-                    w.rope_append(layer)
-                    w.full_attn(layer)
+                    if not w.fuse:
+                        w.rope_append(layer)
+                    w.full_attn(layer, w.fresh(layer) if w.fuse else None)
 
             r_full, _ = capture(torch, full_step, use_graph)
             entry["full_attention_ms_per_step"] = time_events(torch, r_full, 5, warm=1)

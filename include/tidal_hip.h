@@ -108,6 +108,19 @@ typedef struct {
   int64_t workspace_bytes; /* device scratch the call needs (partials + tickets) */
 } td_decode_plan;
 
+/*
+ * The token being decoded, for the fused decode step of td_decode_attn: its un-rotated key and
+ * value rows, the cosines / sines of its rotary angles (td_rope_table) and the physical slot it
+ * occupies.  All device pointers.
+ */
+typedef struct {
+  const void* k;           /* [batch, num_kv_heads, head_dim] */
+  const void* v;           /* [batch, num_kv_heads, head_dim] */
+  const float* cos;        /* [batch, head_dim / 2] */
+  const float* sin;        /* [batch, head_dim / 2] */
+  const int32_t* dst_slot; /* [batch]: page_id * page_size + entry */
+} td_fresh_token;
+
 /* Thread-local message of the last failing call. */
 const char* td_last_error(void);
 
@@ -177,6 +190,13 @@ int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t num_kv_head
  *   scores     optional [batch, num_qo_heads, score_stride]: element i = q . k_i / sqrt(D) of the
  *              i-th attended token in list order (td_dtype scores_dtype); NULL to skip
  *   lse        optional float [batch, num_qo_heads]: natural-log sum of exp of the logits
+ *   fresh      optional (NULL = off) decode-step fusion: q is then the UN-rotated query; the
+ *              kernel rotates it in registers (q in memory is left as it was), rotates fresh->k,
+ *              writes it and fresh->v into the cache at fresh->dst_slot, and attends to that
+ *              token wherever the list names its slot -- one launch instead of
+ *              td_rope_append_decode + td_decode_attn (tidal/models/SearchAttention.py:131-176 runs
+ *              three).  Needs a power-of-two page_size and a pool below 4 GiB
+ *              (TD_ERR_UNSUPPORTED otherwise).
  *   workspace  device scratch of at least plan->workspace_bytes whose first 64 KiB (ticket
  *              counters) were zero-filled once before first use; every call leaves them zero
  *              again, so one workspace serves plans of any shape.  Calls that share a
@@ -189,7 +209,16 @@ int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t num_kv_head
 int td_decode_attn(const td_paged_kv* kv, const td_index_list* list, const td_decode_plan* plan,
                    const void* q, void* o, int32_t batch, int32_t num_qo_heads, float sm_scale,
                    void* scores, int32_t scores_dtype, int64_t score_stride, float* lse,
-                   void* workspace, int64_t workspace_bytes, void* stream);
+                   const td_fresh_token* fresh, void* workspace, int64_t workspace_bytes,
+                   void* stream);
+
+/*
+ * cos[b, j] / sin[b, j] of positions[b] / rope_scale * rope_theta^(-2j/head_dim), j < head_dim/2
+ * (angles formed in double precision, as td_rope_in_place does).  One launch per decode step
+ * serves every layer's fused td_decode_attn.
+ */
+int td_rope_table(const int32_t* positions, int32_t batch, int32_t head_dim, float rope_scale,
+                  float rope_theta, float* cos, float* sin, void* stream);
 
 /*
  * Cross-head reduction of selection-layer scores: out[r, i] = sum over the query heads h of

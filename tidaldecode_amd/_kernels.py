@@ -19,7 +19,7 @@ from typing import Optional
 import torch
 
 from . import _lib
-from ._lib import (DecodePlan, IndexList, PagedKV, TD_BF16, TD_F16, TD_F32, TD_HND, TD_IDX_PAGES,
+from ._lib import (DecodePlan, FreshToken, IndexList, PagedKV, TD_BF16, TD_F16, TD_F32, TD_HND, TD_IDX_PAGES,
                    TD_IDX_SLOTS, TD_NHD, check, lib)
 
 _DTYPES = {torch.float16: TD_F16, torch.bfloat16: TD_BF16, torch.float32: TD_F32}
@@ -250,6 +250,23 @@ def rope_append_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, kv_dat
                                     float(rope_theta), _stream()))
 
 
+def rope_table(positions: torch.Tensor, head_dim: int, rope_scale: float = 1.0,
+               rope_theta: float = 1e4, cos: Optional[torch.Tensor] = None,
+               sin: Optional[torch.Tensor] = None):
+    """Extension: cos / sin ``[B, D/2]`` float32 of the rotary angles of ``positions`` ``[B]``
+    (int32); one call per decode step feeds every layer's fused ``forward(..., fresh=...)``."""
+    _check_input(positions, "positions")
+    _check_i32(positions, "positions")
+    b = positions.numel()
+    if cos is None:
+        cos = torch.empty((b, head_dim // 2), dtype=torch.float32, device=positions.device)
+    if sin is None:
+        sin = torch.empty((b, head_dim // 2), dtype=torch.float32, device=positions.device)
+    check(lib.td_rope_table(positions.data_ptr(), b, int(head_dim), float(rope_scale),
+                            float(rope_theta), cos.data_ptr(), sin.data_ptr(), _stream()))
+    return cos, sin
+
+
 def prefill_with_paged_kv_cache(q, kv_data, kv_indices, kv_last_page_len, causal, layout,
                                 allow_fp16_qk_reduction, rope_scale, rope_theta) -> torch.Tensor:
     """bsk_ops.h:80-88 / batch_prefill.cu:27-117.  Causal attention of the ``q.size(0)`` newest
@@ -342,14 +359,19 @@ class BatchDecodeWithPagedKVCachePyTorchWrapper:
                 paged_kv_last_page_len, paged_kv_last_page_idx,
                 qk_product: Optional[torch.Tensor], rope_scale: float = 1.0,
                 rope_theta: float = 1e4, *, index_kind: str = "pages",
-                lse: Optional[torch.Tensor] = None, n_list: Optional[int] = None) -> None:
+                lse: Optional[torch.Tensor] = None, n_list: Optional[int] = None,
+                fresh=None) -> None:
         """q, o ``[B, H_q, D]``; ``paged_kv_indices`` ``[rows, budget]`` int32 with rows in
         {H_q, H_kv, 1}; sequence b uses columns ``indptr[b]:indptr[b+1]`` of every row and then
         the first ``last_page_len`` entries of page ``last_page_idx`` (ints, or int32 device
         tensors ``[B]``).  ``index_kind="slots"`` reads the entries as token slots.
         ``n_list`` bounds the per-sequence column count (default: all columns).
         rope_scale / rope_theta are accepted for signature parity; RoPE is applied before the
-        cache is written (RotaryMode::kNone in the reference, approx_attn.cu:52,139)."""
+        cache is written (RotaryMode::kNone in the reference, approx_attn.cu:52,139).
+        ``fresh=(k, v, cos, sin, dst_slot)`` fuses the decode step: q, k ``[B, H, D]`` are then
+        UN-rotated, cos/sin ``[B, D/2]`` float32 come from ``rope_table``; the kernel rotates q
+        in registers, writes rotated k and v to ``dst_slot`` and attends to them from registers
+        (power-of-two pages and pools below 4 GiB only)."""
         if not self._begun:
             raise RuntimeError("Please call BatchDecodeHandler's BeginForward() before calling "
                                "BatchDecodeWithPagedKVCacheWrapper()")
@@ -425,10 +447,27 @@ class BatchDecodeWithPagedKVCachePyTorchWrapper:
             if lse.dtype != torch.float32 or lse.numel() != batch * hq:
                 raise RuntimeError("lse must be float32 [B, H_q]")
             lse_ptr = lse.data_ptr()
+        fresh_arg = None
+        if fresh is not None:
+            fk, fv, fcos, fsin, fslot = fresh
+            for t, n in ((fk, "fresh k"), (fv, "fresh v"), (fcos, "fresh cos"), (fsin, "fresh sin"),
+                         (fslot, "fresh dst_slot")):
+                _check_input(t, n)
+            if fk.shape != (batch, hkv, d) or fv.shape != fk.shape or fk.dtype != dtype or \
+                    fv.dtype != dtype:
+                raise RuntimeError("fresh k / v must be [B, H_kv, D] in the cache dtype")
+            if fcos.dtype != torch.float32 or fsin.dtype != torch.float32 or \
+                    fcos.numel() != batch * d // 2 or fsin.numel() != batch * d // 2:
+                raise RuntimeError("fresh cos / sin must be float32 [B, D/2]")
+            _check_i32(fslot, "fresh dst_slot")
+            if fslot.numel() != batch:
+                raise RuntimeError("fresh dst_slot must hold one entry per sequence")
+            fresh_arg = FreshToken(fk.data_ptr(), fv.data_ptr(), fcos.data_ptr(), fsin.data_ptr(),
+                                   fslot.data_ptr())
         ws = self._workspace
         check(lib.td_decode_attn(pool, lst, plan, q.data_ptr(), o.data_ptr(), batch, hq,
                                  1.0 / math.sqrt(d), scores_ptr, scores_dtype, score_stride,
-                                 lse_ptr, ws.data_ptr() if ws is not None else None,
+                                 lse_ptr, fresh_arg, ws.data_ptr() if ws is not None else None,
                                  ws.numel() if ws is not None else 0, _stream()))
 
 

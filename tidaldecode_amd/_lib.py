@@ -49,6 +49,18 @@ class IndexList(Structure):
     ]
 
 
+class FreshToken(Structure):
+    """td_fresh_token"""
+
+    _fields_ = [
+        ("k", c_void_p),
+        ("v", c_void_p),
+        ("cos", c_void_p),
+        ("sin", c_void_p),
+        ("dst_slot", c_void_p),
+    ]
+
+
 class DecodePlan(Structure):
     """td_decode_plan"""
 
@@ -89,7 +101,12 @@ SIGNATURES = {
     "td_decode_attn": (
         c_int32,
         [POINTER(PagedKV), POINTER(IndexList), POINTER(DecodePlan), c_void_p, c_void_p, c_int32,
-         c_int32, c_float, c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_int64, c_void_p],
+         c_int32, c_float, c_void_p, c_int32, c_int64, c_void_p, POINTER(FreshToken), c_void_p,
+         c_int64, c_void_p],
+    ),
+    "td_rope_table": (
+        c_int32,
+        [c_void_p, c_int32, c_int32, c_float, c_float, c_void_p, c_void_p, c_void_p],
     ),
     "td_score_reduce": (
         c_int32,

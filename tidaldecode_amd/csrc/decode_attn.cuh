@@ -67,6 +67,12 @@ struct DecodeParams {
   float* ws_o;      // [batch * H_q * max_splits, D]
   float* ws_ml;     // [batch * H_q * max_splits, 2]
   int32_t* ws_cnt;  // [batch * head rows] ticket counters
+  // the token being decoded (FRESH kernels): un-rotated k, v, its rotary cos/sin and its slot
+  const void* fresh_k;
+  const void* fresh_v;
+  const float* fresh_cos;
+  const float* fresh_sin;
+  const int32_t* fresh_slot;
 };
 
 template <bool LEAN>
@@ -200,8 +206,9 @@ __device__ __forceinline__ int seq_items(const DecodeParams& p, int b, SeqList& 
   return n_splits < 1 ? 1 : n_splits;
 }
 
-template <typename T, int D, int QPG, int U, int NW, bool PAGE_MODE, bool EMIT, bool LEAN>
+template <typename T, int D, int QPG, int U, int NW, bool PAGE_MODE, bool EMIT, bool LEAN, bool FRESH>
 __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams p) {
+  static_assert(!FRESH || LEAN, "the fused decode step exists for the lean addressing only");
   constexpr int LPR = D / 8;     // lanes per K/V row
   constexpr int TPI = 64 / LPR;  // tokens one wave instruction covers
   constexpr int TILE = U * TPI;  // tokens per wave tile
@@ -243,6 +250,63 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
     }
   }
 
+  // Decode-step fusion: q arrives un-rotated and is rotated in registers; the new token's k is
+  // rotated here as well, written to its cache slot by one workgroup per KV head, and used from
+  // registers wherever the list refers to that slot (the cache write races with nobody: no lane
+  // consumes what it loaded from that slot).
+  uint32_t knew[4] = {0, 0, 0, 0}, vnew[4] = {0, 0, 0, 0};
+  uint32_t new_page = 0xffffffffu, new_entry = 0;
+  float rcs[8], rsn[8];  // cos and signed sin of this lane's 8 dimensions
+  if constexpr (FRESH) {
+    constexpr int HALF = LPR / 2;  // lanes holding the first half of the head dimension
+    const uint32_t ns = (uint32_t)p.fresh_slot[b];
+    new_page = ns >> p.page_shift;
+    new_entry = ns & ((1u << p.page_shift) - 1u);
+    const f32x4* cp = reinterpret_cast<const f32x4*>(p.fresh_cos + (int64_t)b * (D / 2) + (li % HALF) * 8);
+    const f32x4* sp = reinterpret_cast<const f32x4*>(p.fresh_sin + (int64_t)b * (D / 2) + (li % HALF) * 8);
+    const f32x4 c0 = cp[0], c1v = cp[1], s0 = sp[0], s1 = sp[1];
+    rcs[0] = c0.x; rcs[1] = c0.y; rcs[2] = c0.z; rcs[3] = c0.w;
+    rcs[4] = c1v.x; rcs[5] = c1v.y; rcs[6] = c1v.z; rcs[7] = c1v.w;
+    const float sgn = li < HALF ? -1.f : 1.f;  // y_lo = x_lo c - x_hi s,  y_hi = x_hi c + x_lo s
+    rsn[0] = sgn * s0.x; rsn[1] = sgn * s0.y; rsn[2] = sgn * s0.z; rsn[3] = sgn * s0.w;
+    rsn[4] = sgn * s1.x; rsn[5] = sgn * s1.y; rsn[6] = sgn * s1.z; rsn[7] = sgn * s1.w;
+    const int64_t fresh_off =
+        ((int64_t)b * (p.num_qo_heads / (QPG > 1 ? QPG : p.q_per_kv)) + kv_head) * LPR + li;
+    const u32x4 kn = reinterpret_cast<const u32x4*>(p.fresh_k)[fresh_off];
+    const u32x4 vn = reinterpret_cast<const u32x4*>(p.fresh_v)[fresh_off];
+    knew[0] = kn.x; knew[1] = kn.y; knew[2] = kn.z; knew[3] = kn.w;
+    vnew[0] = vn.x; vnew[1] = vn.y; vnew[2] = vn.z; vnew[3] = vn.w;
+  }
+  // Rotation of q and of the new key, and the cache write; called once the first K/V tile of
+  // the wave is in flight so that these few loads and shuffles hide behind it.
+  auto finish_fresh = [&]() {
+    if constexpr (FRESH) {
+      constexpr int HALF = LPR / 2;
+      auto rotate = [&](uint32_t(&w)[4]) {
+        float x[8], y[8];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) unpack2<T>(w[c], x[2 * c], x[2 * c + 1]);
+#pragma unroll
+        for (int d = 0; d < 8; ++d) y[d] = x[d] * rcs[d] + __shfl_xor(x[d], HALF, 64) * rsn[d];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) w[c] = pack2<T>(y[2 * c], y[2 * c + 1]);
+      };
+#pragma unroll
+      for (int j = 0; j < QPG; ++j) rotate(qp[j]);
+      rotate(knew);
+      const bool writer_row = QPG > 1 || (hrow % p.q_per_kv) == 0;
+      if (split == 0 && wave == 0 && g == 0 && writer_row) {
+        const uint32_t page_c = new_page > p.max_page ? p.max_page : new_page;
+        char* dst = reinterpret_cast<char*>(const_cast<void*>(p.kv)) + page_c * p.page_stride_b +
+                    new_entry * p.entry_stride_b + (uint32_t)(kv_head * p.head_stride + li * 8) * 2u;
+        u32x4 ko = {knew[0], knew[1], knew[2], knew[3]};
+        u32x4 vo = {vnew[0], vnew[1], vnew[2], vnew[3]};
+        *reinterpret_cast<u32x4*>(dst) = ko;
+        *reinterpret_cast<u32x4*>(dst + p.v_offset * 2) = vo;
+      }
+    }
+  };
+
   float m[QPG], l[QPG], acc[QPG][8];
 #pragma unroll
   for (int j = 0; j < QPG; ++j) {
@@ -261,6 +325,7 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
   // K/V stay in flight per wave.
   u32x4 kA[U], vA[U], kB[U], vB[U];
   int32_t rawA[U], rawB[U];
+  uint32_t hitA = 0, hitB = 0;
 
   // Address generation is branch-free: an item past the end of the chunk is redirected to the
   // chunk's last item (a valid address; its contribution is masked out in the arithmetic) and
@@ -287,7 +352,7 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
                         : 0;
     }
   };
-  auto issue = [&](int base, const int32_t(&raw)[U], u32x4(&kb)[U], u32x4(&vb)[U]) {
+  auto issue = [&](int base, const int32_t(&raw)[U], u32x4(&kb)[U], u32x4(&vb)[U], uint32_t& hit) {
     uint32_t page[U], entry[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -305,6 +370,12 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
         divmod_page<LEAN>(p, slot, page[u], entry[u]);
       }
       page[u] = page[u] > p.max_page ? p.max_page : page[u];
+    }
+    hit = 0;
+    if constexpr (FRESH) {
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        hit |= (page[u] == new_page && entry[u] == new_entry) ? (1u << u) : 0u;
     }
     if constexpr (LEAN) {
       uint32_t offs[U];
@@ -332,7 +403,18 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
             reinterpret_cast<const u32x4*>(kv16 + offs[u] + p.v_offset));
     }
   };
-  auto reduce = [&](const u32x4(&kb)[U], const u32x4(&vb)[U], int base) {
+  auto reduce = [&](u32x4(&kb)[U], u32x4(&vb)[U], int base, uint32_t hit) {
+    if constexpr (FRESH) {
+      if (__ballot(hit != 0)) {  // rare: some lane group of this wave meets the new token
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if ((hit >> u) & 1u) {
+            kb[u].x = knew[0]; kb[u].y = knew[1]; kb[u].z = knew[2]; kb[u].w = knew[3];
+            vb[u].x = vnew[0]; vb[u].y = vnew[1]; vb[u].z = vnew[2]; vb[u].w = vnew[3];
+          }
+        }
+      }
+    }
     float sc[QPG][U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -400,22 +482,25 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
   if (t < c1) {
     fetch_list(t, rawA);
     if (t + STEP < c1) fetch_list(t + STEP, rawB);
-    issue(t, rawA, kA, vA);
+    issue(t, rawA, kA, vA, hitA);
+    finish_fresh();
     while (true) {
       // A: K/V of tile t in flight; rawB: list entries of tile t+STEP in flight
       const int tn = t + STEP;
       const int tnn = tn + STEP;
       if (tnn < c1) fetch_list(tnn, rawA);
-      if (tn < c1) issue(tn, rawB, kB, vB);
-      reduce(kA, vA, t);
+      if (tn < c1) issue(tn, rawB, kB, vB, hitB);
+      reduce(kA, vA, t, hitA);
       if (tn >= c1) break;
       const int tnnn = tnn + STEP;
       if (tnnn < c1) fetch_list(tnnn, rawB);
-      if (tnn < c1) issue(tnn, rawA, kA, vA);
-      reduce(kB, vB, tn);
+      if (tnn < c1) issue(tnn, rawA, kA, vA, hitA);
+      reduce(kB, vB, tn, hitB);
       if (tnn >= c1) break;
       t = tnn;
     }
+  } else {
+    finish_fresh();  // a wave without tokens still takes part in the shuffles and the write
   }
 
   // ---- combine the TPI token slots of the wave (butterfly over lane groups) ---------------------
@@ -542,11 +627,14 @@ static int qpg_for(int num_qo_heads, int num_kv_heads, int idx_rows, int head_di
 
 template <typename T, int D, int QPG, int NW, int U, bool PAGE_MODE, bool EMIT>
 static void launch_lean(const DecodeParams& p, dim3 grid, hipStream_t st) {
-  if (p.lean)
-    hipLaunchKernelGGL((decode_attn_kernel<T, D, QPG, U, NW, PAGE_MODE, EMIT, true>), grid,
+  if (p.lean && p.fresh_k)
+    hipLaunchKernelGGL((decode_attn_kernel<T, D, QPG, U, NW, PAGE_MODE, EMIT, true, true>), grid,
+                       dim3(NW * 64), 0, st, p);
+  else if (p.lean)
+    hipLaunchKernelGGL((decode_attn_kernel<T, D, QPG, U, NW, PAGE_MODE, EMIT, true, false>), grid,
                        dim3(NW * 64), 0, st, p);
   else
-    hipLaunchKernelGGL((decode_attn_kernel<T, D, QPG, U, NW, PAGE_MODE, EMIT, false>), grid,
+    hipLaunchKernelGGL((decode_attn_kernel<T, D, QPG, U, NW, PAGE_MODE, EMIT, false, false>), grid,
                        dim3(NW * 64), 0, st, p);
 }
 

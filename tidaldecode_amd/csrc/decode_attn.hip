@@ -101,7 +101,8 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
                               const td_decode_plan* plan, const void* q, void* o, int32_t batch,
                               int32_t num_qo_heads, float sm_scale, void* scores,
                               int32_t scores_dtype, int64_t score_stride, float* lse,
-                              void* workspace, int64_t workspace_bytes, void* stream) {
+                              const td_fresh_token* fresh, void* workspace,
+                              int64_t workspace_bytes, void* stream) {
   TD_REQUIRE(kv && list && plan && q && o, "td_decode_attn: NULL argument");
   TD_REQUIRE(kv->data != nullptr, "td_decode_attn: kv->data is NULL");
   TD_REQUIRE(batch >= 1, "td_decode_attn: batch %d < 1", batch);
@@ -194,6 +195,23 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
   p.page_stride_b = (uint32_t)(p.page_stride * 2);
   p.entry_stride_b = (uint32_t)(p.entry_stride * 2);
   p.lean = (p.page_shift >= 0 && (int64_t)kv->max_pages * p.page_stride * 2 < ((int64_t)1 << 32)) ? 1 : 0;
+  p.fresh_k = p.fresh_v = nullptr;
+  p.fresh_cos = p.fresh_sin = nullptr;
+  p.fresh_slot = nullptr;
+  if (fresh) {
+    TD_REQUIRE(fresh->k && fresh->v && fresh->cos && fresh->sin && fresh->dst_slot,
+               "td_decode_attn: fresh token with a NULL member");
+    if (!p.lean)
+      return fail(TD_ERR_UNSUPPORTED,
+                  "td_decode_attn: the fused decode step needs a power-of-two page_size and a pool "
+                  "below 4 GiB (page_size %d, pool %lld bytes); use td_rope_append_decode first",
+                  P, (long long)(kv->max_pages * p.page_stride * 2));
+    p.fresh_k = fresh->k;
+    p.fresh_v = fresh->v;
+    p.fresh_cos = fresh->cos;
+    p.fresh_sin = fresh->sin;
+    p.fresh_slot = fresh->dst_slot;
+  }
   p.num_qo_heads = num_qo_heads;
   p.n_hrows = n_hrows;
   p.q_per_kv = num_qo_heads / Hkv;

@@ -84,6 +84,16 @@ __global__ __launch_bounds__(256) void rope_kernel(uint16_t* q, uint16_t* k, int
   }
 }
 
+// grid: batch; block: D/2 threads.  cos/sin of one token's rotary angles
+__global__ void rope_table_kernel(const int32_t* positions, int D, double inv_scale,
+                                  double log2_theta, float* cos_out, float* sin_out) {
+  const int b = blockIdx.x, j = threadIdx.x;
+  float sn, cs;
+  rope_sincos((double)positions[b] * inv_scale, log2_theta, j, D, sn, cs);
+  cos_out[(int64_t)b * (D / 2) + j] = cs;
+  sin_out[(int64_t)b * (D / 2) + j] = sn;
+}
+
 // grid: batch; rotates q in place, rotates k into the cache slot, copies v into the cache slot
 template <typename T>
 __global__ __launch_bounds__(256) void rope_append_decode_kernel(
@@ -329,6 +339,22 @@ extern "C" int td_rope_append_decode(const td_paged_kv* kv, void* q, const void*
   else
     return fail(TD_ERR_UNSUPPORTED, "td_rope_append_decode failed to dispatch with dtype %d",
                 kv->dtype);
+  TD_HIP_CHECK(hipGetLastError());
+  return TD_OK;
+}
+
+extern "C" int td_rope_table(const int32_t* positions, int32_t batch, int32_t head_dim,
+                             float rope_scale, float rope_theta, float* cos, float* sin,
+                             void* stream) {
+  TD_REQUIRE(positions && cos && sin, "td_rope_table: NULL argument");
+  TD_REQUIRE(batch >= 1, "td_rope_table: batch %d", batch);
+  TD_REQUIRE(rope_scale > 0.f && rope_theta > 0.f, "td_rope_table: scale %g theta %g", rope_scale,
+             rope_theta);
+  if (head_dim != 64 && head_dim != 128 && head_dim != 256)
+    return fail(TD_ERR_UNSUPPORTED, "td_rope_table: head_dim %d (supported: 64, 128, 256)", head_dim);
+  hipLaunchKernelGGL(rope_table_kernel, dim3(batch), dim3(head_dim / 2), 0,
+                     reinterpret_cast<hipStream_t>(stream), positions, head_dim,
+                     1.0 / (double)rope_scale, log2((double)rope_theta), cos, sin);
   TD_HIP_CHECK(hipGetLastError());
   return TD_OK;
 }

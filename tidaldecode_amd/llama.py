@@ -18,6 +18,7 @@ from typing import Optional, Tuple
 
 import torch
 
+from . import _kernels
 from . import utils as tidal_utils
 from .utils import InferenceController
 
@@ -87,6 +88,9 @@ class TidalLlama:
         self.iController: Optional[InferenceController] = None
         self._positions = torch.zeros(1, dtype=torch.int32, device=self.device)
         self._dst_slot = torch.zeros(1, dtype=torch.int32, device=self.device)
+        self._cos = torch.zeros((1, c.head_dim // 2), dtype=torch.float32, device=self.device)
+        self._sin = torch.zeros((1, c.head_dim // 2), dtype=torch.float32, device=self.device)
+        self.fuse_decode_step = True  # RoPE + append inside the attention launch when possible
 
     # ----- cache lifecycle (tidal/models/llama.py:616-656) -----------------------------------
     def tidal_init(self, page_size: int, max_seq_len: int, token_budget: Optional[int] = None,
@@ -168,6 +172,8 @@ class TidalLlama:
         page = ctrl.kv_cache.indicies[pos // ctrl.page_size]
         self._positions.fill_(pos)
         self._dst_slot.fill_(page * ctrl.page_size + pos % ctrl.page_size)
+        _kernels.rope_table(self._positions, self.config.head_dim, self.config.rope_scale,
+                            self.config.rope_theta, self._cos, self._sin)
 
     @torch.no_grad()
     def decode_layers(self, x: torch.Tensor) -> torch.Tensor:
@@ -177,14 +183,19 @@ class TidalLlama:
         for idx, layer in enumerate(self.layers):
             h = self._rms(x, layer["ln1"])
             q, k, v = self._qkv(layer, h)
-            tidal_utils.rope_append_kv(q, k, v, ctrl, idx, self._positions, self._dst_slot,
-                                       c.rope_scale, c.rope_theta)
+            fresh = None
+            if self.fuse_decode_step and ctrl.fused_step_ok:
+                fresh = (k, v, self._cos, self._sin, self._dst_slot)
+            else:
+                tidal_utils.rope_append_kv(q, k, v, ctrl, idx, self._positions, self._dst_slot,
+                                           c.rope_scale, c.rope_theta)
             kind = c.layer_kind(idx)
             if kind == "sparse":
-                o = tidal_utils.decode_sparse_attn(q, ctrl, idx, ctrl.topk_dindices_buffer, False)
+                o = tidal_utils.decode_sparse_attn(q, ctrl, idx, ctrl.topk_dindices_buffer, False,
+                                                   fresh=fresh)
             else:
                 o = tidal_utils.decode_sparse_attn(q, ctrl, idx, ctrl.kv_indices_without_last,
-                                                   kind == "select")
+                                                   kind == "select", fresh=fresh)
                 if kind == "select":
                     tidal_utils.decode_topk(ctrl)
             x = x + o.reshape(1, -1) @ layer["wo"].t()

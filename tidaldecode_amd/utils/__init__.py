@@ -110,13 +110,16 @@ def decode_topk(iController: InferenceController):
 
 def decode_sparse_attn(q: torch.Tensor, iController: InferenceController, layer_idx: int,
                        topk_indices: torch.Tensor, output_qk_product: bool,
-                       rope_scale: Optional[float] = None, rope_theta: Optional[float] = None
-                       ) -> torch.Tensor:
+                       rope_scale: Optional[float] = None, rope_theta: Optional[float] = None,
+                       fresh=None) -> torch.Tensor:
     """Attention of the new token ``q [1, H, D]`` over the listed part of the cache.
 
     ``topk_indices is iController.kv_indices_without_last``: every page in order plus the last
     page, i.e. full attention; with ``output_qk_product`` the logits (and log-sum-exp) are kept
     for ``decode_topk``.  Otherwise ``topk_indices`` holds token slots chosen by ``decode_topk``.
+
+    ``fresh=(k, v, cos, sin, dst_slot)`` (extension) folds ``apply_rope_in_place`` and
+    ``append_kv`` of the new token into this launch: q and k are then un-rotated.
     """
     c = iController
     o = torch.empty_like(q)
@@ -125,12 +128,13 @@ def decode_sparse_attn(q: torch.Tensor, iController: InferenceController, layer_
         c._decode_handler.forward(q, o, c.kv_cache.buf_layer(layer_idx), topk_indices, None,
                                   c.kv_cache.last_page_len, c.kv_last_page_idx,
                                   c.qk_product if output_qk_product else None, rope_scale,
-                                  rope_theta, lse=c.lse if output_qk_product else None)
+                                  rope_theta, lse=c.lse if output_qk_product else None,
+                                  fresh=fresh)
     else:
         forced = c.select_scope == "exclude_last_page"
         c._decode_handler.forward(q, o, c.kv_cache.buf_layer(layer_idx), topk_indices, None,
                                   c.kv_cache.last_page_len if forced else 0,
                                   c.kv_last_page_idx if forced else 0,
                                   c.qk_product if output_qk_product else None, rope_scale,
-                                  rope_theta, index_kind="slots")
+                                  rope_theta, index_kind="slots", fresh=fresh)
     return o

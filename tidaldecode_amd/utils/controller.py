@@ -100,6 +100,10 @@ class InferenceController:
 
         self.prefill_latency = []
         self.decode_latency = []
+        # the fused decode step (RoPE + append inside the attention launch) exists for
+        # power-of-two pages and per-layer pools below 4 GiB
+        layer_bytes = self.kv_cache.pool.buf[0].numel() * self.kv_cache.pool.buf.element_size()
+        self.fused_step_ok = (page_size & (page_size - 1)) == 0 and layer_bytes < (1 << 32)
 
     # Used for controlling the number of pages (the reference skips its first layers with it)
     def set_token_budget(self, token_budget: int):
