@@ -240,13 +240,22 @@ int td_score_reduce(const float* logits, int64_t logits_stride, const float* lse
  *     page_table != NULL          -> page_table[p / page_size] * page_size + p % page_size
  *     both NULL                   -> p
  * k is clamped to len.  NaNs order above +inf.  out rows have stride out_stride.
+ * workspace: see td_topk_workspace_bytes (optional).
  * Replaces topk_filtering (bsk_ops.h:34-39, tidal/ops/csrc/topk.cu:7-44) and decode_select_k
  * (kernels/include/topk/decode_select_k.cuh:25-62; RAFT radix_topk_one_block_kernel).
  */
 int td_topk(const void* values, int32_t values_dtype, int64_t values_stride, int32_t rows,
             int32_t len, int32_t k, const int32_t* in_idx, int64_t in_idx_stride,
             const int32_t* page_table, int32_t page_size, void* out_values, int32_t* out_idx,
-            int64_t out_stride, void* stream);
+            int64_t out_stride, void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
+ * Bytes of device scratch that lets td_topk spread a row over several workgroups (rows of more
+ * than 8192 elements; two launches).  The scratch must be zero-filled once before its first use;
+ * every call leaves it ready for the next.  Without it (NULL) one workgroup handles each row.
+ * Plays the part of the `buf` argument of topk_filtering (tidal/utils/controller.py:164-168).
+ */
+int64_t td_topk_workspace_bytes(int32_t rows);
 
 /*
  * RMSNorm: out[r, :] = x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * weight, fp32 math.

@@ -11,14 +11,30 @@ import torch
 pytestmark = pytest.mark.gpu
 
 
-def _gpu_topk(values, k, cuda, in_idx=None, page_table=None, page_size=1, want_vals=True):
+_scratch = {}
+
+
+def _shared_scratch(cuda, rows):
+    """One scratch tensor for the whole module: zeroed at allocation only, so every cooperative
+    call after the first relies on the previous call having left it clean."""
+    from tidaldecode_amd import _kernels
+
+    need = _kernels.topk_workspace_bytes(64)
+    assert rows <= 64
+    if "buf" not in _scratch:
+        _scratch["buf"] = torch.zeros(need, dtype=torch.uint8, device=cuda)
+    return _scratch["buf"]
+
+
+def _gpu_topk(values, k, cuda, in_idx=None, page_table=None, page_size=1, want_vals=True,
+              scratch=False):
     from tidaldecode_amd import _kernels
 
     rows = values.shape[0]
     out_idx = torch.full((rows, k), -1, dtype=torch.int32, device=cuda)
     out_val = torch.zeros((rows, k), dtype=values.dtype, device=cuda) if want_vals else None
     _kernels.topk_filtering(values.to(cuda), None if in_idx is None else in_idx.to(cuda), out_val,
-                            out_idx, None, k,
+                            out_idx, _shared_scratch(cuda, rows) if scratch else None, k,
                             page_table=None if page_table is None else page_table.to(cuda),
                             page_size=page_size)
     torch.cuda.synchronize()
@@ -35,6 +51,10 @@ def _check(values, k, cuda):
     assert np.array_equal(got.numpy(), want_c)
     expect = torch.gather(values, 1, want)  # values travel with their index (NaN == NaN here)
     assert torch.equal(torch.nan_to_num(vals.float(), nan=1e38), torch.nan_to_num(expect.float(), nan=1e38))
+    # the several-workgroups-per-row path (taken for rows longer than 8192 when scratch is given)
+    got2, vals2 = _gpu_topk(values, k, cuda, scratch=True)
+    assert torch.equal(got2, got), "cooperative path differs"
+    assert torch.equal(torch.nan_to_num(vals2.float(), nan=1e38), torch.nan_to_num(vals.float(), nan=1e38))
     return got
 
 
@@ -64,6 +84,42 @@ def test_ties_go_to_the_lower_position(cuda):
     # all equal: the first k positions
     got = _check(torch.full((4, 5000), 1.25), 777, cuda)
     assert torch.equal(got, torch.arange(777, dtype=torch.int32).repeat(4, 1))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_long_rows_with_crowded_threshold_bins(cuda, dtype):
+    """Rows whose keys share their leading bits (more candidates than the cooperative kernel keeps
+    in LDS), rows of a single value, NaN-heavy rows and a length that is not a slice multiple."""
+    g = torch.Generator().manual_seed(11)
+    n = 40000 + 77
+    tight = (1.0 + torch.rand((3, n), generator=g) * 1e-3).to(dtype)      # one 11-bit bin
+    _check(tight, 2048, cuda)
+    _check(tight, n - 5, cuda)
+    tighter = (1.0 + torch.rand((2, n), generator=g) * 2e-7).to(dtype)    # 2-3 distinct fp32 keys
+    _check(tighter, 5000, cuda)
+    _check(torch.full((2, n), -3.5).to(dtype), 4097, cuda)
+    v = torch.randn((4, n), generator=g)
+    v[:, ::3] = float("nan")
+    v[1, 1::3] = float("inf")
+    v[2, :] = -v[2, :].abs()
+    _check(v.to(dtype), 20000, cuda)
+    _check(v.to(dtype), 1, cuda)
+    _check(v.to(dtype), n, cuda)
+
+
+def test_payloads_on_long_rows(cuda):
+    from oracle import tidal_oracle as orc
+
+    g = torch.Generator().manual_seed(5)
+    n, k, page = 50000, 3000, 16
+    v = torch.randn((4, n), generator=g)
+    want = orc.stable_topk(v, k)
+    in_idx = torch.randint(0, 1 << 30, (4, n), generator=g, dtype=torch.int32)
+    got, _ = _gpu_topk(v, k, cuda, in_idx=in_idx, scratch=True)
+    assert torch.equal(got.long(), torch.gather(in_idx.long(), 1, want))
+    table = torch.randperm((n + page - 1) // page, generator=g).int()
+    got, _ = _gpu_topk(v, k, cuda, page_table=table, page_size=page, scratch=True, want_vals=False)
+    assert torch.equal(got.long(), table.long()[want // page] * page + want % page)
 
 
 def test_signed_zero_inf_and_nan(cuda):

@@ -120,7 +120,10 @@ def topk_filtering(estimated_value: torch.Tensor, estimated_indices: Optional[to
                    page_table: Optional[torch.Tensor] = None, page_size: int = 1) -> None:
     """bsk_ops.h:34-39 / topk.cu:7-44.  Row-wise top-``page_budget`` of ``estimated_value``
     ``[H, len]``; ``indices_out[h, j]`` is ``estimated_indices[h, p]`` of the selected position
-    ``p``.  ``buf`` (RAFT scratch in the reference) is accepted and unused.
+    ``p``.  ``buf`` is scratch, as in the reference (there: RAFT's): a zero-initialised uint8 /
+    any-dtype device tensor of at least ``topk_workspace_bytes(H)`` bytes lets rows longer than
+    8192 elements be spread over several workgroups; smaller or ``None``: one workgroup per row.
+    The call leaves ``buf`` zeroed where it must be for the next call.
 
     Deterministic where the reference is not: ties at the threshold go to the lower position
     and each output row is sorted by position.  If ``estimated_indices`` has fewer columns than
@@ -162,11 +165,21 @@ def topk_filtering(estimated_value: torch.Tensor, estimated_indices: Optional[to
         if page_table.numel() * page_size < length:
             raise RuntimeError("page_table does not cover the row")
         pt_ptr = page_table.data_ptr()
+    ws_ptr, ws_bytes = None, 0
+    if buf is not None and buf.is_cuda and buf.is_contiguous():
+        ws_bytes = buf.numel() * buf.element_size()
+        if ws_bytes >= topk_workspace_bytes(rows):
+            ws_ptr = buf.data_ptr()
     check(lib.td_topk(estimated_value.data_ptr(),
                       _dtype_code(estimated_value.dtype, "Top-k filtering"),
                       estimated_value.stride(0), rows, length, k, in_ptr, in_stride, pt_ptr,
                       int(page_size), out_vals, indices_out.data_ptr(), indices_out.stride(0),
-                      _stream()))
+                      ws_ptr, ws_bytes if ws_ptr else 0, _stream()))
+
+
+def topk_workspace_bytes(rows: int) -> int:
+    """Bytes of zero-initialised scratch ``topk_filtering`` wants in ``buf`` for `rows` rows."""
+    return int(lib.td_topk_workspace_bytes(int(rows)))
 
 
 def estimate_attn_score(*args, **kwargs):

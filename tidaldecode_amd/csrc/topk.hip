@@ -1,7 +1,8 @@
 // Row-wise top-k selection and the cross-head score reduction for gfx950 (MI355X).
 //
 // One 1024-thread workgroup (16 wavefronts) per row (rows of up to 65536 elements are held in
-// registers, longer ones are re-read from L2 per pass) runs an MSB-first radix select over
+// registers, longer ones are re-read from L2 per pass; given scratch memory, rows of more than
+// 8192 elements are split over several workgroups, see topk_coop_select_kernel) runs an MSB-first radix select over
 // order-preserving integer keys with LDS histograms (11/11/10-bit digits for fp32 keys, 8/8 for
 // fp16/bf16 keys), which yields the exact k-th largest key T and the number r of elements equal
 // to T that still fit.  A final ordered pass emits every element above T plus the first r
@@ -28,10 +29,18 @@ struct TopkParams {
   int64_t in_idx_stride;
   const int32_t* page_table;
   int32_t page_size;
+  int32_t page_shift;  // log2(page_size) when it is a power of two, else -1
   void* out_values;
   int32_t* out_idx;
   int64_t out_stride;
 };
+
+// physical slot of position i through the page table
+__device__ __forceinline__ int32_t slot_of(const TopkParams& p, int i) {
+  if (p.page_shift >= 0)
+    return (p.page_table[i >> p.page_shift] << p.page_shift) | (i & (p.page_size - 1));
+  return p.page_table[i / p.page_size] * p.page_size + i % p.page_size;
+}
 
 struct F32 {};
 
@@ -205,7 +214,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_kernel(const TopkParams p) 
       if (p.in_idx)
         payload = p.in_idx[(int64_t)row * p.in_idx_stride + i];
       else if (p.page_table)
-        payload = p.page_table[i / p.page_size] * p.page_size + i % p.page_size;
+        payload = slot_of(p, i);
       else
         payload = i;
       out_idx[pos] = payload;
@@ -273,7 +282,8 @@ __global__ __launch_bounds__(kTopkThreads) void topk_reg_kernel(const TopkParams
 #pragma unroll
   for (int j = 0; j < IPT; ++j) {
     const int i = j * kTopkThreads + tid;
-    key[j] = i < len ? KT::key(vals[i]) : 0u;
+    const uint32_t kv = KT::key(vals[i < len ? i : len - 1]);  // unconditional load: all IPT in flight
+    key[j] = i < len ? kv : 0u;
   }
 
   uint32_t prefix = 0, mask = 0, krem = (uint32_t)k;
@@ -366,13 +376,409 @@ __global__ __launch_bounds__(kTopkThreads) void topk_reg_kernel(const TopkParams
       if (p.in_idx)
         payload = p.in_idx[(int64_t)row * p.in_idx_stride + i];
       else if (p.page_table)
-        payload = p.page_table[i / p.page_size] * p.page_size + i % p.page_size;
+        payload = slot_of(p, i);
       else
         payload = i;
       out_idx[pos] = payload;
       if (out_val) out_val[pos] = vals[i];
     }
   }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Cooperative variant: G workgroups per row, two launches.  One compute unit needs ~40 us to
+// push a 32K-element row through the single-workgroup kernels above (the row costs ~40K wave
+// instructions); with a handful of rows that leaves the other 200+ compute units idle.
+//
+//   launch 1 (topk_coop_select_kernel, grid G x rows): every workgroup histograms the top 11 key
+//     bits of its slice in LDS and adds the non-empty bins to a per-row global histogram; the last
+//     workgroup of a row to arrive (ticket) locates the threshold bin, re-reads the row once to
+//     gather that bin's candidates into LDS (counting, per slice, what lies above the bin),
+//     finishes the radix select on the candidates, and publishes the threshold key T, the number
+//     r of ties to take and per-slice output / tie offsets.
+//   launch 2 (topk_coop_emit_kernel, grid G x rows): every workgroup emits its slice in index
+//     order at its published offset.
+//
+// Scratch per row (uint32): [0,2048) histogram, 2048 ticket, 2049 T, 2050 r, then per slice
+// (out_before, eq_before).  The histogram and ticket must be zero before the first call; launch 1
+// leaves them zero again.  Values are keyed as fp32 whatever the input type.
+// ---------------------------------------------------------------------------------------------
+constexpr int kCoopIPT = 8;                       // keys per thread and slice
+constexpr int kCoopSlice = kCoopIPT * kTopkThreads;  // 8192 elements per workgroup
+constexpr int kCoopMaxSlices = 32;
+constexpr int kCoopBatch = 4;                     // slices per trip of the row pass
+constexpr int kCoopCand = 6144;                   // candidates kept in LDS
+constexpr int kCoopRowWords = 2048 + 3 + 2 * kCoopMaxSlices;
+
+template <typename T>
+__device__ __forceinline__ uint32_t coop_key(const void* base, int64_t i);
+template <>
+__device__ __forceinline__ uint32_t coop_key<F32>(const void* base, int64_t i) {
+  return KeyTraits<F32>::key(reinterpret_cast<const float*>(base)[i]);
+}
+template <>
+__device__ __forceinline__ uint32_t coop_key<F16>(const void* base, int64_t i) {
+  return KeyTraits<F32>::key(to_float<F16>(reinterpret_cast<const uint16_t*>(base)[i]));
+}
+template <>
+__device__ __forceinline__ uint32_t coop_key<BF16>(const void* base, int64_t i) {
+  return KeyTraits<F32>::key(to_float<BF16>(reinterpret_cast<const uint16_t*>(base)[i]));
+}
+
+// Workgroups are handed to the 8 XCDs round-robin by linear id.  All slices of a row go to one
+// XCD, so that what the row's workgroups read in the first phase is in the L2 that the row's
+// last workgroup (and the emit launch) reads again: linear id = (row / 8 * slices + slice) * 8 +
+// row % 8, grid = ceil(rows / 8) * slices * 8 workgroups; ids of rows past the end do nothing.
+constexpr int kXcds = 8;
+__device__ __forceinline__ bool coop_decode(int n_slices, int rows, int& slice, int& row) {
+  const int id = blockIdx.x;
+  const int t = id / kXcds;
+  row = t / n_slices * kXcds + id % kXcds;
+  slice = t % n_slices;
+  return row < rows;
+}
+
+template <typename T> struct ElemOf { typedef uint16_t type; };
+template <> struct ElemOf<F32> { typedef float type; };
+
+// lanes below this one whose bit is set in a wave-wide mask
+__device__ __forceinline__ uint32_t lanes_below(uint64_t m) {
+  return __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+}
+
+// One radix level over the candidates in LDS: histogram the `bits`-wide digit at `shift` of the
+// candidates whose key matches (mask, prefix); updates prefix / mask / krem.
+__device__ __forceinline__ void coop_level(const uint32_t* ckey, int n_cand, uint32_t* hist,
+                                           uint32_t* wave_tot, uint32_t* sh, int bits, int shift,
+                                           uint32_t& prefix, uint32_t& mask, uint32_t& krem, int tid,
+                                           int lane, int wave) {
+  const int nb = 1 << bits;
+  for (int i = tid; i < nb; i += kTopkThreads) hist[i] = 0;
+  __syncthreads();
+  for (int i = tid; i < n_cand; i += kTopkThreads) {
+    const uint32_t key = ckey[i];
+    if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & (nb - 1)], 1u);
+  }
+  __syncthreads();
+  const int bpt = nb >= kTopkThreads ? nb / kTopkThreads : 1;
+  const int my_bin = tid * bpt;
+  uint32_t local = 0;
+  if (my_bin < nb)
+    for (int j = 0; j < bpt; ++j) local += hist[my_bin + j];
+  const uint32_t suf = wave_suffix_sum(local, lane);
+  if (lane == 0) wave_tot[wave] = suf;
+  __syncthreads();
+  uint32_t above = suf - local;
+  for (int w = wave + 1; w < kTopkWaves; ++w) above += wave_tot[w];
+  if (my_bin < nb) {
+    for (int j = bpt - 1; j >= 0; --j) {
+      const uint32_t c = hist[my_bin + j];
+      if (above < krem && krem <= above + c) {
+        sh[0] = (uint32_t)(my_bin + j);
+        sh[1] = krem - above;
+      }
+      above += c;
+    }
+  }
+  __syncthreads();
+  prefix |= sh[0] << shift;
+  mask |= (uint32_t)(nb - 1) << shift;
+  krem = sh[1];
+  __syncthreads();
+}
+
+template <typename T>
+__global__ __launch_bounds__(kTopkThreads) void topk_coop_select_kernel(const TopkParams p,
+                                                                        uint32_t* scratch,
+                                                                        int n_slices, int rows) {
+  int slice, row;
+  if (!coop_decode(n_slices, rows, slice, row)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int len = p.len;
+  const void* vals = reinterpret_cast<const char*>(p.values) +
+                     (int64_t)row * p.values_stride * sizeof(typename ElemOf<T>::type);
+  uint32_t* rs = scratch + (int64_t)row * kCoopRowWords;
+
+  __shared__ uint32_t hist[2048];
+  __shared__ uint32_t wave_tot[kTopkWaves];
+  __shared__ uint32_t sh[4];
+  __shared__ uint32_t ckey[kCoopCand];
+  __shared__ int32_t cidx[kCoopCand];
+  __shared__ uint32_t slice_gt[kCoopMaxSlices], slice_eq[kCoopMaxSlices];
+  __shared__ uint32_t n_cand_sh;
+
+  // ---- phase 1: slice histogram of the top 11 bits -> global row histogram -------------------
+  for (int i = tid; i < 2048; i += kTopkThreads) hist[i] = 0;
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < kCoopIPT; ++j) {
+    const int i = slice * kCoopSlice + j * kTopkThreads + tid;
+    const uint32_t kv = coop_key<T>(vals, i < len ? i : len - 1);  // loads stay unconditional
+    if (i < len) atomicAdd(&hist[kv >> 21], 1u);
+  }
+  __syncthreads();
+  for (int i = tid; i < 2048; i += kTopkThreads) {
+    const uint32_t c = hist[i];
+    if (c) __hip_atomic_fetch_add(rs + i, c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this workgroup's additions are performed
+  __syncthreads();
+  if (tid == 0)
+    sh[2] = __hip_atomic_fetch_add(rs + 2048, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  if (sh[2] != (uint32_t)(n_slices - 1)) return;
+
+  // ---- phase 2 (last workgroup of the row): threshold bin of level 1 ------------------------
+  for (int i = tid; i < 2048; i += kTopkThreads) {
+    hist[i] = __hip_atomic_load(rs + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(rs + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  if (tid < kCoopMaxSlices) slice_gt[tid] = slice_eq[tid] = 0;
+  if (tid == 0) {
+    __hip_atomic_store(rs + 2048, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    n_cand_sh = 0;
+  }
+  __syncthreads();
+  uint32_t prefix = 0, mask = 0, krem = (uint32_t)p.k;
+  {
+    const int my_bin = tid * 2;
+    const uint32_t local = hist[my_bin] + hist[my_bin + 1];
+    const uint32_t suf = wave_suffix_sum(local, lane);
+    if (lane == 0) wave_tot[wave] = suf;
+    __syncthreads();
+    uint32_t above = suf - local;
+    for (int w = wave + 1; w < kTopkWaves; ++w) above += wave_tot[w];
+    for (int j = 1; j >= 0; --j) {
+      const uint32_t c = hist[my_bin + j];
+      if (above < krem && krem <= above + c) {
+        sh[0] = (uint32_t)(my_bin + j);
+        sh[1] = krem - above;
+        sh[3] = c;  // candidates in the threshold bin
+      }
+      above += c;
+    }
+    __syncthreads();
+    prefix = sh[0] << 21;
+    mask = 0x7ffu << 21;
+    krem = sh[1];
+  }
+  int n_in_bin = (int)sh[3];
+  __syncthreads();
+
+  // If the bin is too crowded for LDS, narrow it with streaming passes over the row
+  // (11 more bits, then 10): only pathological rows (most keys share 11 leading bits) get here.
+  int shift = 21;
+  while (n_in_bin > kCoopCand && shift > 0) {
+    const int bits = shift > 10 ? 11 : 10;
+    const int nb = 1 << bits;
+    shift -= bits;
+    for (int i = tid; i < nb; i += kTopkThreads) hist[i] = 0;
+    __syncthreads();
+    for (int i = tid; i < len; i += kTopkThreads) {
+      const uint32_t key = coop_key<T>(vals, i);
+      if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & (nb - 1)], 1u);
+    }
+    __syncthreads();
+    const int bpt = nb / kTopkThreads;  // 2 or 1
+    const int my_bin = tid * bpt;
+    uint32_t local = 0;
+    for (int j = 0; j < bpt; ++j) local += hist[my_bin + j];
+    const uint32_t suf = wave_suffix_sum(local, lane);
+    if (lane == 0) wave_tot[wave] = suf;
+    __syncthreads();
+    uint32_t above = suf - local;
+    for (int w = wave + 1; w < kTopkWaves; ++w) above += wave_tot[w];
+    for (int j = bpt - 1; j >= 0; --j) {
+      const uint32_t c = hist[my_bin + j];
+      if (above < krem && krem <= above + c) {
+        sh[0] = (uint32_t)(my_bin + j);
+        sh[1] = krem - above;
+        sh[3] = c;
+      }
+      above += c;
+    }
+    __syncthreads();
+    prefix |= sh[0] << shift;
+    mask |= (uint32_t)(nb - 1) << shift;
+    krem = sh[1];
+    n_in_bin = (int)sh[3];
+    __syncthreads();
+  }
+
+  // ---- phase 3: one pass over the row: count per slice what lies above the candidate range,
+  //      gather the candidates (keys matching the prefix) unless the range is a single key -------
+  const bool gather = shift > 0;  // shift == 0: all bits fixed, every candidate equals the threshold
+  // kCoopBatch slices per trip: a thread keeps 32 loads in flight, which is what it takes to
+  // cover the memory latency from one compute unit
+  for (int base0 = 0; base0 < len; base0 += kCoopBatch * kCoopSlice) {
+    uint32_t key[kCoopBatch][kCoopIPT];
+#pragma unroll
+    for (int s = 0; s < kCoopBatch; ++s)
+#pragma unroll
+      for (int j = 0; j < kCoopIPT; ++j) {
+        const int i = base0 + s * kCoopSlice + j * kTopkThreads + tid;
+        const uint32_t kv = coop_key<T>(vals, i < len ? i : len - 1);
+        key[s][j] = i < len ? kv : 0u;  // 0 lies below every real key
+      }
+#pragma unroll
+    for (int s = 0; s < kCoopBatch; ++s) {
+      const int base = base0 + s * kCoopSlice;
+      if (base >= len) break;
+      const int sl = base / kCoopSlice;
+      uint32_t n_above = 0, n_in = 0;
+      uint64_t cm[kCoopIPT];
+#pragma unroll
+      for (int j = 0; j < kCoopIPT; ++j) {
+        n_above += (uint32_t)__popcll(__ballot((key[s][j] & mask) > prefix));
+        cm[j] = __ballot(key[s][j] != 0u && (key[s][j] & mask) == prefix);
+        n_in += (uint32_t)__popcll(cm[j]);
+      }
+      if (gather && n_in) {  // wave-uniform: one LDS reservation per wave and slice
+        uint32_t at = 0;
+        if (lane == 0) at = atomicAdd(&n_cand_sh, n_in);
+        at = __shfl(at, 0, 64);
+#pragma unroll
+        for (int j = 0; j < kCoopIPT; ++j) {
+          const uint32_t mine = at + lanes_below(cm[j]);
+          if (((cm[j] >> lane) & 1ull) && mine < (uint32_t)kCoopCand) {
+            ckey[mine] = key[s][j];
+            cidx[mine] = base + j * kTopkThreads + tid;
+          }
+          at += (uint32_t)__popcll(cm[j]);
+        }
+      }
+      if (lane == 0) {
+        if (n_above) atomicAdd(&slice_gt[sl], n_above);
+        if (!gather && n_in) atomicAdd(&slice_eq[sl], n_in);
+      }
+    }
+  }
+  __syncthreads();
+  uint32_t thr = prefix, r = krem;
+  if (gather) {
+    const int n_cand = (int)n_cand_sh;  // == n_in_bin <= kCoopCand
+    // ---- phase 4: finish the radix select on the candidates ----------------------------------
+    while (shift > 0) {
+      const int bits = shift > 10 ? 11 : 10;
+      shift -= bits;
+      coop_level(ckey, n_cand, hist, wave_tot, sh, bits, shift, prefix, mask, krem, tid, lane, wave);
+    }
+    thr = prefix;
+    r = krem;
+    // ---- phase 5: candidates above / equal to T, per slice -----------------------------------
+    for (int base = 0; base < n_cand; base += kTopkThreads) {
+      const int i = base + tid;
+      const bool have = i < n_cand;
+      const uint32_t ck = have ? ckey[i] : 0u;
+      const int csl = have ? cidx[i] / kCoopSlice : -1;
+      for (int sl = 0; sl < n_slices; ++sl) {
+        const uint64_t gm = __ballot(csl == sl && ck > thr);
+        const uint64_t em = __ballot(csl == sl && ck == thr);
+        if (lane == 0) {
+          if (gm) atomicAdd(&slice_gt[sl], (uint32_t)__popcll(gm));
+          if (em) atomicAdd(&slice_eq[sl], (uint32_t)__popcll(em));
+        }
+      }
+    }
+    __syncthreads();
+  }
+  // ---- phase 6: publish T, r and the per-slice offsets ------------------------------------------
+  if (tid == 0) {
+    rs[2049] = thr;
+    rs[2050] = r;
+    uint32_t out_run = 0, eq_run = 0;
+    for (int sl = 0; sl < n_slices; ++sl) {
+      rs[2051 + 2 * sl] = out_run;
+      rs[2052 + 2 * sl] = eq_run;
+      const uint32_t e = slice_eq[sl];
+      const uint32_t room = r > eq_run ? r - eq_run : 0u;
+      out_run += slice_gt[sl] + (e < room ? e : room);
+      eq_run += e;
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kTopkThreads) void topk_coop_emit_kernel(const TopkParams p,
+                                                                      const uint32_t* scratch,
+                                                                      int n_slices, int rows) {
+  typedef typename ElemOf<T>::type elem_t;
+  int slice, row;
+  if (!coop_decode(n_slices, rows, slice, row)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int len = p.len;
+  const elem_t* vals = reinterpret_cast<const elem_t*>(p.values) + (int64_t)row * p.values_stride;
+  const uint32_t* rs = scratch + (int64_t)row * kCoopRowWords;
+  const uint32_t thr = rs[2049], r = rs[2050];
+  const uint32_t slice_out = rs[2051 + 2 * slice], slice_eq = rs[2052 + 2 * slice];
+
+  __shared__ uint32_t wave_tot[kTopkWaves];
+  __shared__ uint32_t run_eq[kCoopIPT * kTopkWaves], run_out[kCoopIPT * kTopkWaves];
+
+  uint32_t key[kCoopIPT];
+#pragma unroll
+  for (int j = 0; j < kCoopIPT; ++j) {
+    const int i = slice * kCoopSlice + j * kTopkThreads + tid;
+    const uint32_t kv = coop_key<T>(vals, i < len ? i : len - 1);
+    key[j] = i < len ? kv : 0u;  // 0 lies below every real key
+  }
+#pragma unroll
+  for (int j = 0; j < kCoopIPT; ++j) {
+    const uint32_t n_gt = (uint32_t)__popcll(__ballot(key[j] > thr));
+    const uint32_t n_eq = (uint32_t)__popcll(__ballot(key[j] == thr));
+    if (lane == 0) {
+      run_eq[j * kTopkWaves + wave] = n_eq;
+      run_out[j * kTopkWaves + wave] = n_gt;
+    }
+  }
+  __syncthreads();
+  {
+    const bool has = tid < kCoopIPT * kTopkWaves;
+    const uint32_t e = has ? run_eq[tid] : 0u;
+    const uint32_t g = has ? run_out[tid] : 0u;
+    uint32_t total;
+    const uint32_t eq_before = slice_eq + block_exclusive_sum(e, lane, wave, wave_tot, total);
+    const uint32_t room = r > eq_before ? r - eq_before : 0u;
+    const uint32_t take = e < room ? e : room;
+    const uint32_t out_before = slice_out + block_exclusive_sum(g + take, lane, wave, wave_tot, total);
+    if (has) {
+      run_eq[tid] = eq_before;
+      run_out[tid] = out_before;
+    }
+  }
+  __syncthreads();
+  int32_t* out_idx = p.out_idx + (int64_t)row * p.out_stride;
+  elem_t* out_val =
+      p.out_values ? reinterpret_cast<elem_t*>(p.out_values) + (int64_t)row * p.out_stride : nullptr;
+#pragma unroll
+  for (int j = 0; j < kCoopIPT; ++j) {
+    const bool gt = key[j] > thr;
+    const bool eq = key[j] == thr;
+    const uint64_t eq_mask = __ballot(eq);
+    const uint32_t eq_rank = run_eq[j * kTopkWaves + wave] + lanes_below(eq_mask);
+    const bool sel = gt || (eq && eq_rank < r);
+    const uint64_t sel_mask = __ballot(sel);
+    const uint32_t pos = run_out[j * kTopkWaves + wave] + lanes_below(sel_mask);
+    if (sel && pos < (uint32_t)p.k) {
+      const int i = slice * kCoopSlice + j * kTopkThreads + tid;
+      int32_t payload;
+      if (p.in_idx)
+        payload = p.in_idx[(int64_t)row * p.in_idx_stride + i];
+      else if (p.page_table)
+        payload = slot_of(p, i);
+      else
+        payload = i;
+      out_idx[pos] = payload;
+      if (out_val) out_val[pos] = vals[i];
+    }
+  }
+}
+
+// workgroups per row for the cooperative path, 0 if it does not apply
+static int coop_slices(int len, int rows) {
+  const int g = (len + kCoopSlice - 1) / kCoopSlice;
+  if (g < 2 || g > kCoopMaxSlices) return 0;  // short rows: one workgroup is as fast
+  return g;
 }
 
 template <typename T>
@@ -417,7 +823,8 @@ using namespace tidal;
 extern "C" int td_topk(const void* values, int32_t values_dtype, int64_t values_stride,
                        int32_t rows, int32_t len, int32_t k, const int32_t* in_idx,
                        int64_t in_idx_stride, const int32_t* page_table, int32_t page_size,
-                       void* out_values, int32_t* out_idx, int64_t out_stride, void* stream) {
+                       void* out_values, int32_t* out_idx, int64_t out_stride, void* workspace,
+                       int64_t workspace_bytes, void* stream) {
   TD_REQUIRE(values && out_idx, "td_topk: NULL values or out_idx");
   TD_REQUIRE(rows >= 1, "td_topk: rows %d < 1", rows);
   TD_REQUIRE(len >= 0 && k >= 0, "td_topk: len %d / k %d", len, k);
@@ -437,10 +844,30 @@ extern "C" int td_topk(const void* values, int32_t values_dtype, int64_t values_
   p.in_idx_stride = in_idx_stride;
   p.page_table = in_idx ? nullptr : page_table;
   p.page_size = page_size;
+  p.page_shift = -1;
+  if (page_size >= 1 && (page_size & (page_size - 1)) == 0) p.page_shift = __builtin_ctz(page_size);
   p.out_values = out_values;
   p.out_idx = out_idx;
   p.out_stride = out_stride;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const int slices = coop_slices(len, rows);
+  if (slices && workspace && workspace_bytes >= (int64_t)rows * kCoopRowWords * 4 &&
+      (values_dtype == TD_F32 || values_dtype == TD_F16 || values_dtype == TD_BF16)) {
+    uint32_t* ws = reinterpret_cast<uint32_t*>(workspace);
+    const dim3 grid((rows + kXcds - 1) / kXcds * slices * kXcds), block(kTopkThreads);
+    if (values_dtype == TD_F32) {
+      hipLaunchKernelGGL(topk_coop_select_kernel<F32>, grid, block, 0, st, p, ws, slices, rows);
+      hipLaunchKernelGGL(topk_coop_emit_kernel<F32>, grid, block, 0, st, p, ws, slices, rows);
+    } else if (values_dtype == TD_F16) {
+      hipLaunchKernelGGL(topk_coop_select_kernel<F16>, grid, block, 0, st, p, ws, slices, rows);
+      hipLaunchKernelGGL(topk_coop_emit_kernel<F16>, grid, block, 0, st, p, ws, slices, rows);
+    } else {
+      hipLaunchKernelGGL(topk_coop_select_kernel<BF16>, grid, block, 0, st, p, ws, slices, rows);
+      hipLaunchKernelGGL(topk_coop_emit_kernel<BF16>, grid, block, 0, st, p, ws, slices, rows);
+    }
+    TD_HIP_CHECK(hipGetLastError());
+    return TD_OK;
+  }
   switch (values_dtype) {
     case TD_F32: launch_topk<F32>(p, rows, st); break;
     case TD_F16: launch_topk<F16>(p, rows, st); break;
@@ -451,6 +878,10 @@ extern "C" int td_topk(const void* values, int32_t values_dtype, int64_t values_
   }
   TD_HIP_CHECK(hipGetLastError());
   return TD_OK;
+}
+
+extern "C" int64_t td_topk_workspace_bytes(int32_t rows) {
+  return (int64_t)(rows < 1 ? 1 : rows) * kCoopRowWords * 4;
 }
 
 extern "C" int td_score_reduce(const float* logits, int64_t logits_stride, const float* lse,

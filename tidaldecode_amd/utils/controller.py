@@ -92,7 +92,11 @@ class InferenceController:
                                                      dtype=torch.int32, device=device)
         self.topk_dindices_buffer = self.topk_dindices_buffer_full
         self.topk_dout_buffer = None  # selected values are not needed downstream
-        self.topk_buf = None          # RAFT scratch of the reference; unused
+        # scratch of the top-k kernels (the reference's RAFT buffer): zeroed once, kept zeroed
+        from .. import _kernels
+        self.topk_buf = torch.zeros(_kernels.topk_workspace_bytes(self.index_rows),
+                                    dtype=torch.uint8, device=device) \
+            if torch.device(device).type == "cuda" else None
         self.num_candidates = 0
         self.num_selected = 0
         self._indptr2 = torch.zeros(2, dtype=torch.int32, device=device)
