@@ -26,7 +26,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # HBM bytes one sparse-layer launch of the default workload moves, from rocprofv3 FETCH_SIZE /
 # WRITE_SIZE scaled by a plain 256 MiB copy (profiles/decode_attn_sparse_llama2-7b_ctx32k_top2048.md)
-TRAFFIC_DEFAULT_WORKLOAD = 35372816
+TRAFFIC_DEFAULT_WORKLOAD = 35333933
 
 
 def parse():
@@ -300,6 +300,15 @@ def main():
         sparse_ms = time_events(torch, r_sparse, max(args.steps, 20))
         entry = {"sparse_us_per_layer": sparse_ms * 1e3 / len(sparse), "launch": how,
                  "fused_rope_append": bool(w.fuse)}
+        if w.fuse:
+            # the attention launch alone (RoPE and append done elsewhere), for comparison
+            def run_sparse_plain():
+                for layer in sparse:
+                    w.sparse_attn(layer, None)
+
+            r_plain, _ = capture(torch, run_sparse_plain, use_graph)
+            entry["sparse_unfused_us_per_layer"] = (time_events(torch, r_plain, max(args.steps, 20))
+                                                    * 1e3 / len(sparse))
         if not args.only_sparse:
             def run_select():
                 for layer in w.sel_layers:
