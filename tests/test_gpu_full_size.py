@@ -1,0 +1,105 @@
+"""GPU parity at the full sizes of the benchmark configurations: one selection layer, the top-k
+selection and one sparse layer through the operator surface, against the CPU oracle.
+
+  cfg1  Llama-2-7B shape: 32/32 heads x 128, bf16, page 16, 32768 (+1) tokens, top_k 2048
+  cfg2  GQA 32/8, 102400 tokens, top_k 4096
+  cfg4  40/40 heads, 32768 tokens, top_k 2048
+
+The oracle's sparse layer gathers the selected rows (equal to the reference's masked dense form,
+pinned in tests/test_oracle.py), so it finishes in seconds at these sizes.  Index sets are
+compared bit-exact from the scores the GPU wrote; attention within 2e-3 (fp16) / 1e-2 (bf16).
+Size-independent properties on top: a permuted list gives the same output, and a list naming
+every token equals full attention.
+"""
+import pytest
+import torch
+
+from _util import ATOL, PagedCase, randn, tolerance_report
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("name,hq,hkv,n,k,mode,dtype", [
+    ("cfg1", 32, 32, 32769, 2048, "per_head", torch.bfloat16),
+    ("cfg1-head-sum", 32, 32, 32769, 2048, "head_sum", torch.bfloat16),
+    ("cfg2", 32, 8, 102400, 4096, "per_head", torch.bfloat16),
+    ("cfg2-group", 32, 8, 102400, 4096, "group_sum", torch.float16),
+    ("cfg4", 40, 40, 32768, 2048, "per_head", torch.float16),
+])
+def test_selection_topk_sparse_at_full_size(cuda, name, hq, hkv, n, k, mode, dtype):
+    from oracle import tidal_oracle as orc
+    from tidaldecode_amd import _kernels
+
+    d, page = 128, 16
+    case = PagedCase(n, hkv, d, page, dtype, seed=len(name) + n)
+    q_sel, q_sp = randn((hq, d), 5, dtype), randn((hq, d), 6, dtype)
+    pool = case.pool.to(cuda)
+    table = case.page_table.to(torch.int32).to(cuda)
+
+    w = _kernels.BatchDecodeWithPagedKVCachePyTorchWrapper(0)
+    w.begin_forward(None, hq, hkv, d, page, torch.empty(0, dtype=dtype))
+    stride = case.n_pages * page
+    scores = torch.zeros((hq, stride), dtype=torch.float32, device=cuda)
+    lse = torch.zeros((1, hq), dtype=torch.float32, device=cuda)
+    o_sel = torch.empty((1, hq, d), dtype=dtype, device=cuda)
+    w.forward(q_sel.to(dtype).to(cuda)[None], o_sel, pool, table[:-1][None].contiguous(), None,
+              case.last_page_len, int(table[-1]), scores, lse=lse)
+    rows = {"per_head": hq, "group_sum": hkv, "head_sum": 1}[mode]
+    sel_scores = scores if mode == "per_head" else _kernels.score_reduce(scores, lse.view(-1), hkv, n, mode)
+    scratch = torch.zeros(_kernels.topk_workspace_bytes(rows), dtype=torch.uint8, device=cuda)
+    slots = torch.empty((rows, k), dtype=torch.int32, device=cuda)
+    pos = torch.empty((rows, k), dtype=torch.int32, device=cuda)
+    _kernels.topk_filtering(sel_scores[:, :n], None, None, slots, scratch, k, page_table=table,
+                            page_size=page)
+    _kernels.topk_filtering(sel_scores[:, :n], None, None, pos, scratch, k)  # scratch left clean
+    o_sp = torch.empty((1, hq, d), dtype=dtype, device=cuda)
+    w.forward(q_sp.to(dtype).to(cuda)[None], o_sp, pool, slots, None, 0, 0, None, index_kind="slots")
+    torch.cuda.synchronize()
+
+    # selection layer: output and logits
+    logits = orc.attn_logits(q_sel, case.k)
+    assert tolerance_report(o_sel[0], orc.softmax_pv(logits, case.v)) <= ATOL[dtype]
+    if mode == "per_head":
+        assert (scores[:, :n].cpu() - logits).abs().max() <= 2e-4 * max(1.0, logits.abs().max().item())
+    # top-k: bit-exact from the same scores; slots are the positions seen through the page table
+    pos_c = pos.cpu().long()
+    assert torch.equal(pos_c, orc.stable_topk(sel_scores[:, :n].cpu(), k))
+    assert torch.equal(slots.cpu().long(), case.slots_of(pos_c))
+    # sparse layer
+    want = orc.sparse_layer_gather(q_sp, case.k, case.v, pos_c)
+    assert tolerance_report(o_sp[0], want) <= ATOL[dtype]
+
+    # a permuted list names the same set: same output up to the summation order
+    g = torch.Generator().manual_seed(1)
+    perm = torch.stack([torch.randperm(k, generator=g) for _ in range(rows)]).to(cuda)
+    o_perm = torch.empty_like(o_sp)
+    w.forward(q_sp.to(dtype).to(cuda)[None], o_perm, pool, torch.gather(slots, 1, perm).contiguous(),
+              None, 0, 0, None, index_kind="slots")
+    torch.cuda.synchronize()
+    assert tolerance_report(o_perm[0], want) <= ATOL[dtype]
+    assert tolerance_report(o_perm[0], o_sp[0]) <= ATOL[dtype] / 2
+
+
+def test_list_of_every_token_equals_full_attention(cuda):
+    """k = N at the benchmark length: the sparse path over all 32768 slots (shared list) equals
+    the selection-layer path over the page table."""
+    from oracle import tidal_oracle as orc
+    from tidaldecode_amd import _kernels
+
+    hq, hkv, d, page, n, dtype = 32, 32, 128, 16, 32768, torch.bfloat16
+    case = PagedCase(n, hkv, d, page, dtype, seed=9)
+    q = randn((hq, d), 8, dtype)
+    pool = case.pool.to(cuda)
+    w = _kernels.BatchDecodeWithPagedKVCachePyTorchWrapper(0)
+    w.begin_forward(None, hq, hkv, d, page, torch.empty(0, dtype=dtype))
+    qd = q.to(dtype).to(cuda)[None]
+    o_full, o_all = torch.empty_like(qd), torch.empty_like(qd)
+    table = case.page_table.to(torch.int32).to(cuda)
+    w.forward(qd, o_full, pool, table[:-1][None].contiguous(), None, case.last_page_len,
+              int(table[-1]), None)
+    slots = case.slots_of(torch.arange(n))[None].to(torch.int32).to(cuda)
+    w.forward(qd, o_all, pool, slots, None, 0, 0, None, index_kind="slots")
+    torch.cuda.synchronize()
+    want = orc.softmax_pv(orc.attn_logits(q, case.k), case.v)
+    assert tolerance_report(o_full[0], want) <= ATOL[dtype]
+    assert tolerance_report(o_all[0], want) <= ATOL[dtype]
