@@ -37,7 +37,10 @@ def parse():
     ap.add_argument("--ctx", type=int, default=32768)
     ap.add_argument("--top-k", type=int, default=2048)
     ap.add_argument("--layers", type=int, default=32)
-    ap.add_argument("--select-mode", default="per_head", choices=["per_head", "head_sum"])
+    ap.add_argument("--select-mode", default="per_head", choices=["per_head", "group_sum", "head_sum"])
+    ap.add_argument("--heads", type=int, default=32, help="query heads")
+    ap.add_argument("--kv-heads", type=int, default=32, help="KV heads")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16"])
     ap.add_argument("--waves", type=int, default=0, help="waves per workgroup (0 = default)")
     ap.add_argument("--chunk", type=int, default=0, help="tokens per workgroup (0 = default)")
     ap.add_argument("--merge", type=int, default=-1, help="1 fused / 0 second kernel / -1 default")
@@ -69,13 +72,14 @@ class Workload:
 
         self.torch = torch
         self.dev = torch.device("cuda:0")
-        self.L, self.H, self.D, self.P = args.layers, 32, 128, 16
+        self.L, self.H, self.D, self.P = args.layers, args.heads, 128, 16
+        self.HKV = args.kv_heads
         self.N, self.K = args.ctx, args.top_k
         self.sel_layers = (0, 2)
-        self.dtype = torch.bfloat16
+        self.dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float16
         c = InferenceController(self.L, self.H, self.D, self.P, self.K, self.N + 64, self.dtype,
-                                self.dev, select_mode=select_mode, page_order_seed=0,
-                                kv_layout=args.layout)
+                                self.dev, num_kv_heads=self.HKV, select_mode=select_mode,
+                                page_order_seed=0, kv_layout=args.layout)
         h = c._decode_handler._wrapper
         h.waves_per_block, h.chunk_tokens, h.fused_merge = args.waves, args.chunk, args.merge
         h.tile_rows = args.rows
@@ -85,10 +89,10 @@ class Workload:
         c.begin_forward(1)
         self.c = c
         g = torch.Generator(device=self.dev).manual_seed(0)
-        shape = (self.L, 1, self.H, self.D)
+        shape, kv_shape = (self.L, 1, self.H, self.D), (self.L, 1, self.HKV, self.D)
         self.q = torch.randn(shape, generator=g, device=self.dev).to(self.dtype)
-        self.k = torch.randn(shape, generator=g, device=self.dev).to(self.dtype)
-        self.v = torch.randn(shape, generator=g, device=self.dev).to(self.dtype)
+        self.k = torch.randn(kv_shape, generator=g, device=self.dev).to(self.dtype)
+        self.v = torch.randn(kv_shape, generator=g, device=self.dev).to(self.dtype)
         pos = c.kv_cache.seqlen - 1
         self.positions = torch.tensor([pos], dtype=torch.int32, device=self.dev)
         page = c.kv_cache.indicies[pos // self.P]
@@ -353,12 +357,13 @@ def main():
             entry["full_attention_ms_per_step"] = time_events(torch, r_full, 5, warm=1)
             entry["attention_ratio_vs_full"] = entry["ms_per_step"] / entry["full_attention_ms_per_step"]
         rows = w.c.index_rows
-        algo = (w.K * w.H * w.D * 2 * 2      # K and V rows of the attended tokens
+        gathered_heads = w.H if rows == w.H else w.HKV   # lists per query head gather per query head
+        algo = (w.K * gathered_heads * w.D * 2 * 2   # K and V rows of the attended tokens
                 + w.K * rows * 4             # the token list(s)
                 + 2 * w.H * w.D * 2)         # q in, o out
         entry["algorithmic_bytes"] = algo
         entry["achieved_gbs"] = algo / (entry["sparse_us_per_layer"] * 1e-6) / 1e9
-        sel_bytes = (w.c.kv_cache.seqlen * w.H * w.D * 2 * 2 + w.H * w.c.kv_cache.seqlen * 4
+        sel_bytes = (w.c.kv_cache.seqlen * w.HKV * w.D * 2 * 2 + w.H * w.c.kv_cache.seqlen * 4
                      + 2 * w.H * w.D * 2)
         if "selection_attn_us_per_layer" in entry:
             entry["selection_achieved_gbs"] = sel_bytes / (entry["selection_attn_us_per_layer"] * 1e-6) / 1e9
@@ -379,11 +384,11 @@ def main():
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16",
+        "dtype": args.dtype,
         "data": "synthetic",
         "config": {
-            "workload": f"llama2-7b-shape decode attention path: {args.layers} layers, 32/32 heads, "
-                        f"head_dim 128, paged bf16 KV page 16, ctx {args.ctx}, top_k {args.top_k}, "
+            "workload": f"llama2-7b-shape decode attention path: {args.layers} layers, {args.heads}/{args.kv_heads} heads, "
+                        f"head_dim 128, paged {args.dtype} KV page 16, ctx {args.ctx}, top_k {args.top_k}, "
                         f"selection at layers 0 and 2 ({main_mode} lists), batch 1",
             "select_mode": main_mode,
             "launch": e["launch"],
@@ -395,7 +400,8 @@ def main():
             "unit": "GB/s",
             "frac": round(e["achieved_gbs"] / HBM_PEAK_GBS, 4),
             "traffic": (TRAFFIC_DEFAULT_WORKLOAD
-                        if (args.ctx, args.top_k, args.layers, main_mode) == (32768, 2048, 32, "per_head")
+                        if (args.ctx, args.top_k, args.layers, main_mode, args.heads, args.kv_heads,
+                            args.dtype) == (32768, 2048, 32, "per_head", 32, 32, "bf16")
                         else None),
             "kernel": "decode_attn_kernel (sparse layer, token-slot lists)",
             "algorithmic_bytes_per_launch": e["algorithmic_bytes"],

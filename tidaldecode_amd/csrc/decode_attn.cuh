@@ -119,7 +119,7 @@ template <typename T, int D, int QPG, int NT>
 __device__ __forceinline__ void merge_splits(const DecodeParams& p, int b, int qh0, int n_splits) {
   constexpr int COLS = QPG * D / 2;
   constexpr int SLOTS = NT / COLS;
-  constexpr int PRE = 4;  // partial loads kept in flight per thread
+  constexpr int PRE = SLOTS >= 8 ? 4 : (SLOTS >= 4 ? 8 : 16);  // partial loads in flight per thread
   static_assert(SLOTS >= 1, "workgroup too small for the merge");
   __shared__ float mg_m[QPG][64], mg_l[QPG][64];
   __shared__ float mg_part[SLOTS][COLS][2];
@@ -135,13 +135,18 @@ __device__ __forceinline__ void merge_splits(const DecodeParams& p, int b, int q
     load_coherent(p.ws_ml + (((int64_t)b * p.num_qo_heads + qh0 + jj) * p.max_splits + ss) * 2,
                   ml_m, ml_l);
   }
+  // Loads are unconditional (index clamped, contribution zeroed) so that a batch of PRE of them
+  // is in flight per thread; a branch around a load makes the compiler wait for each one.
   float pa[PRE], pb[PRE];
+  auto issue = [&](int base) {
 #pragma unroll
-  for (int u = 0; u < PRE; ++u) {
-    const int sidx = slot + u * SLOTS;
-    pa[u] = pb[u] = 0.f;
-    if (slot < SLOTS && sidx < n_splits) load_coherent(p.ws_o + (part0 + sidx) * D + d2 * 2, pa[u], pb[u]);
-  }
+    for (int u = 0; u < PRE; ++u) {
+      int sidx = base + u * SLOTS;
+      sidx = sidx < n_splits ? sidx : n_splits - 1;
+      load_coherent(p.ws_o + (part0 + sidx) * D + d2 * 2, pa[u], pb[u]);
+    }
+  };
+  if (slot < SLOTS) issue(slot);
   if (has_ml) {
     mg_m[tid / n_splits][tid % n_splits] = ml_m;
     mg_l[tid / n_splits][tid % n_splits] = ml_l;
@@ -151,21 +156,17 @@ __device__ __forceinline__ void merge_splits(const DecodeParams& p, int b, int q
   for (int sidx = 0; sidx < n_splits; ++sidx) M = fmaxf(M, mg_m[j][sidx]);
   float ra = 0.f, rb = 0.f;
   if (slot < SLOTS) {
+    for (int base = slot; base < n_splits; base += PRE * SLOTS) {
+      if (base != slot) issue(base);
 #pragma unroll
-    for (int u = 0; u < PRE; ++u) {
-      const int sidx = slot + u * SLOTS;
-      if (sidx < n_splits) {
-        const float f = fast_exp2(mg_m[j][sidx] - M);
-        ra = fmaf(pa[u], f, ra);
-        rb = fmaf(pb[u], f, rb);
+      for (int u = 0; u < PRE; ++u) {
+        const int sidx = base + u * SLOTS;
+        const int sc = sidx < n_splits ? sidx : n_splits - 1;
+        const bool live = sidx < n_splits;
+        const float f = fast_exp2(mg_m[j][sc] - M);
+        ra = fmaf(live ? pa[u] : 0.f, f, ra);
+        rb = fmaf(live ? pb[u] : 0.f, f, rb);
       }
-    }
-    for (int sidx = slot + PRE * SLOTS; sidx < n_splits; sidx += SLOTS) {
-      float xa, xb;
-      load_coherent(p.ws_o + (part0 + sidx) * D + d2 * 2, xa, xb);
-      const float f = fast_exp2(mg_m[j][sidx] - M);
-      ra = fmaf(xa, f, ra);
-      rb = fmaf(xb, f, rb);
     }
     mg_part[slot][c][0] = ra;
     mg_part[slot][c][1] = rb;
@@ -523,34 +524,37 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
   }
 
   // ---- merge the NW wave states of the workgroup through LDS ------------------------------------
-  __shared__ float sm_o[NW][8][LPR];
-  __shared__ float sm_ml[NW][2];
+  // every wave publishes its QPG states, one barrier, then wave j reduces query head j
+  // (QPG <= NW; heads beyond the waves are handled by the waves again in a second trip)
+  __shared__ float sm_o[QPG][NW][8][LPR];
+  __shared__ float sm_ml[QPG][NW][2];
   __shared__ int sm_ticket;
+  if (lane < LPR) {
 #pragma unroll
-  for (int j = 0; j < QPG; ++j) {
-    if (j > 0) __syncthreads();
-    if (lane < LPR) {
+    for (int j = 0; j < QPG; ++j) {
 #pragma unroll
-      for (int d = 0; d < 8; ++d) sm_o[wave][d][lane] = acc[j][d];
+      for (int d = 0; d < 8; ++d) sm_o[j][wave][d][lane] = acc[j][d];
       if (lane == 0) {
-        sm_ml[wave][0] = m[j];
-        sm_ml[wave][1] = l[j];
+        sm_ml[j][wave][0] = m[j];
+        sm_ml[j][wave][1] = l[j];
       }
     }
-    __syncthreads();
-    if (wave == (j % NW) && lane < LPR) {
+  }
+  __syncthreads();
+  for (int j = wave; j < QPG; j += NW) {
+    if (lane < LPR) {
       float M = kNegBig;
 #pragma unroll
-      for (int w = 0; w < NW; ++w) M = fmaxf(M, sm_ml[w][0]);
+      for (int w = 0; w < NW; ++w) M = fmaxf(M, sm_ml[j][w][0]);
       float L = 0.f, r[8];
 #pragma unroll
       for (int d = 0; d < 8; ++d) r[d] = 0.f;
 #pragma unroll
       for (int w = 0; w < NW; ++w) {
-        const float f = fast_exp2(sm_ml[w][0] - M);
-        L = fmaf(sm_ml[w][1], f, L);
+        const float f = fast_exp2(sm_ml[j][w][0] - M);
+        L = fmaf(sm_ml[j][w][1], f, L);
 #pragma unroll
-        for (int d = 0; d < 8; ++d) r[d] = fmaf(sm_o[w][d][lane], f, r[d]);
+        for (int d = 0; d < 8; ++d) r[d] = fmaf(sm_o[j][w][d][lane], f, r[d]);
       }
       const int qh = qh0 + j;
       if (n_splits == 1) {
