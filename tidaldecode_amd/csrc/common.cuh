@@ -150,6 +150,82 @@ __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_lo
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
+// ---- pieces of the shared-KV-row (grouped-query) path ------------------------------------------
+// exchange with the lane whose index differs in one bit (inside a 16-lane DPP row)
+template <int MASK>
+__device__ __forceinline__ float lane_xor16(float x) {
+  static_assert(MASK == 1 || MASK == 2 || MASK == 4, "one of the low three bits");
+  if constexpr (MASK == 1) return dpp_move<0xB1>(x);   // quad_perm [1,0,3,2]
+  if constexpr (MASK == 2) return dpp_move<0x4E>(x);   // quad_perm [2,3,0,1]
+  // row_half_mirror gives lane i ^ 7, quad_perm [3,2,1,0] then gives (i ^ 7) ^ 3 = i ^ 4
+  return dpp_move<0x1B>(dpp_move<0x141>(x));
+}
+
+// a[j] holds this lane's partial sum for query head j (Q heads, Q = 2, 4 or 8).  Returns the
+// sum over the 16 lanes of the row for head (lane % Q): the first log2(Q) butterfly steps halve
+// the set of heads a lane keeps while exchanging the other half (reduce-scatter), the remaining
+// steps are plain sums among lanes that hold the same head.
+template <int Q>
+__device__ __forceinline__ float reduce_scatter16(float (&a)[Q], int li) {
+  static_assert(Q == 2 || Q == 4 || Q == 8, "query heads per shared row");
+  float cur[Q];
+#pragma unroll
+  for (int j = 0; j < Q; ++j) cur[j] = a[j];
+  if constexpr (Q >= 2) {
+    const bool hi = li & 1;
+#pragma unroll
+    for (int i = 0; i < Q / 2; ++i) {
+      const float keep = hi ? cur[2 * i + 1] : cur[2 * i];
+      const float send = hi ? cur[2 * i] : cur[2 * i + 1];
+      cur[i] = keep + lane_xor16<1>(send);
+    }
+  }
+  if constexpr (Q >= 4) {
+    const bool hi = li & 2;
+#pragma unroll
+    for (int i = 0; i < Q / 4; ++i) {
+      const float keep = hi ? cur[2 * i + 1] : cur[2 * i];
+      const float send = hi ? cur[2 * i] : cur[2 * i + 1];
+      cur[i] = keep + lane_xor16<2>(send);
+    }
+  } else {
+    cur[0] += lane_xor16<2>(cur[0]);
+  }
+  if constexpr (Q >= 8) {
+    const bool hi = li & 4;
+    const float keep = hi ? cur[1] : cur[0];
+    const float send = hi ? cur[0] : cur[1];
+    cur[0] = keep + lane_xor16<4>(send);
+  } else {
+    cur[0] += dpp_move<0x124>(cur[0]);  // row_ror:4 (sums need no exact partner, only the class)
+  }
+  cur[0] += dpp_move<0x128>(cur[0]);    // row_ror:8
+  return cur[0];
+}
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h16x4 __attribute__((ext_vector_type(4)));
+
+// D(16x16, fp32) += A(16x16) * B(16x16) with 16-bit operands: a lane holds A[lane % 16][4g .. 4g+3]
+// and B[4g .. 4g+3][lane % 16] (g = lane / 16) as two packed dwords, and D[4g + i][lane % 16].
+template <typename T>
+__device__ __forceinline__ f32x4 mfma_16x16x16(uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1,
+                                               f32x4 c);
+template <>
+__device__ __forceinline__ f32x4 mfma_16x16x16<BF16>(uint32_t a0, uint32_t a1, uint32_t b0,
+                                                     uint32_t b1, f32x4 c) {
+  const u32x2 a = {a0, a1}, b = {b0, b1};
+  return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, a),
+                                                   __builtin_bit_cast(s16x4, b), c, 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ f32x4 mfma_16x16x16<F16>(uint32_t a0, uint32_t a1, uint32_t b0,
+                                                    uint32_t b1, f32x4 c) {
+  const u32x2 a = {a0, a1}, b = {b0, b1};
+  return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(h16x4, a),
+                                               __builtin_bit_cast(h16x4, b), c, 0, 0, 0);
+}
+
 constexpr float kNegBig = -1.0e30f;  // finite stand-in for -inf in running maxima
 
 __host__ __device__ __forceinline__ int64_t ceil_div64(int64_t a, int64_t b) {

@@ -308,6 +308,16 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
     }
   };
 
+  // Shared-row path (QPG > 1): after the reduce-scatter of q.k a lane works on ONE query head,
+  // hsel = li % QPG; the running maximum mh of a head is kept equal in all lanes of the wave, lh
+  // is the lane group's share of the denominator, and p.V runs on the matrix cores with the 16
+  // tokens of a tile as the inner dimension: accm[dd][i] = o[head (4g + i) % QPG][li * 8 + dd].
+  static_assert(QPG == 1 || (U == 4 && TPI == 4), "shared-row tiles are 16 tokens: 4 rows x 4 groups");
+  float mh = kNegBig, lh = 0.f;
+  f32x4 accm[8];
+#pragma unroll
+  for (int d = 0; d < 8; ++d) accm[d] = f32x4{0.f, 0.f, 0.f, 0.f};
+
   float m[QPG], l[QPG], acc[QPG][8];
 #pragma unroll
   for (int j = 0; j < QPG; ++j) {
@@ -416,6 +426,86 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
         }
       }
     }
+    if constexpr (QPG > 1) {
+      float sv[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        float a[QPG];
+#pragma unroll
+        for (int j = 0; j < QPG; ++j) {
+          a[j] = dot2<T>(qp[j][0], kb[u].x, 0.f);
+          a[j] = dot2<T>(qp[j][1], kb[u].y, a[j]);
+          a[j] = dot2<T>(qp[j][2], kb[u].z, a[j]);
+          a[j] = dot2<T>(qp[j][3], kb[u].w, a[j]);
+        }
+        const float x = reduce_scatter16<QPG>(a, li) * p.scale_log2;  // head li % QPG
+        const int i = base + u * TPI + g;
+        const bool valid = i < c1;
+        if constexpr (EMIT) {
+          if (valid && li < QPG) {
+            const int64_t at = ((int64_t)b * p.num_qo_heads + qh0 + li) * p.score_stride + i;
+            const float nat = x * kLn2;
+            if (p.scores_f32)
+              reinterpret_cast<float*>(p.scores)[at] = nat;
+            else
+              reinterpret_cast<uint16_t*>(p.scores)[at] = from_float<T>(nat);
+          }
+        }
+        sv[u] = valid ? x : kNegBig;
+      }
+      float mt = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
+      mt = fmaxf(mt, __shfl_xor(mt, 16, 64));  // the tile's maximum over all four lane groups
+      mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+      const float m_new = fmaxf(mh, mt);
+      const float alpha = fast_exp2(mh - m_new);
+      mh = m_new;
+      float pr[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        pr[u] = (base + u * TPI + g < c1) ? fast_exp2(sv[u] - m_new) : 0.f;
+      // the probabilities enter the matrix product rounded to the KV type (zero-mean rounding of
+      // weights in [0, 1]); the denominator, which also gives the log-sum-exp, stays in fp32
+      const uint32_t p01 = pack2<T>(pr[0], pr[1]), p23 = pack2<T>(pr[2], pr[3]);
+      lh = fmaf(lh, alpha, (pr[0] + pr[1]) + (pr[2] + pr[3]));
+      // rescale the accumulators: row 4g + i belongs to head (4g + i) % QPG; the factors are
+      // wave-uniform per head (lane x < QPG holds head x), so they travel through SGPRs
+      float ah[QPG];
+      bool any = false;
+#pragma unroll
+      for (int x = 0; x < QPG; ++x) {
+        ah[x] = __builtin_bit_cast(
+            float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, alpha), x));
+        any |= ah[x] != 1.f;
+      }
+      if (any) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float f;
+          if constexpr (QPG == 8)
+            f = (g & 1) ? ah[4 + i] : ah[i];
+          else
+            f = ah[i % QPG];
+#pragma unroll
+          for (int d = 0; d < 8; ++d) accm[d][i] *= f;
+        }
+      }
+      // B operand of dimension dd: the four rows of the tile held by this lane, one 16-bit value
+      // each (v_perm picks the low or the high halves of two dwords)
+      const uint32_t vw[U][4] = {{vb[0].x, vb[0].y, vb[0].z, vb[0].w},
+                                 {vb[1].x, vb[1].y, vb[1].z, vb[1].w},
+                                 {vb[2].x, vb[2].y, vb[2].z, vb[2].w},
+                                 {vb[3].x, vb[3].y, vb[3].z, vb[3].w}};
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const uint32_t lo0 = __builtin_amdgcn_perm(vw[1][c], vw[0][c], 0x05040100u);
+        const uint32_t lo1 = __builtin_amdgcn_perm(vw[3][c], vw[2][c], 0x05040100u);
+        const uint32_t hi0 = __builtin_amdgcn_perm(vw[1][c], vw[0][c], 0x07060302u);
+        const uint32_t hi1 = __builtin_amdgcn_perm(vw[3][c], vw[2][c], 0x07060302u);
+        accm[2 * c] = mfma_16x16x16<T>(p01, p23, lo0, lo1, accm[2 * c]);
+        accm[2 * c + 1] = mfma_16x16x16<T>(p01, p23, hi0, hi1, accm[2 * c + 1]);
+      }
+      return;
+    }
     float sc[QPG][U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -505,8 +595,12 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
   }
 
   // ---- combine the TPI token slots of the wave (butterfly over lane groups) ---------------------
+  if constexpr (QPG > 1) {  // the matrix product already summed the groups; only lh is per group
+    lh += __shfl_xor(lh, 16, 64);
+    lh += __shfl_xor(lh, 32, 64);
+  }
 #pragma unroll
-  for (int j = 0; j < QPG; ++j) {
+  for (int j = 0; j < (QPG > 1 ? 0 : QPG); ++j) {
     float mw = m[j];
 #pragma unroll
     for (int off = LPR; off < 64; off <<= 1) mw = fmaxf(mw, __shfl_xor(mw, off, 64));
@@ -529,7 +623,19 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
   __shared__ float sm_o[QPG][NW][8][LPR];
   __shared__ float sm_ml[QPG][NW][2];
   __shared__ int sm_ticket;
-  if (lane < LPR) {
+  if constexpr (QPG > 1) {
+#pragma unroll
+    for (int j = 0; j < QPG; ++j) {  // head j is row j of the accumulator tile: group j / 4, i = j % 4
+      if (g == j / 4) {
+#pragma unroll
+        for (int d = 0; d < 8; ++d) sm_o[j][wave][d][li] = accm[d][j % 4];
+      }
+    }
+    if (lane < QPG) {
+      sm_ml[lane][wave][0] = mh;
+      sm_ml[lane][wave][1] = lh;
+    }
+  } else if (lane < LPR) {
 #pragma unroll
     for (int j = 0; j < QPG; ++j) {
 #pragma unroll
