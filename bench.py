@@ -234,8 +234,8 @@ def cpu_baseline(args, budget_s=20.0):
 
 
 def e2e_leg(args):
-    """End-to-end decode of a Llama-2-7B-shape decoder with random bf16 weights (torch GEMMs and
-    norms around the library's attention path), TidalDecode schedule vs. the same decoder with
+    """End-to-end decode of a Llama-2-7B-shape decoder with random bf16 weights (the library's
+    fused matrix-vector launches around its attention path), TidalDecode schedule vs. the same decoder with
     full attention in every layer, at each context length.  One decode step at that context is
     captured as a hipGraph and replayed (steady-state per-token latency; the cache holds
     synthetic N(0,1) data)."""
@@ -261,6 +261,15 @@ def e2e_leg(args):
             row[f"{kind}_tokens_per_s"] = round(1.0 / dt, 2)
             row["launch"] = how
         row["speedup_vs_full_attention"] = round(row["full_ms_per_token"] / row["tidal_ms_per_token"], 3)
+        # the same TidalDecode step with torch's GEMMs and element-wise kernels around attention
+        cfg.attn_type = "tidal"
+        model.use_gemv = False
+        model.tidal_clear()
+        model.synthetic_prefill(ctx)
+        dt, _ = model.timed_decode(steps=max(10, args.steps // 2), warmup=3,
+                                   use_graph=not args.no_graph)
+        model.use_gemv = True
+        row["tidal_torch_linear_ms_per_token"] = round(dt * 1e3, 4)
         out[str(ctx)] = row
     del model
     torch.cuda.empty_cache()

@@ -71,12 +71,15 @@ def _close(got, want, rel=3e-2):
     return (got.float() - want).abs().max().item() <= rel * scale
 
 
+@pytest.mark.parametrize("use_gemv", [True, False])
 @pytest.mark.parametrize("select_mode", ["per_head", "head_sum"])
-def test_budget_covering_the_context_equals_dense_attention(cuda, select_mode):
+def test_budget_covering_the_context_equals_dense_attention(cuda, select_mode, use_gemv):
+    """use_gemv: the fused matrix-vector launches of the library; otherwise torch GEMMs"""
     from tidaldecode_amd.llama import TidalLlama
 
     torch.manual_seed(0)
     model = TidalLlama(_small(select_mode=select_mode), cuda, seed=1, init_std=0.05)
+    model.use_gemv = use_gemv
     model.tidal_init(page_size=16, max_seq_len=256, page_order_seed=3)
     ids = torch.randint(0, 1000, (70,), device=cuda)
     logits = model.prefill(ids)

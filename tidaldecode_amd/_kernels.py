@@ -114,6 +114,44 @@ def rms_norm_forward(input: torch.Tensor, weight: torch.Tensor, output: torch.Te
                           _dtype_code(input.dtype, "rms_norm_forward"), _stream()))
 
 
+def gemv(weight: torch.Tensor, x: torch.Tensor, *, norm_weight: Optional[torch.Tensor] = None,
+         eps: float = 1e-5, gated: bool = False, residual: Optional[torch.Tensor] = None,
+         out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Extension for the batch-1 decode driver: ``y = weight @ f(x) (+ residual)`` in one launch.
+
+    ``weight [rows, cols]`` (an ``nn.Linear`` weight, rows may be strided), ``x`` one token.
+    ``norm_weight``: ``f(x) = RMSNorm(x, eps) * norm_weight``; ``gated``: ``x`` holds
+    ``[gate | up]`` (2 cols) and ``f(x) = silu(gate) * up``; otherwise ``f(x) = x``.
+    ``residual`` (may be ``out``) is added to the product.  Returns ``out`` (``[rows]``)."""
+    _check_input(x, "x")
+    if not weight.is_cuda or weight.dim() != 2 or weight.stride(1) != 1:
+        raise RuntimeError("gemv: weight must be a CUDA matrix with contiguous rows")
+    rows, cols = weight.shape
+    if weight.dtype != x.dtype or x.numel() != (2 * cols if gated else cols):
+        raise RuntimeError("gemv: x does not fit the weight")
+    if norm_weight is not None and gated:
+        raise RuntimeError("gemv: norm_weight and gated exclude each other")
+    if norm_weight is not None:
+        _check_input(norm_weight, "norm_weight")
+        if norm_weight.numel() != cols or norm_weight.dtype != x.dtype:
+            raise RuntimeError("gemv: norm_weight does not fit")
+    if out is None:
+        out = torch.empty(rows, dtype=x.dtype, device=x.device)
+    _check_input(out, "out")
+    if out.numel() != rows or out.dtype != x.dtype:
+        raise RuntimeError("gemv: out does not fit")
+    if residual is not None:
+        _check_input(residual, "residual")
+        if residual.numel() != rows or residual.dtype != x.dtype:
+            raise RuntimeError("gemv: residual does not fit")
+    mode = 1 if norm_weight is not None else (2 if gated else 0)
+    check(lib.td_gemv(weight.data_ptr(), weight.stride(0), rows, cols, x.data_ptr(), mode,
+                      None if norm_weight is None else norm_weight.data_ptr(), float(eps),
+                      None if residual is None else residual.data_ptr(), out.data_ptr(),
+                      _dtype_code(x.dtype, "gemv"), _stream()))
+    return out
+
+
 def topk_filtering(estimated_value: torch.Tensor, estimated_indices: Optional[torch.Tensor],
                    d_out: Optional[torch.Tensor], indices_out: torch.Tensor,
                    buf: Optional[torch.Tensor], page_budget: int, *,

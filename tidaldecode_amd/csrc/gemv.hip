@@ -1,0 +1,189 @@
+// Matrix-vector products of a batch-1 decode step for gfx950 (MI355X): y = W x with a row-major
+// 16-bit W, fp32 accumulation, and the element-wise work around it folded in:
+//   x_mode 0  x as given
+//   x_mode 1  x = RMSNorm(x) * norm_weight            (the norm before the q/k/v and MLP products)
+//   x_mode 2  x = silu(x[:cols]) * x[cols:]           (the gated MLP, before the down projection)
+//   residual  y = residual + W x                      (the two residual additions of a layer)
+// HBM-bound: every weight is read once (non-temporal 16-byte loads, 16 of them in flight per
+// lane), x is staged in LDS once per workgroup, a wavefront owns two rows at a time and reduces
+// with DPP.  Used by the decoder harness around the attention path (the reference runs torch
+// nn.Linear there: tidal/models/SparseAttention.py:122,216, tidal/models/llama.py:108-122).
+
+#include "common.cuh"
+
+namespace tidal {
+
+constexpr int kGemvThreads = 256;
+constexpr int kGemvWaves = kGemvThreads / 64;
+constexpr int kGemvRows = 2;        // rows per wave and trip
+constexpr int kGemvUnroll = 8;      // 16-byte chunks per lane, row and trip
+constexpr int kGemvMaxCols = 16384; // x in LDS: 32 KiB
+
+struct GemvParams {
+  const uint16_t* w;
+  int64_t w_row_stride;  // elements
+  int32_t rows, cols;
+  const uint16_t* x;
+  const uint16_t* norm_weight;
+  float eps;
+  const uint16_t* residual;
+  uint16_t* y;
+};
+
+__device__ __forceinline__ float wave_sum64(float x) {
+  x = group_sum<16>(x);
+  x += __shfl_xor(x, 16, 64);
+  x += __shfl_xor(x, 32, 64);
+  return x;
+}
+
+template <typename T, int MODE>
+__global__ __launch_bounds__(kGemvThreads) void gemv_kernel(const GemvParams p) {
+  __shared__ uint32_t xs[kGemvMaxCols / 2];
+  __shared__ float red[kGemvWaves];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int cols = p.cols;
+  const int chunks = cols / 8;
+
+  // ---- stage x (and what is folded into it) in LDS, as packed 16-bit pairs ----------------------
+  if constexpr (MODE == 0) {
+    for (int c = tid; c < chunks; c += kGemvThreads)
+      reinterpret_cast<u32x4*>(xs)[c] = reinterpret_cast<const u32x4*>(p.x)[c];
+  } else if constexpr (MODE == 1) {
+    // RMSNorm as the model computes it: fp32 statistics, the normalised value rounded to the
+    // storage type, then the weight applied in the storage type
+    float ss = 0.f;
+    for (int c = tid; c < chunks; c += kGemvThreads) {
+      const u32x4 v = reinterpret_cast<const u32x4*>(p.x)[c];
+      reinterpret_cast<u32x4*>(xs)[c] = v;
+      float a, b;
+      unpack2<T>(v.x, a, b); ss = fmaf(a, a, fmaf(b, b, ss));
+      unpack2<T>(v.y, a, b); ss = fmaf(a, a, fmaf(b, b, ss));
+      unpack2<T>(v.z, a, b); ss = fmaf(a, a, fmaf(b, b, ss));
+      unpack2<T>(v.w, a, b); ss = fmaf(a, a, fmaf(b, b, ss));
+    }
+    ss = wave_sum64(ss);
+    if (lane == 0) red[wave] = ss;
+    __syncthreads();
+    float tot = 0.f;
+#pragma unroll
+    for (int w = 0; w < kGemvWaves; ++w) tot += red[w];
+    const float inv = rsqrtf(tot / (float)cols + p.eps);
+    // (the barrier above also ordered the staging stores before these reads of other threads' dwords)
+    for (int c = tid; c < cols / 2; c += kGemvThreads) {
+      float a, b, wa, wb;
+      unpack2<T>(xs[c], a, b);
+      unpack2<T>(reinterpret_cast<const uint32_t*>(p.norm_weight)[c], wa, wb);
+      float na, nb;
+      unpack2<T>(pack2<T>(a * inv, b * inv), na, nb);
+      xs[c] = pack2<T>(na * wa, nb * wb);
+    }
+  } else {
+    // gated MLP input: silu(gate) rounded to the storage type, times up, rounded again
+    for (int c = tid; c < cols / 2; c += kGemvThreads) {
+      float ga, gb, ua, ub;
+      unpack2<T>(reinterpret_cast<const uint32_t*>(p.x)[c], ga, gb);
+      unpack2<T>(reinterpret_cast<const uint32_t*>(p.x + cols)[c], ua, ub);
+      float sa, sb;
+      unpack2<T>(pack2<T>(ga / (1.f + __expf(-ga)), gb / (1.f + __expf(-gb))), sa, sb);
+      xs[c] = pack2<T>(sa * ua, sb * ub);
+    }
+  }
+  __syncthreads();
+
+  // ---- rows ---------------------------------------------------------------------------------------
+  const int row0 = (blockIdx.x * kGemvWaves + wave) * kGemvRows;
+  if (row0 >= p.rows) return;
+  float acc[kGemvRows];
+#pragma unroll
+  for (int r = 0; r < kGemvRows; ++r) acc[r] = 0.f;
+  const u32x4* wrow[kGemvRows];
+#pragma unroll
+  for (int r = 0; r < kGemvRows; ++r) {
+    const int row = row0 + r < p.rows ? row0 + r : p.rows - 1;  // a clamped row is computed, not stored
+    wrow[r] = reinterpret_cast<const u32x4*>(p.w + (int64_t)row * p.w_row_stride);
+  }
+  for (int c0 = 0; c0 < chunks; c0 += 64 * kGemvUnroll) {
+    u32x4 wv[kGemvRows][kGemvUnroll];
+#pragma unroll
+    for (int u = 0; u < kGemvUnroll; ++u) {
+      const int c = c0 + u * 64 + lane;
+      const int cc = c < chunks ? c : chunks - 1;  // unconditional loads; masked below
+#pragma unroll
+      for (int r = 0; r < kGemvRows; ++r) wv[r][u] = __builtin_nontemporal_load(wrow[r] + cc);
+    }
+#pragma unroll
+    for (int u = 0; u < kGemvUnroll; ++u) {
+      const int c = c0 + u * 64 + lane;
+      const int cc = c < chunks ? c : chunks - 1;
+      u32x4 xv = reinterpret_cast<const u32x4*>(xs)[cc];
+      if (c >= chunks) xv = u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int r = 0; r < kGemvRows; ++r) {
+        acc[r] = dot2<T>(wv[r][u].x, xv.x, acc[r]);
+        acc[r] = dot2<T>(wv[r][u].y, xv.y, acc[r]);
+        acc[r] = dot2<T>(wv[r][u].z, xv.z, acc[r]);
+        acc[r] = dot2<T>(wv[r][u].w, xv.w, acc[r]);
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < kGemvRows; ++r) {
+    const float s = wave_sum64(acc[r]);
+    const int row = row0 + r;
+    if (lane == 0 && row < p.rows) {
+      float out = s;
+      if (p.residual) out += to_float<T>(p.residual[row]);
+      p.y[row] = from_float<T>(out);
+    }
+  }
+}
+
+template <typename T>
+static void launch_gemv(const GemvParams& p, int mode, hipStream_t st) {
+  const int rows_per_block = kGemvWaves * kGemvRows;
+  const dim3 grid((p.rows + rows_per_block - 1) / rows_per_block), block(kGemvThreads);
+  if (mode == 0)
+    hipLaunchKernelGGL((gemv_kernel<T, 0>), grid, block, 0, st, p);
+  else if (mode == 1)
+    hipLaunchKernelGGL((gemv_kernel<T, 1>), grid, block, 0, st, p);
+  else
+    hipLaunchKernelGGL((gemv_kernel<T, 2>), grid, block, 0, st, p);
+}
+
+}  // namespace tidal
+
+using namespace tidal;
+
+extern "C" int td_gemv(const void* w, int64_t w_row_stride, int32_t rows, int32_t cols,
+                       const void* x, int32_t x_mode, const void* norm_weight, float eps,
+                       const void* residual, void* y, int32_t dtype, void* stream) {
+  TD_REQUIRE(w && x && y, "td_gemv: NULL argument");
+  TD_REQUIRE(rows >= 1 && cols >= 8 && cols % 8 == 0 && cols <= kGemvMaxCols,
+             "td_gemv: rows %d, cols %d (cols: multiple of 8, at most %d)", rows, cols, kGemvMaxCols);
+  TD_REQUIRE(w_row_stride >= cols && w_row_stride % 8 == 0,
+             "td_gemv: row stride %lld (multiple of 8, at least cols)", (long long)w_row_stride);
+  TD_REQUIRE(x_mode >= 0 && x_mode <= 2, "td_gemv: x_mode %d", x_mode);
+  TD_REQUIRE(x_mode != 1 || norm_weight, "td_gemv: x_mode 1 needs norm_weight");
+  TD_REQUIRE((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(x)) % 16 == 0,
+             "td_gemv: w and x must be 16-byte aligned");
+  GemvParams p;
+  p.w = reinterpret_cast<const uint16_t*>(w);
+  p.w_row_stride = w_row_stride;
+  p.rows = rows;
+  p.cols = cols;
+  p.x = reinterpret_cast<const uint16_t*>(x);
+  p.norm_weight = reinterpret_cast<const uint16_t*>(norm_weight);
+  p.eps = eps;
+  p.residual = reinterpret_cast<const uint16_t*>(residual);
+  p.y = reinterpret_cast<uint16_t*>(y);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (dtype == TD_F16)
+    launch_gemv<F16>(p, x_mode, st);
+  else if (dtype == TD_BF16)
+    launch_gemv<BF16>(p, x_mode, st);
+  else
+    return fail(TD_ERR_UNSUPPORTED, "td_gemv failed to dispatch with dtype %d", dtype);
+  TD_HIP_CHECK(hipGetLastError());
+  return TD_OK;
+}

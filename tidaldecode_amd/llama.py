@@ -91,6 +91,9 @@ class TidalLlama:
         self._cos = torch.zeros((1, c.head_dim // 2), dtype=torch.float32, device=self.device)
         self._sin = torch.zeros((1, c.head_dim // 2), dtype=torch.float32, device=self.device)
         self.fuse_decode_step = True  # RoPE + append inside the attention launch when possible
+        # batch-1 decode: one launch per projection with the norm / gate / residual folded in
+        # (False: torch GEMMs and separate element-wise kernels, as the reference's driver)
+        self.use_gemv = True
 
     # ----- cache lifecycle (tidal/models/llama.py:616-656) -----------------------------------
     def tidal_init(self, page_size: int, max_seq_len: int, token_budget: Optional[int] = None,
@@ -175,29 +178,49 @@ class TidalLlama:
         _kernels.rope_table(self._positions, self.config.head_dim, self.config.rope_scale,
                             self.config.rope_theta, self._cos, self._sin)
 
+    def _attention(self, idx, q, k, v):
+        """attention of one decode step for layer idx; q [1, H, D], k/v [1, H_kv, D] un-rotated"""
+        c, ctrl = self.config, self.iController
+        fresh = None
+        if self.fuse_decode_step and ctrl.fused_step_ok:
+            fresh = (k, v, self._cos, self._sin, self._dst_slot)
+        else:
+            tidal_utils.rope_append_kv(q, k, v, ctrl, idx, self._positions, self._dst_slot,
+                                       c.rope_scale, c.rope_theta)
+        kind = c.layer_kind(idx)
+        if kind == "sparse":
+            return tidal_utils.decode_sparse_attn(q, ctrl, idx, ctrl.topk_dindices_buffer, False,
+                                                  fresh=fresh)
+        o = tidal_utils.decode_sparse_attn(q, ctrl, idx, ctrl.kv_indices_without_last,
+                                           kind == "select", fresh=fresh)
+        if kind == "select":
+            tidal_utils.decode_topk(ctrl)
+        return o
+
     @torch.no_grad()
     def decode_layers(self, x: torch.Tensor) -> torch.Tensor:
         """The layer loop of one decode step on hidden state x [1, hidden]; device work only (safe
         to capture in a hipGraph once begin_decode_step has run)."""
-        c, ctrl = self.config, self.iController
+        c = self.config
+        if self.use_gemv:
+            eps = c.rms_norm_eps
+            q_end = c.num_heads * c.head_dim
+            k_end = q_end + c.num_kv_heads * c.head_dim
+            h = x.reshape(-1).clone()  # residual stream, updated in place by the projections
+            for idx, layer in enumerate(self.layers):
+                qkv = _kernels.gemv(layer["wqkv"], h, norm_weight=layer["ln1"], eps=eps)
+                q = qkv[:q_end].view(1, c.num_heads, c.head_dim)
+                k = qkv[q_end:k_end].view(1, c.num_kv_heads, c.head_dim)
+                v = qkv[k_end:].view(1, c.num_kv_heads, c.head_dim)
+                o = self._attention(idx, q, k, v)
+                _kernels.gemv(layer["wo"], o.view(-1), residual=h, out=h)
+                gu = _kernels.gemv(layer["w_gate_up"], h, norm_weight=layer["ln2"], eps=eps)
+                _kernels.gemv(layer["w_down"], gu, gated=True, residual=h, out=h)
+            return _kernels.gemv(self.lm_head, h, norm_weight=self.norm, eps=eps).view(1, -1)
         for idx, layer in enumerate(self.layers):
-            h = self._rms(x, layer["ln1"])
-            q, k, v = self._qkv(layer, h)
-            fresh = None
-            if self.fuse_decode_step and ctrl.fused_step_ok:
-                fresh = (k, v, self._cos, self._sin, self._dst_slot)
-            else:
-                tidal_utils.rope_append_kv(q, k, v, ctrl, idx, self._positions, self._dst_slot,
-                                           c.rope_scale, c.rope_theta)
-            kind = c.layer_kind(idx)
-            if kind == "sparse":
-                o = tidal_utils.decode_sparse_attn(q, ctrl, idx, ctrl.topk_dindices_buffer, False,
-                                                   fresh=fresh)
-            else:
-                o = tidal_utils.decode_sparse_attn(q, ctrl, idx, ctrl.kv_indices_without_last,
-                                                   kind == "select", fresh=fresh)
-                if kind == "select":
-                    tidal_utils.decode_topk(ctrl)
+            hn = self._rms(x, layer["ln1"])
+            q, k, v = self._qkv(layer, hn)
+            o = self._attention(idx, q, k, v)
             x = x + o.reshape(1, -1) @ layer["wo"].t()
             x = x + self._mlp(layer, self._rms(x, layer["ln2"]))
         return self._rms(x, self.norm) @ self.lm_head.t()
