@@ -268,14 +268,16 @@ int td_rms_norm(const void* x, const void* weight, void* out, int32_t rows, int3
  * Matrix-vector product of a batch-1 decode step: y[rows] = W[rows, cols] . f(x) (+ residual),
  * 16-bit storage, fp32 accumulation.  x_mode 0: f(x) = x[cols]; 1: f(x) = RMSNorm(x) * norm_weight
  * (eps); 2: f(x) = silu(x[:cols]) * x[cols:2 cols] (gated MLP).  residual (or NULL) is added to
- * the result and may alias y.  cols: multiple of 8, at most 16384; w and x 16-byte aligned.
+ * the result and may alias y.  pair_gated != 0: rows is even and y has rows/2 entries,
+ * y[i] = silu(W[i] . f(x)) * (W[i + rows/2] . f(x)) (gate and up projections stacked in W).
+ * cols: multiple of 8, at most 16384; w and x 16-byte aligned.
  * Serves the decoder harness around the attention path, where the reference calls torch's
  * nn.Linear, LlamaRMSNorm and act_fn one by one (tidal/models/SparseAttention.py:122-124,216,
  * tidal/models/llama.py:99,108-122,563-578).
  */
 int td_gemv(const void* w, int64_t w_row_stride, int32_t rows, int32_t cols, const void* x,
-            int32_t x_mode, const void* norm_weight, float eps, const void* residual, void* y,
-            int32_t dtype, void* stream);
+            int32_t x_mode, const void* norm_weight, float eps, const void* residual,
+            int32_t pair_gated, void* y, int32_t dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -57,6 +57,25 @@ def test_gemv_matches_fp32_reference(cuda, dtype, rows, cols, mode, with_residua
     assert (err <= bound).all(), float((err / bound).max())
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,cols", [(22016, 4096), (28672, 4096), (6, 64)])
+def test_gemv_gate_up_pairs(cuda, dtype, rows, cols):
+    """stacked gate/up projection with the activation in the epilogue == the two-launch form"""
+    from tidaldecode_amd import _kernels
+
+    g = torch.Generator(device=cuda).manual_seed(rows + cols)
+    w = (torch.randn((rows, cols), generator=g, device=cuda) * 0.05).to(dtype)
+    x = torch.randn(cols, generator=g, device=cuda).to(dtype)
+    nw = (1 + 0.1 * torch.randn(cols, generator=g, device=cuda)).to(dtype)
+    act = _kernels.gemv(w, x, norm_weight=nw, eps=1e-5, pair_gated=True)
+    gu = _kernels.gemv(w, x, norm_weight=nw, eps=1e-5)          # [gate | up], rounded
+    torch.cuda.synchronize()
+    assert act.shape == (rows // 2,)
+    want = (torch.nn.functional.silu(gu[: rows // 2].float()).to(dtype) * gu[rows // 2:])
+    # same roundings; the fast exponential may flip the last bit of silu
+    assert ((act.float() - want.float()).abs() <= 2 * EPS_OF[dtype] * want.float().abs() + 1e-6).all()
+
+
 def test_gemv_on_a_row_slice_of_a_fused_weight(cuda):
     """rows of a larger matrix (a q/k/v block of a fused projection): the row stride is honoured"""
     from tidaldecode_amd import _kernels

@@ -116,13 +116,15 @@ def rms_norm_forward(input: torch.Tensor, weight: torch.Tensor, output: torch.Te
 
 def gemv(weight: torch.Tensor, x: torch.Tensor, *, norm_weight: Optional[torch.Tensor] = None,
          eps: float = 1e-5, gated: bool = False, residual: Optional[torch.Tensor] = None,
-         out: Optional[torch.Tensor] = None) -> torch.Tensor:
+         pair_gated: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Extension for the batch-1 decode driver: ``y = weight @ f(x) (+ residual)`` in one launch.
 
     ``weight [rows, cols]`` (an ``nn.Linear`` weight, rows may be strided), ``x`` one token.
     ``norm_weight``: ``f(x) = RMSNorm(x, eps) * norm_weight``; ``gated``: ``x`` holds
     ``[gate | up]`` (2 cols) and ``f(x) = silu(gate) * up``; otherwise ``f(x) = x``.
-    ``residual`` (may be ``out``) is added to the product.  Returns ``out`` (``[rows]``)."""
+    ``residual`` (may be ``out``) is added to the product.  ``pair_gated``: ``weight`` stacks the
+    gate and the up projection and ``out[i] = silu(weight[i] . f(x)) * (weight[i + rows/2] . f(x))``
+    (``rows/2`` values).  Returns ``out``."""
     _check_input(x, "x")
     if not weight.is_cuda or weight.dim() != 2 or weight.stride(1) != 1:
         raise RuntimeError("gemv: weight must be a CUDA matrix with contiguous rows")
@@ -135,10 +137,13 @@ def gemv(weight: torch.Tensor, x: torch.Tensor, *, norm_weight: Optional[torch.T
         _check_input(norm_weight, "norm_weight")
         if norm_weight.numel() != cols or norm_weight.dtype != x.dtype:
             raise RuntimeError("gemv: norm_weight does not fit")
+    n_out = rows // 2 if pair_gated else rows
+    if pair_gated and (rows % 2 or gated or residual is not None):
+        raise RuntimeError("gemv: pair_gated needs an even row count, no gated input, no residual")
     if out is None:
-        out = torch.empty(rows, dtype=x.dtype, device=x.device)
+        out = torch.empty(n_out, dtype=x.dtype, device=x.device)
     _check_input(out, "out")
-    if out.numel() != rows or out.dtype != x.dtype:
+    if out.numel() != n_out or out.dtype != x.dtype:
         raise RuntimeError("gemv: out does not fit")
     if residual is not None:
         _check_input(residual, "residual")
@@ -147,8 +152,8 @@ def gemv(weight: torch.Tensor, x: torch.Tensor, *, norm_weight: Optional[torch.T
     mode = 1 if norm_weight is not None else (2 if gated else 0)
     check(lib.td_gemv(weight.data_ptr(), weight.stride(0), rows, cols, x.data_ptr(), mode,
                       None if norm_weight is None else norm_weight.data_ptr(), float(eps),
-                      None if residual is None else residual.data_ptr(), out.data_ptr(),
-                      _dtype_code(x.dtype, "gemv"), _stream()))
+                      None if residual is None else residual.data_ptr(), int(pair_gated),
+                      out.data_ptr(), _dtype_code(x.dtype, "gemv"), _stream()))
     return out
 
 

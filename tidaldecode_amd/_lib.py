@@ -122,7 +122,7 @@ SIGNATURES = {
     "td_gemv": (
         c_int32,
         [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_int32, c_void_p, c_float, c_void_p,
-         c_void_p, c_int32, c_void_p],
+         c_int32, c_void_p, c_int32, c_void_p],
     ),
     "td_rms_norm": (
         c_int32,

@@ -4,6 +4,8 @@
 //   x_mode 1  x = RMSNorm(x) * norm_weight            (the norm before the q/k/v and MLP products)
 //   x_mode 2  x = silu(x[:cols]) * x[cols:]           (the gated MLP, before the down projection)
 //   residual  y = residual + W x                      (the two residual additions of a layer)
+//   pair      y[i] = silu(W[i] x) * (W[i + rows/2] x) (gate and up projection in one launch: a
+//             wavefront owns row i and row i + rows/2, so the down projection gets a plain vector)
 // HBM-bound: every weight is read once (non-temporal 16-byte loads, 16 of them in flight per
 // lane), x is staged in LDS once per workgroup, a wavefront owns two rows at a time and reduces
 // with DPP.  Used by the decoder harness around the attention path (the reference runs torch
@@ -37,7 +39,7 @@ __device__ __forceinline__ float wave_sum64(float x) {
   return x;
 }
 
-template <typename T, int MODE>
+template <typename T, int MODE, bool PAIR>
 __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(const GemvParams p) {
   __shared__ uint32_t xs[kGemvMaxCols / 2];
   __shared__ float red[kGemvWaves];
@@ -92,15 +94,20 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(const GemvParams p) 
   __syncthreads();
 
   // ---- rows ---------------------------------------------------------------------------------------
-  const int row0 = (blockIdx.x * kGemvWaves + wave) * kGemvRows;
-  if (row0 >= p.rows) return;
+  const int half = p.rows / 2;
+  const int unit = blockIdx.x * kGemvWaves + wave;  // two consecutive rows, or a gate/up row pair
+  const int n_units = PAIR ? half : (p.rows + kGemvRows - 1) / kGemvRows;
+  if (unit >= n_units) return;
+  int row_of[kGemvRows];
+  row_of[0] = PAIR ? unit : unit * kGemvRows;
+  row_of[1] = PAIR ? unit + half : unit * kGemvRows + 1;
   float acc[kGemvRows];
 #pragma unroll
   for (int r = 0; r < kGemvRows; ++r) acc[r] = 0.f;
   const u32x4* wrow[kGemvRows];
 #pragma unroll
   for (int r = 0; r < kGemvRows; ++r) {
-    const int row = row0 + r < p.rows ? row0 + r : p.rows - 1;  // a clamped row is computed, not stored
+    const int row = row_of[r] < p.rows ? row_of[r] : p.rows - 1;  // a clamped row is computed, not stored
     wrow[r] = reinterpret_cast<const u32x4*>(p.w + (int64_t)row * p.w_row_stride);
   }
   for (int c0 = 0; c0 < chunks; c0 += 64 * kGemvUnroll) {
@@ -127,28 +134,44 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(const GemvParams p) 
       }
     }
   }
+  float sum[kGemvRows];
 #pragma unroll
-  for (int r = 0; r < kGemvRows; ++r) {
-    const float s = wave_sum64(acc[r]);
-    const int row = row0 + r;
-    if (lane == 0 && row < p.rows) {
-      float out = s;
-      if (p.residual) out += to_float<T>(p.residual[row]);
-      p.y[row] = from_float<T>(out);
+  for (int r = 0; r < kGemvRows; ++r) sum[r] = wave_sum64(acc[r]);
+  if (lane != 0) return;
+  if constexpr (PAIR) {
+    // as the model does it: both products, silu(gate) and the product each rounded to the storage type
+    const float gte = to_float<T>(from_float<T>(sum[0]));
+    const float up = to_float<T>(from_float<T>(sum[1]));
+    const float act = to_float<T>(from_float<T>(gte / (1.f + __expf(-gte))));
+    p.y[unit] = from_float<T>(act * up);
+  } else {
+#pragma unroll
+    for (int r = 0; r < kGemvRows; ++r) {
+      if (row_of[r] < p.rows) {
+        float out = sum[r];
+        if (p.residual) out += to_float<T>(p.residual[row_of[r]]);
+        p.y[row_of[r]] = from_float<T>(out);
+      }
     }
   }
 }
 
 template <typename T>
-static void launch_gemv(const GemvParams& p, int mode, hipStream_t st) {
-  const int rows_per_block = kGemvWaves * kGemvRows;
-  const dim3 grid((p.rows + rows_per_block - 1) / rows_per_block), block(kGemvThreads);
-  if (mode == 0)
-    hipLaunchKernelGGL((gemv_kernel<T, 0>), grid, block, 0, st, p);
-  else if (mode == 1)
-    hipLaunchKernelGGL((gemv_kernel<T, 1>), grid, block, 0, st, p);
-  else
-    hipLaunchKernelGGL((gemv_kernel<T, 2>), grid, block, 0, st, p);
+static void launch_gemv(const GemvParams& p, int mode, bool pair, hipStream_t st) {
+  const int units = pair ? p.rows / 2 : (p.rows + kGemvRows - 1) / kGemvRows;
+  const dim3 grid((units + kGemvWaves - 1) / kGemvWaves), block(kGemvThreads);
+  if (pair) {
+    if (mode == 0)
+      hipLaunchKernelGGL((gemv_kernel<T, 0, true>), grid, block, 0, st, p);
+    else
+      hipLaunchKernelGGL((gemv_kernel<T, 1, true>), grid, block, 0, st, p);
+  } else if (mode == 0) {
+    hipLaunchKernelGGL((gemv_kernel<T, 0, false>), grid, block, 0, st, p);
+  } else if (mode == 1) {
+    hipLaunchKernelGGL((gemv_kernel<T, 1, false>), grid, block, 0, st, p);
+  } else {
+    hipLaunchKernelGGL((gemv_kernel<T, 2, false>), grid, block, 0, st, p);
+  }
 }
 
 }  // namespace tidal
@@ -157,7 +180,8 @@ using namespace tidal;
 
 extern "C" int td_gemv(const void* w, int64_t w_row_stride, int32_t rows, int32_t cols,
                        const void* x, int32_t x_mode, const void* norm_weight, float eps,
-                       const void* residual, void* y, int32_t dtype, void* stream) {
+                       const void* residual, int32_t pair_gated, void* y, int32_t dtype,
+                       void* stream) {
   TD_REQUIRE(w && x && y, "td_gemv: NULL argument");
   TD_REQUIRE(rows >= 1 && cols >= 8 && cols % 8 == 0 && cols <= kGemvMaxCols,
              "td_gemv: rows %d, cols %d (cols: multiple of 8, at most %d)", rows, cols, kGemvMaxCols);
@@ -165,6 +189,8 @@ extern "C" int td_gemv(const void* w, int64_t w_row_stride, int32_t rows, int32_
              "td_gemv: row stride %lld (multiple of 8, at least cols)", (long long)w_row_stride);
   TD_REQUIRE(x_mode >= 0 && x_mode <= 2, "td_gemv: x_mode %d", x_mode);
   TD_REQUIRE(x_mode != 1 || norm_weight, "td_gemv: x_mode 1 needs norm_weight");
+  TD_REQUIRE(!pair_gated || (rows % 2 == 0 && x_mode != 2 && !residual),
+             "td_gemv: pair_gated needs an even row count, x_mode 0 or 1 and no residual");
   TD_REQUIRE((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(x)) % 16 == 0,
              "td_gemv: w and x must be 16-byte aligned");
   GemvParams p;
@@ -179,9 +205,9 @@ extern "C" int td_gemv(const void* w, int64_t w_row_stride, int32_t rows, int32_
   p.y = reinterpret_cast<uint16_t*>(y);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   if (dtype == TD_F16)
-    launch_gemv<F16>(p, x_mode, st);
+    launch_gemv<F16>(p, x_mode, pair_gated != 0, st);
   else if (dtype == TD_BF16)
-    launch_gemv<BF16>(p, x_mode, st);
+    launch_gemv<BF16>(p, x_mode, pair_gated != 0, st);
   else
     return fail(TD_ERR_UNSUPPORTED, "td_gemv failed to dispatch with dtype %d", dtype);
   TD_HIP_CHECK(hipGetLastError());

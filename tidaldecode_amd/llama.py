@@ -214,8 +214,9 @@ class TidalLlama:
                 v = qkv[k_end:].view(1, c.num_kv_heads, c.head_dim)
                 o = self._attention(idx, q, k, v)
                 _kernels.gemv(layer["wo"], o.view(-1), residual=h, out=h)
-                gu = _kernels.gemv(layer["w_gate_up"], h, norm_weight=layer["ln2"], eps=eps)
-                _kernels.gemv(layer["w_down"], gu, gated=True, residual=h, out=h)
+                act = _kernels.gemv(layer["w_gate_up"], h, norm_weight=layer["ln2"], eps=eps,
+                                    pair_gated=True)
+                _kernels.gemv(layer["w_down"], act, residual=h, out=h)
             return _kernels.gemv(self.lm_head, h, norm_weight=self.norm, eps=eps).view(1, -1)
         for idx, layer in enumerate(self.layers):
             hn = self._rms(x, layer["ln1"])
