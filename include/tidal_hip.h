@@ -265,6 +265,17 @@ int td_rms_norm(const void* x, const void* weight, void* out, int32_t rows, int3
                 float eps, int32_t dtype, void* stream);
 
 /*
+ * Prefill: attention of the n_q newest tokens of one sequence (q, o: [n_q, num_qo_heads, head_dim])
+ * over its kv_len cached tokens, whose pages are page_table[0 .. n_pages) in order (K/V of the
+ * new tokens already appended).  causal != 0: query row i sees positions <= kv_len - n_q + i.
+ * head_dim 64 or 128, fp16 / bf16.  Replaces prefill_with_paged_kv_cache (bsk_ops.h:80-88,
+ * tidal/ops/csrc/batch_prefill.cu:27-117, kernels/include/prefill/prefill.cuh:674-870).
+ */
+int td_prefill_attn(const td_paged_kv* kv, const int32_t* page_table, int32_t n_pages,
+                    int32_t kv_len, const void* q, void* o, int32_t n_q, int32_t num_qo_heads,
+                    float sm_scale, int32_t causal, void* stream);
+
+/*
  * Matrix-vector product of a batch-1 decode step: y[rows] = W[rows, cols] . f(x) (+ residual),
  * 16-bit storage, fp32 accumulation.  x_mode 0: f(x) = x[cols]; 1: f(x) = RMSNorm(x) * norm_weight
  * (eps); 2: f(x) = silu(x[:cols]) * x[cols:2 cols] (gated MLP).  residual (or NULL) is added to

@@ -119,6 +119,11 @@ SIGNATURES = {
          c_int32, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p],
     ),
     "td_topk_workspace_bytes": (c_int64, [c_int32]),
+    "td_prefill_attn": (
+        c_int32,
+        [POINTER(PagedKV), c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_int32, c_int32,
+         c_float, c_int32, c_void_p],
+    ),
     "td_gemv": (
         c_int32,
         [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_int32, c_void_p, c_float, c_void_p,

@@ -1,0 +1,325 @@
+// Causal attention of the n_q newest tokens of a sequence over its paged KV cache (prefill) for
+// gfx950 (MI355X), on the matrix cores.  Replaces BatchPrefillWithPagedKVCache of the reference
+// (kernels/include/prefill/prefill.cuh:674-870, bound in tidal/ops/csrc/batch_prefill.cu:27-117).
+//
+// One 256-thread workgroup per (128 query rows, query head); a wavefront owns 32 query rows as
+// two 16-row tiles.  The loop walks the keys in tiles of 64 tokens that the workgroup stages once
+// in LDS (rows padded to 272 bytes: conflict-free 16-byte reads) while the global loads of the
+// next tile are already in flight.  Per 16 tokens and query tile:
+//   S^T = K Q^T   mfma_f32_16x16x16, A = K rows from LDS, B = Q rows kept in registers; the head
+//                 dimension is walked in a permuted order (the same for Q and K), so that every
+//                 operand is a 16-byte piece of a row;
+//   softmax       base-2, online; the result tile has the query row in lane % 16 and four
+//                 tokens per lane, which is the A-operand layout of the next product;
+//   O += P V      A = P (rounded to the KV type), B = V: a lane reads the rows of its four tokens
+//                 (16 bytes each) and re-packs them with v_perm into one operand per dimension.
+// Pages are looked up per staged row; rows past the end of the sequence are clamped (never
+// out of the pool) and masked.
+
+#include "common.cuh"
+#include "../../include/tidal_hip.h"
+
+namespace tidal {
+
+constexpr int kPfThreads = 256;
+constexpr int kPfBM = 128;  // query rows per workgroup
+constexpr int kPfBN = 64;   // tokens per key tile
+
+struct PrefillParams {
+  const uint16_t* kv;
+  int64_t page_stride, v_offset;  // elements
+  int32_t entry_stride, head_stride, page_size, page_shift;
+  uint32_t max_page;
+  const int32_t* page_table;
+  int32_t n_pages, kv_len;
+  const uint16_t* q;
+  uint16_t* o;
+  int32_t n_q, num_qo_heads, q_per_kv;
+  float scale_log2;
+  int32_t causal;
+};
+
+template <typename T, int D>
+__global__ __launch_bounds__(kPfThreads) void prefill_attn_kernel(const PrefillParams p) {
+  constexpr int NS = D / 32;        // 16-byte pieces of a Q/K row per lane (two MFMA k-steps each)
+  constexpr int DC = D / 16;        // head dimensions per lane in the P.V product
+  constexpr int PITCH = D + 8;      // LDS row pitch in elements: +16 bytes
+  constexpr int CPR = D / 8;        // 16-byte chunks per row
+  constexpr int CPT = kPfBN * CPR / kPfThreads;  // chunks a thread stages per tile and matrix
+  static_assert(D == 64 || D == 128, "head dimensions of the prefill kernel");
+  __shared__ __attribute__((aligned(16))) uint16_t ks[kPfBN * PITCH];
+  __shared__ __attribute__((aligned(16))) uint16_t vs[kPfBN * PITCH];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int qtile = gridDim.x - 1 - blockIdx.x;  // longest rows first
+  const int qh = blockIdx.y;
+  const int kvh = qh / p.q_per_kv;
+  const int q0 = qtile * kPfBM;
+  const int q_off = p.kv_len - p.n_q;  // position of query row 0
+
+  // ---- Q operands: row (q0 + 32 wave + 16 mt + r), pieces [32 s + 8 g, +8) ----------------------
+  u32x4 qb[2][NS];
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt) {
+    int row = q0 + wave * 32 + mt * 16 + r;
+    row = row < p.n_q ? row : p.n_q - 1;
+    const u32x4* src =
+        reinterpret_cast<const u32x4*>(p.q + ((int64_t)row * p.num_qo_heads + qh) * D);
+#pragma unroll
+    for (int s = 0; s < NS; ++s) qb[mt][s] = src[4 * s + g];
+  }
+
+  f32x4 oacc[2][DC];
+  float m_run[2], l_run[2];
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt) {
+    m_run[mt] = kNegBig;
+    l_run[mt] = 0.f;
+#pragma unroll
+    for (int d = 0; d < DC; ++d) oacc[mt][d] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  // keys this workgroup needs: up to the position of its last query row
+  int last_row = q0 + kPfBM - 1;
+  last_row = last_row < p.n_q ? last_row : p.n_q - 1;
+  const int kv_end = p.causal ? (q_off + last_row + 1) : p.kv_len;
+
+  // ---- staging: thread -> CPT chunks of K and of V per tile --------------------------------------
+  u32x4 kreg[CPT], vreg[CPT];
+  auto fetch = [&](int kt) {
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) {
+      const int c = tid + j * kPfThreads;
+      const int row = c / CPR, cc = c % CPR;
+      int tok = kt + row;
+      tok = tok < p.kv_len ? tok : p.kv_len - 1;
+      int pg_i, entry;
+      if (p.page_shift >= 0) {
+        pg_i = tok >> p.page_shift;
+        entry = tok & (p.page_size - 1);
+      } else {
+        pg_i = tok / p.page_size;
+        entry = tok - pg_i * p.page_size;
+      }
+      uint32_t page = (uint32_t)p.page_table[pg_i];
+      page = page > p.max_page ? p.max_page : page;
+      const int64_t off = (int64_t)page * p.page_stride + (int64_t)entry * p.entry_stride +
+                          (int64_t)kvh * p.head_stride + cc * 8;
+      kreg[j] = *reinterpret_cast<const u32x4*>(p.kv + off);
+      vreg[j] = *reinterpret_cast<const u32x4*>(p.kv + off + p.v_offset);
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) {
+      const int c = tid + j * kPfThreads;
+      const int row = c / CPR, cc = c % CPR;
+      *reinterpret_cast<u32x4*>(&ks[row * PITCH + cc * 8]) = kreg[j];
+      *reinterpret_cast<u32x4*>(&vs[row * PITCH + cc * 8]) = vreg[j];
+    }
+  };
+
+  const int wave_first_pos = q_off + q0 + wave * 32;  // position of the wave's first query row
+  fetch(0);
+  stash();
+  __syncthreads();
+  for (int kt = 0; kt < kv_end; kt += kPfBN) {
+    const bool more = kt + kPfBN < kv_end;
+    if (more) fetch(kt + kPfBN);
+    // tiles entirely behind the causal frontier of this wave contribute nothing
+    const bool wave_active = !p.causal || kt <= wave_first_pos + 31;
+    if (wave_active) {
+      const bool need_mask = (p.causal && kt + kPfBN - 1 > wave_first_pos) || kt + kPfBN > p.kv_len;
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) {
+        const int qpos = wave_first_pos + mt * 16 + r;  // position of this lane's query row
+        // ---- S^T for the four 16-token sub-tiles ---------------------------------------------------
+        f32x4 st[4];
+#pragma unroll
+        for (int sub = 0; sub < 4; ++sub) {
+          f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+          const uint16_t* krow = &ks[(sub * 16 + r) * PITCH + 8 * g];
+#pragma unroll
+          for (int s = 0; s < NS; ++s) {
+            const u32x4 ka = *reinterpret_cast<const u32x4*>(krow + 32 * s);
+            acc = mfma_16x16x16<T>(ka.x, ka.y, qb[mt][s].x, qb[mt][s].y, acc);
+            acc = mfma_16x16x16<T>(ka.z, ka.w, qb[mt][s].z, qb[mt][s].w, acc);
+          }
+          st[sub] = acc * p.scale_log2;
+        }
+        if (need_mask) {
+#pragma unroll
+          for (int sub = 0; sub < 4; ++sub)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int tpos = kt + sub * 16 + 4 * g + i;
+              const bool ok = tpos < p.kv_len && (!p.causal || tpos <= qpos);
+              st[sub][i] = ok ? st[sub][i] : kNegBig;
+            }
+        }
+        // ---- online softmax of query row r (lanes r, r+16, r+32, r+48 share the row) ---------------
+        float mt_max = kNegBig;
+#pragma unroll
+        for (int sub = 0; sub < 4; ++sub)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) mt_max = fmaxf(mt_max, st[sub][i]);
+        mt_max = fmaxf(mt_max, __shfl_xor(mt_max, 16, 64));
+        mt_max = fmaxf(mt_max, __shfl_xor(mt_max, 32, 64));
+        const float m_new = fmaxf(m_run[mt], mt_max);
+        const float alpha = fast_exp2(m_run[mt] - m_new);
+        m_run[mt] = m_new;
+        float psum = 0.f;
+        uint32_t pa[4][2];
+#pragma unroll
+        for (int sub = 0; sub < 4; ++sub) {
+          float pr[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            pr[i] = st[sub][i] > 0.5f * kNegBig ? fast_exp2(st[sub][i] - m_new) : 0.f;
+            psum += pr[i];
+          }
+          pa[sub][0] = pack2<T>(pr[0], pr[1]);
+          pa[sub][1] = pack2<T>(pr[2], pr[3]);
+        }
+        l_run[mt] = fmaf(l_run[mt], alpha, psum);
+        // rescale: accumulator row 4g + i is query row 4g + i, whose factor sits in lane 4g + i
+        if (__ballot(alpha != 1.f)) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float f = __shfl(alpha, 4 * g + i, 64);
+#pragma unroll
+            for (int d = 0; d < DC; ++d) oacc[mt][d][i] *= f;
+          }
+        }
+        // ---- O += P V ---------------------------------------------------------------------------------
+#pragma unroll
+        for (int sub = 0; sub < 4; ++sub) {
+          uint32_t vw[4][DC / 2];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const uint16_t* vrow = &vs[(sub * 16 + 4 * g + u) * PITCH + DC * r];
+            if constexpr (DC == 8) {
+              const u32x4 v = *reinterpret_cast<const u32x4*>(vrow);
+              vw[u][0] = v.x; vw[u][1] = v.y; vw[u][2] = v.z; vw[u][3] = v.w;
+            } else {
+              const u32x2 v = *reinterpret_cast<const u32x2*>(vrow);
+              vw[u][0] = v.x; vw[u][1] = v.y;
+            }
+          }
+#pragma unroll
+          for (int c = 0; c < DC / 2; ++c) {
+            const uint32_t lo0 = __builtin_amdgcn_perm(vw[1][c], vw[0][c], 0x05040100u);
+            const uint32_t lo1 = __builtin_amdgcn_perm(vw[3][c], vw[2][c], 0x05040100u);
+            const uint32_t hi0 = __builtin_amdgcn_perm(vw[1][c], vw[0][c], 0x07060302u);
+            const uint32_t hi1 = __builtin_amdgcn_perm(vw[3][c], vw[2][c], 0x07060302u);
+            oacc[mt][2 * c] = mfma_16x16x16<T>(pa[sub][0], pa[sub][1], lo0, lo1, oacc[mt][2 * c]);
+            oacc[mt][2 * c + 1] =
+                mfma_16x16x16<T>(pa[sub][0], pa[sub][1], hi0, hi1, oacc[mt][2 * c + 1]);
+          }
+        }
+      }
+    }
+    __syncthreads();  // every wave is done with the tile in LDS
+    if (more) {
+      stash();
+      __syncthreads();
+    }
+  }
+
+  // ---- normalise and store: lane holds rows 4g + i, dimensions [DC r, DC r + DC) ------------------
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt) {
+    float l = l_run[mt];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float li = __shfl(l, 4 * g + i, 64);
+      const float inv = li > 0.f ? 1.f / li : 0.f;
+      const int row = q0 + wave * 32 + mt * 16 + 4 * g + i;
+      if (row < p.n_q) {
+        uint16_t* dst = p.o + ((int64_t)row * p.num_qo_heads + qh) * D + DC * r;
+        if constexpr (DC == 8) {
+          u32x4 out;
+          out.x = pack2<T>(oacc[mt][0][i] * inv, oacc[mt][1][i] * inv);
+          out.y = pack2<T>(oacc[mt][2][i] * inv, oacc[mt][3][i] * inv);
+          out.z = pack2<T>(oacc[mt][4][i] * inv, oacc[mt][5][i] * inv);
+          out.w = pack2<T>(oacc[mt][6][i] * inv, oacc[mt][7][i] * inv);
+          *reinterpret_cast<u32x4*>(dst) = out;
+        } else {
+          u32x2 out;
+          out.x = pack2<T>(oacc[mt][0][i] * inv, oacc[mt][1][i] * inv);
+          out.y = pack2<T>(oacc[mt][2][i] * inv, oacc[mt][3][i] * inv);
+          *reinterpret_cast<u32x2*>(dst) = out;
+        }
+      }
+    }
+  }
+}
+
+template <typename T>
+static int launch_prefill(const PrefillParams& p, int head_dim, hipStream_t st) {
+  const dim3 grid((p.n_q + kPfBM - 1) / kPfBM, p.num_qo_heads), block(kPfThreads);
+  if (head_dim == 128)
+    hipLaunchKernelGGL((prefill_attn_kernel<T, 128>), grid, block, 0, st, p);
+  else if (head_dim == 64)
+    hipLaunchKernelGGL((prefill_attn_kernel<T, 64>), grid, block, 0, st, p);
+  else
+    return fail(TD_ERR_UNSUPPORTED, "BatchPrefillWithPagedKVCache failed to dispatch with head_dim %d",
+                head_dim);
+  return TD_OK;
+}
+
+}  // namespace tidal
+
+using namespace tidal;
+
+extern "C" int td_prefill_attn(const td_paged_kv* kv, const int32_t* page_table, int32_t n_pages,
+                               int32_t kv_len, const void* q, void* o, int32_t n_q,
+                               int32_t num_qo_heads, float sm_scale, int32_t causal, void* stream) {
+  TD_REQUIRE(kv && kv->data && page_table && q && o, "td_prefill_attn: NULL argument");
+  TD_REQUIRE(kv->page_size >= 1 && kv->num_kv_heads >= 1 && kv->max_pages >= 1,
+             "td_prefill_attn: bad pool geometry");
+  TD_REQUIRE(num_qo_heads >= kv->num_kv_heads && num_qo_heads % kv->num_kv_heads == 0,
+             "td_prefill_attn: num_qo_heads %d is not a multiple of num_kv_heads %d", num_qo_heads,
+             kv->num_kv_heads);
+  TD_REQUIRE(n_q >= 0 && kv_len >= n_q, "td_prefill_attn: n_q %d, kv_len %d", n_q, kv_len);
+  TD_REQUIRE((int64_t)n_pages * kv->page_size >= kv_len,
+             "td_prefill_attn: %d pages of %d entries do not hold %d tokens", n_pages,
+             kv->page_size, kv_len);
+  TD_REQUIRE(kv->layout == TD_NHD || kv->layout == TD_HND, "td_prefill_attn: layout %d", kv->layout);
+  if (n_q == 0) return TD_OK;
+  const int P = kv->page_size, H = kv->num_kv_heads, D = kv->head_dim;
+  PrefillParams p;
+  p.kv = reinterpret_cast<const uint16_t*>(kv->data);
+  p.page_stride = (int64_t)2 * P * H * D;
+  p.v_offset = (int64_t)P * H * D;
+  p.entry_stride = kv->layout == TD_NHD ? H * D : D;
+  p.head_stride = kv->layout == TD_NHD ? D : P * D;
+  p.page_size = P;
+  p.page_shift = (P & (P - 1)) == 0 ? __builtin_ctz(P) : -1;
+  p.max_page = (uint32_t)(kv->max_pages - 1);
+  p.page_table = page_table;
+  p.n_pages = n_pages;
+  p.kv_len = kv_len;
+  p.q = reinterpret_cast<const uint16_t*>(q);
+  p.o = reinterpret_cast<uint16_t*>(o);
+  p.n_q = n_q;
+  p.num_qo_heads = num_qo_heads;
+  p.q_per_kv = num_qo_heads / H;
+  p.scale_log2 = sm_scale * 1.4426950408889634f;
+  p.causal = causal;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  int rc;
+  if (kv->dtype == TD_F16)
+    rc = launch_prefill<F16>(p, D, st);
+  else if (kv->dtype == TD_BF16)
+    rc = launch_prefill<BF16>(p, D, st);
+  else
+    return fail(TD_ERR_UNSUPPORTED, "BatchPrefillWithPagedKVCache failed to dispatch with dtype %d",
+                kv->dtype);
+  if (rc != TD_OK) return rc;
+  TD_HIP_CHECK(hipGetLastError());
+  return TD_OK;
+}
