@@ -226,6 +226,23 @@ __device__ __forceinline__ f32x4 mfma_16x16x16<F16>(uint32_t a0, uint32_t a1, ui
                                                __builtin_bit_cast(h16x4, b), c, 0, 0, 0);
 }
 
+// gfx950: D(16x16, fp32) += A(16x32) * B(32x16); a lane holds A[lane % 16][8g .. 8g+7] and
+// B[8g .. 8g+7][lane % 16] (g = lane / 16) as four packed dwords.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+template <typename T>
+__device__ __forceinline__ f32x4 mfma_16x16x32(u32x4 a, u32x4 b, f32x4 c);
+template <>
+__device__ __forceinline__ f32x4 mfma_16x16x32<BF16>(u32x4 a, u32x4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                 __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ f32x4 mfma_16x16x32<F16>(u32x4 a, u32x4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
+                                                __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+
 constexpr float kNegBig = -1.0e30f;  // finite stand-in for -inf in running maxima
 
 __host__ __device__ __forceinline__ int64_t ceil_div64(int64_t a, int64_t b) {

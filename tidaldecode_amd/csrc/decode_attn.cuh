@@ -215,7 +215,9 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
   constexpr int TILE = U * TPI;  // tokens per wave tile
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  // scalar on purpose: control flow that depends on the wave index must be a real branch, because
+  // matrix instructions do not honour the EXEC mask of a masked-off region
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int g = lane / LPR;   // lane group = token slot inside the instruction
   const int li = lane % LPR;  // 16-byte column of the row
   const int hrow = blockIdx.x;

@@ -2,17 +2,17 @@
 // gfx950 (MI355X), on the matrix cores.  Replaces BatchPrefillWithPagedKVCache of the reference
 // (kernels/include/prefill/prefill.cuh:674-870, bound in tidal/ops/csrc/batch_prefill.cu:27-117).
 //
-// One 256-thread workgroup per (128 query rows, query head); a wavefront owns 32 query rows as
-// two 16-row tiles.  The loop walks the keys in tiles of 64 tokens that the workgroup stages once
+// One 256-thread workgroup per (64 MT query rows, query head); a wavefront owns 16 MT query rows
+// as MT = 2 16-row tiles: every K/V operand read from LDS feeds two matrix instructions.  The loop walks the keys in tiles of 64 tokens that the workgroup stages once
 // in LDS (rows padded to 272 bytes: conflict-free 16-byte reads) while the global loads of the
 // next tile are already in flight.  Per 16 tokens and query tile:
-//   S^T = K Q^T   mfma_f32_16x16x16, A = K rows from LDS, B = Q rows kept in registers; the head
-//                 dimension is walked in a permuted order (the same for Q and K), so that every
-//                 operand is a 16-byte piece of a row;
+//   S^T = K Q^T   mfma_f32_16x16x32, A = K rows from LDS, B = Q rows kept in registers: an operand
+//                 is a 16-byte piece of a row;
 //   softmax       base-2, online; the result tile has the query row in lane % 16 and four
 //                 tokens per lane, which is the A-operand layout of the next product;
-//   O += P V      A = P (rounded to the KV type), B = V: a lane reads the rows of its four tokens
-//                 (16 bytes each) and re-packs them with v_perm into one operand per dimension.
+//   O += P V      per 32 tokens: A = P (rounded to the KV type), B = V: a lane reads the rows of its
+//                 eight tokens (16 bytes each) and re-packs them with v_perm into one operand
+//                 per head dimension.
 // Pages are looked up per staged row; rows past the end of the sequence are clamped (never
 // out of the pool) and masked.
 
@@ -22,7 +22,6 @@
 namespace tidal {
 
 constexpr int kPfThreads = 256;
-constexpr int kPfBM = 128;  // query rows per workgroup
 constexpr int kPfBN = 64;   // tokens per key tile
 
 struct PrefillParams {
@@ -39,9 +38,11 @@ struct PrefillParams {
   int32_t causal;
 };
 
-template <typename T, int D>
-__global__ __launch_bounds__(kPfThreads) void prefill_attn_kernel(const PrefillParams p) {
-  constexpr int NS = D / 32;        // 16-byte pieces of a Q/K row per lane (two MFMA k-steps each)
+template <typename T, int D, int MT>
+__global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kernel(const PrefillParams p) {
+  constexpr int kPfBM = 64 * MT;    // query rows per workgroup
+  constexpr int WR = 16 * MT;       // query rows per wavefront
+  constexpr int NS = D / 32;        // 16-byte pieces of a Q/K row per lane (one MFMA each)
   constexpr int DC = D / 16;        // head dimensions per lane in the P.V product
   constexpr int PITCH = D + 8;      // LDS row pitch in elements: +16 bytes
   constexpr int CPR = D / 8;        // 16-byte chunks per row
@@ -50,7 +51,9 @@ __global__ __launch_bounds__(kPfThreads) void prefill_attn_kernel(const PrefillP
   __shared__ __attribute__((aligned(16))) uint16_t ks[kPfBN * PITCH];
   __shared__ __attribute__((aligned(16))) uint16_t vs[kPfBN * PITCH];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // the wave index is made scalar: the per-tile activity tests below must be real branches, because
+  // matrix instructions do not honour the EXEC mask of a masked-off region
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, g = lane >> 4;
   const int qtile = gridDim.x - 1 - blockIdx.x;  // longest rows first
   const int qh = blockIdx.y;
@@ -58,11 +61,11 @@ __global__ __launch_bounds__(kPfThreads) void prefill_attn_kernel(const PrefillP
   const int q0 = qtile * kPfBM;
   const int q_off = p.kv_len - p.n_q;  // position of query row 0
 
-  // ---- Q operands: row (q0 + 32 wave + 16 mt + r), pieces [32 s + 8 g, +8) ----------------------
-  u32x4 qb[2][NS];
+  // ---- Q operands: row (q0 + WR wave + 16 mt + r), pieces [32 s + 8 g, +8) ----------------------
+  u32x4 qb[MT][NS];
 #pragma unroll
-  for (int mt = 0; mt < 2; ++mt) {
-    int row = q0 + wave * 32 + mt * 16 + r;
+  for (int mt = 0; mt < MT; ++mt) {
+    int row = q0 + wave * WR + mt * 16 + r;
     row = row < p.n_q ? row : p.n_q - 1;
     const u32x4* src =
         reinterpret_cast<const u32x4*>(p.q + ((int64_t)row * p.num_qo_heads + qh) * D);
@@ -70,10 +73,10 @@ __global__ __launch_bounds__(kPfThreads) void prefill_attn_kernel(const PrefillP
     for (int s = 0; s < NS; ++s) qb[mt][s] = src[4 * s + g];
   }
 
-  f32x4 oacc[2][DC];
-  float m_run[2], l_run[2];
+  f32x4 oacc[MT][DC];
+  float m_run[MT], l_run[MT];
 #pragma unroll
-  for (int mt = 0; mt < 2; ++mt) {
+  for (int mt = 0; mt < MT; ++mt) {
     m_run[mt] = kNegBig;
     l_run[mt] = 0.f;
 #pragma unroll
@@ -120,34 +123,43 @@ __global__ __launch_bounds__(kPfThreads) void prefill_attn_kernel(const PrefillP
     }
   };
 
-  const int wave_first_pos = q_off + q0 + wave * 32;  // position of the wave's first query row
+  const int wave_first_pos = q_off + q0 + wave * WR;  // position of the wave's first query row
   fetch(0);
   stash();
   __syncthreads();
   for (int kt = 0; kt < kv_end; kt += kPfBN) {
     const bool more = kt + kPfBN < kv_end;
     if (more) fetch(kt + kPfBN);
-    // tiles entirely behind the causal frontier of this wave contribute nothing
-    const bool wave_active = !p.causal || kt <= wave_first_pos + 31;
-    if (wave_active) {
-      const bool need_mask = (p.causal && kt + kPfBN - 1 > wave_first_pos) || kt + kPfBN > p.kv_len;
+    // a query tile whose last row lies before the key tile sees none of it (causal)
+    bool act[MT];
 #pragma unroll
-      for (int mt = 0; mt < 2; ++mt) {
-        const int qpos = wave_first_pos + mt * 16 + r;  // position of this lane's query row
-        // ---- S^T for the four 16-token sub-tiles ---------------------------------------------------
-        f32x4 st[4];
+    for (int mt = 0; mt < MT; ++mt) act[mt] = !p.causal || kt <= wave_first_pos + mt * 16 + 15;
+    if (act[MT - 1]) {
+      // ---- S^T: each K operand is read once and used by every active query tile -----------------
+      f32x4 st[MT][4];
 #pragma unroll
-        for (int sub = 0; sub < 4; ++sub) {
+      for (int sub = 0; sub < 4; ++sub) {
+        u32x4 ka[NS];
+        const uint16_t* krow = &ks[(sub * 16 + r) * PITCH + 8 * g];
+#pragma unroll
+        for (int s = 0; s < NS; ++s) ka[s] = *reinterpret_cast<const u32x4*>(krow + 32 * s);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          if (!act[mt]) continue;
           f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-          const uint16_t* krow = &ks[(sub * 16 + r) * PITCH + 8 * g];
 #pragma unroll
-          for (int s = 0; s < NS; ++s) {
-            const u32x4 ka = *reinterpret_cast<const u32x4*>(krow + 32 * s);
-            acc = mfma_16x16x16<T>(ka.x, ka.y, qb[mt][s].x, qb[mt][s].y, acc);
-            acc = mfma_16x16x16<T>(ka.z, ka.w, qb[mt][s].z, qb[mt][s].w, acc);
-          }
-          st[sub] = acc * p.scale_log2;
+          for (int s = 0; s < NS; ++s) acc = mfma_16x16x32<T>(ka[s], qb[mt][s], acc);
+          st[mt][sub] = acc * p.scale_log2;
         }
+      }
+      // ---- online softmax of query row r (lanes r, r+16, r+32, r+48 share the row) ---------------
+      uint32_t pa[MT][4][2];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        if (!act[mt]) continue;
+        const int qpos = wave_first_pos + mt * 16 + r;  // position of this lane's query row
+        const bool need_mask =
+            (p.causal && kt + kPfBN - 1 > wave_first_pos + mt * 16) || kt + kPfBN > p.kv_len;
         if (need_mask) {
 #pragma unroll
           for (int sub = 0; sub < 4; ++sub)
@@ -155,32 +167,30 @@ __global__ __launch_bounds__(kPfThreads) void prefill_attn_kernel(const PrefillP
             for (int i = 0; i < 4; ++i) {
               const int tpos = kt + sub * 16 + 4 * g + i;
               const bool ok = tpos < p.kv_len && (!p.causal || tpos <= qpos);
-              st[sub][i] = ok ? st[sub][i] : kNegBig;
+              st[mt][sub][i] = ok ? st[mt][sub][i] : kNegBig;
             }
         }
-        // ---- online softmax of query row r (lanes r, r+16, r+32, r+48 share the row) ---------------
         float mt_max = kNegBig;
 #pragma unroll
         for (int sub = 0; sub < 4; ++sub)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) mt_max = fmaxf(mt_max, st[sub][i]);
+          for (int i = 0; i < 4; ++i) mt_max = fmaxf(mt_max, st[mt][sub][i]);
         mt_max = fmaxf(mt_max, __shfl_xor(mt_max, 16, 64));
         mt_max = fmaxf(mt_max, __shfl_xor(mt_max, 32, 64));
         const float m_new = fmaxf(m_run[mt], mt_max);
         const float alpha = fast_exp2(m_run[mt] - m_new);
         m_run[mt] = m_new;
         float psum = 0.f;
-        uint32_t pa[4][2];
 #pragma unroll
         for (int sub = 0; sub < 4; ++sub) {
           float pr[4];
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            pr[i] = st[sub][i] > 0.5f * kNegBig ? fast_exp2(st[sub][i] - m_new) : 0.f;
+            pr[i] = st[mt][sub][i] > 0.5f * kNegBig ? fast_exp2(st[mt][sub][i] - m_new) : 0.f;
             psum += pr[i];
           }
-          pa[sub][0] = pack2<T>(pr[0], pr[1]);
-          pa[sub][1] = pack2<T>(pr[2], pr[3]);
+          pa[mt][sub][0] = pack2<T>(pr[0], pr[1]);
+          pa[mt][sub][1] = pack2<T>(pr[2], pr[3]);
         }
         l_run[mt] = fmaf(l_run[mt], alpha, psum);
         // rescale: accumulator row 4g + i is query row 4g + i, whose factor sits in lane 4g + i
@@ -192,30 +202,41 @@ __global__ __launch_bounds__(kPfThreads) void prefill_attn_kernel(const PrefillP
             for (int d = 0; d < DC; ++d) oacc[mt][d][i] *= f;
           }
         }
-        // ---- O += P V ---------------------------------------------------------------------------------
+      }
+      // ---- O += P V, 32 tokens (two sub-tiles) per matrix instruction ------------------------------
 #pragma unroll
-        for (int sub = 0; sub < 4; ++sub) {
-          uint32_t vw[4][DC / 2];
+      for (int pair = 0; pair < 2; ++pair) {
+        uint32_t vw[8][DC / 2];  // rows 4g + u of sub-tile 2 pair (u < 4) and of sub-tile 2 pair + 1
 #pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            const uint16_t* vrow = &vs[(sub * 16 + 4 * g + u) * PITCH + DC * r];
-            if constexpr (DC == 8) {
-              const u32x4 v = *reinterpret_cast<const u32x4*>(vrow);
-              vw[u][0] = v.x; vw[u][1] = v.y; vw[u][2] = v.z; vw[u][3] = v.w;
-            } else {
-              const u32x2 v = *reinterpret_cast<const u32x2*>(vrow);
-              vw[u][0] = v.x; vw[u][1] = v.y;
-            }
+        for (int u = 0; u < 8; ++u) {
+          const int row = (2 * pair + u / 4) * 16 + 4 * g + (u % 4);
+          const uint16_t* vrow = &vs[row * PITCH + DC * r];
+          if constexpr (DC == 8) {
+            const u32x4 v = *reinterpret_cast<const u32x4*>(vrow);
+            vw[u][0] = v.x; vw[u][1] = v.y; vw[u][2] = v.z; vw[u][3] = v.w;
+          } else {
+            const u32x2 v = *reinterpret_cast<const u32x2*>(vrow);
+            vw[u][0] = v.x; vw[u][1] = v.y;
           }
+        }
 #pragma unroll
-          for (int c = 0; c < DC / 2; ++c) {
-            const uint32_t lo0 = __builtin_amdgcn_perm(vw[1][c], vw[0][c], 0x05040100u);
-            const uint32_t lo1 = __builtin_amdgcn_perm(vw[3][c], vw[2][c], 0x05040100u);
-            const uint32_t hi0 = __builtin_amdgcn_perm(vw[1][c], vw[0][c], 0x07060302u);
-            const uint32_t hi1 = __builtin_amdgcn_perm(vw[3][c], vw[2][c], 0x07060302u);
-            oacc[mt][2 * c] = mfma_16x16x16<T>(pa[sub][0], pa[sub][1], lo0, lo1, oacc[mt][2 * c]);
-            oacc[mt][2 * c + 1] =
-                mfma_16x16x16<T>(pa[sub][0], pa[sub][1], hi0, hi1, oacc[mt][2 * c + 1]);
+        for (int c = 0; c < DC / 2; ++c) {
+          u32x4 lo, hi;
+          lo.x = __builtin_amdgcn_perm(vw[1][c], vw[0][c], 0x05040100u);
+          lo.y = __builtin_amdgcn_perm(vw[3][c], vw[2][c], 0x05040100u);
+          lo.z = __builtin_amdgcn_perm(vw[5][c], vw[4][c], 0x05040100u);
+          lo.w = __builtin_amdgcn_perm(vw[7][c], vw[6][c], 0x05040100u);
+          hi.x = __builtin_amdgcn_perm(vw[1][c], vw[0][c], 0x07060302u);
+          hi.y = __builtin_amdgcn_perm(vw[3][c], vw[2][c], 0x07060302u);
+          hi.z = __builtin_amdgcn_perm(vw[5][c], vw[4][c], 0x07060302u);
+          hi.w = __builtin_amdgcn_perm(vw[7][c], vw[6][c], 0x07060302u);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            if (!act[mt]) continue;
+            const u32x4 pp = {pa[mt][2 * pair][0], pa[mt][2 * pair][1], pa[mt][2 * pair + 1][0],
+                              pa[mt][2 * pair + 1][1]};
+            oacc[mt][2 * c] = mfma_16x16x32<T>(pp, lo, oacc[mt][2 * c]);
+            oacc[mt][2 * c + 1] = mfma_16x16x32<T>(pp, hi, oacc[mt][2 * c + 1]);
           }
         }
       }
@@ -229,7 +250,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_attn_kernel(const PrefillP
 
   // ---- normalise and store: lane holds rows 4g + i, dimensions [DC r, DC r + DC) ------------------
 #pragma unroll
-  for (int mt = 0; mt < 2; ++mt) {
+  for (int mt = 0; mt < MT; ++mt) {
     float l = l_run[mt];
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
@@ -237,7 +258,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_attn_kernel(const PrefillP
     for (int i = 0; i < 4; ++i) {
       const float li = __shfl(l, 4 * g + i, 64);
       const float inv = li > 0.f ? 1.f / li : 0.f;
-      const int row = q0 + wave * 32 + mt * 16 + 4 * g + i;
+      const int row = q0 + wave * WR + mt * 16 + 4 * g + i;
       if (row < p.n_q) {
         uint16_t* dst = p.o + ((int64_t)row * p.num_qo_heads + qh) * D + DC * r;
         if constexpr (DC == 8) {
@@ -258,17 +279,26 @@ __global__ __launch_bounds__(kPfThreads) void prefill_attn_kernel(const PrefillP
   }
 }
 
-template <typename T>
-static int launch_prefill(const PrefillParams& p, int head_dim, hipStream_t st) {
-  const dim3 grid((p.n_q + kPfBM - 1) / kPfBM, p.num_qo_heads), block(kPfThreads);
+template <typename T, int MT>
+static int launch_prefill_mt(const PrefillParams& p, int head_dim, hipStream_t st) {
+  const dim3 grid((p.n_q + 64 * MT - 1) / (64 * MT), p.num_qo_heads), block(kPfThreads);
   if (head_dim == 128)
-    hipLaunchKernelGGL((prefill_attn_kernel<T, 128>), grid, block, 0, st, p);
+    hipLaunchKernelGGL((prefill_attn_kernel<T, 128, MT>), grid, block, 0, st, p);
   else if (head_dim == 64)
-    hipLaunchKernelGGL((prefill_attn_kernel<T, 64>), grid, block, 0, st, p);
+    hipLaunchKernelGGL((prefill_attn_kernel<T, 64, MT>), grid, block, 0, st, p);
   else
     return fail(TD_ERR_UNSUPPORTED, "BatchPrefillWithPagedKVCache failed to dispatch with head_dim %d",
                 head_dim);
   return TD_OK;
+}
+
+template <typename T>
+static int launch_prefill(const PrefillParams& p, int head_dim, hipStream_t st) {
+  // Two query tiles per wavefront keep the kernel at 256 registers, i.e. two workgroups per
+  // compute unit: one computes while the other waits for its next K/V tile.  Four tiles per
+  // wavefront halve the LDS traffic per flop but run one workgroup per compute unit with every
+  // memory and barrier latency exposed (measured: 2.5x slower).
+  return launch_prefill_mt<T, 2>(p, head_dim, st);
 }
 
 }  // namespace tidal
