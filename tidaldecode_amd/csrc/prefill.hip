@@ -149,7 +149,7 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
           f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int s = 0; s < NS; ++s) acc = mfma_16x16x32<T>(ka[s], qb[mt][s], acc);
-          st[mt][sub] = acc * p.scale_log2;
+          st[mt][sub] = acc;  // raw q.k; the softmax scale is folded into the exponent below
         }
       }
       // ---- online softmax of query row r (lanes r, r+16, r+32, r+48 share the row) ---------------
@@ -177,7 +177,9 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
           for (int i = 0; i < 4; ++i) mt_max = fmaxf(mt_max, st[mt][sub][i]);
         mt_max = fmaxf(mt_max, __shfl_xor(mt_max, 16, 64));
         mt_max = fmaxf(mt_max, __shfl_xor(mt_max, 32, 64));
-        const float m_new = fmaxf(m_run[mt], mt_max);
+        // m_run is kept in the scaled base-2 domain.  A masked entry (kNegBig) gives exp2(-huge) = 0
+        // by itself: every query row sees token 0 in its first tile, so m_new is a real maximum.
+        const float m_new = fmaxf(m_run[mt], mt_max * p.scale_log2);
         const float alpha = fast_exp2(m_run[mt] - m_new);
         m_run[mt] = m_new;
         float psum = 0.f;
@@ -186,7 +188,7 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
           float pr[4];
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            pr[i] = st[mt][sub][i] > 0.5f * kNegBig ? fast_exp2(st[mt][sub][i] - m_new) : 0.f;
+            pr[i] = fast_exp2(fmaf(st[mt][sub][i], p.scale_log2, -m_new));
             psum += pr[i];
           }
           pa[mt][sub][0] = pack2<T>(pr[0], pr[1]);
