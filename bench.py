@@ -54,6 +54,8 @@ def parse():
                     help="profile helper: run only the sparse-layer launches")
     ap.add_argument("--no-e2e", action="store_true",
                     help="skip the end-to-end decoder leg (Llama-2-7B shape, random weights)")
+    ap.add_argument("--no-prefill", action="store_true",
+                    help="skip the prefill-attention leg (one layer, causal, whole context)")
     ap.add_argument("--e2e-ctx", type=str, default="32768,102400",
                     help="context lengths of the end-to-end leg")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -276,6 +278,33 @@ def e2e_leg(args):
     return out
 
 
+def prefill_leg(args):
+    """Causal prefill attention of one layer over the whole context through the paged cache
+    (td_prefill_attn): ms per layer and matrix-core throughput on the causal flop count."""
+    import torch
+
+    from tidaldecode_amd import _kernels
+
+    dev = torch.device("cuda:0")
+    n, hq, hkv, d, page = args.ctx, args.heads, args.kv_heads, 128, 16
+    dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float16
+    n_pages = (n + page - 1) // page
+    g = torch.Generator(device=dev).manual_seed(0)
+    pool = torch.randn((n_pages, 2, page, hkv, d), generator=g, device=dev).to(dtype)
+    table = torch.randperm(n_pages, generator=g, device=dev).to(torch.int32)
+    q = torch.randn((n, hq, d), generator=g, device=dev).to(dtype)
+    last = (n - 1) % page + 1
+
+    def run():
+        return _kernels.prefill_with_paged_kv_cache(q, pool, table, last, True, 0, False, 1.0, 1e4)
+
+    ms = time_events(torch, run, 3, warm=2)
+    flops = 4.0 * n * n * d * hq / 2
+    return {"ms_per_layer": round(ms, 3), "tflops_causal": round(flops / ms / 1e9, 1),
+            "peak_tflops": 2500.0, "frac": round(flops / ms / 1e9 / 2500.0, 4),
+            "shape": f"{n} tokens, {hq}/{hkv} heads x {d}, page {page}, {args.dtype}"}
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -420,6 +449,8 @@ def main():
     }
     if "ms_per_step" in e:
         line["attention_path_tokens_per_s"] = round(1e3 / e["ms_per_step"], 1)
+    if not args.no_prefill and not args.only_sparse:
+        line["prefill_attn"] = prefill_leg(args)
     if not args.no_e2e and not args.only_sparse:
         line["e2e_decode_llama2_7b_shape"] = e2e_leg(args)
     if not args.no_cpu and not args.only_sparse:

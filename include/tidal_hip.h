@@ -258,6 +258,18 @@ int td_topk(const void* values, int32_t values_dtype, int64_t values_stride, int
 int64_t td_topk_workspace_bytes(int32_t rows);
 
 /*
+ * Page-level upper bound of the attention logits from the per-page key max / min metadata that
+ * td_append_kv maintains: o[h, e] = sum_d max(q[h,d] * max[e,d], q[h,d] * min[e,d]) for every
+ * metadata entry e but the newest ((n_meta_pages - 1) * page_size + meta_last_page_len - 1
+ * entries; o rows have stride o_stride, o in the pool's dtype).  Replaces estimate_attn_score
+ * (bsk_ops.h:41-48, tidal/ops/csrc/estimate.cu:6-88, MaxPossibleSampleWithPagedKVCacheKernel,
+ * kernels/include/decode/decode_attn.cuh:142-172,236-405).
+ */
+int td_estimate_score(const td_paged_kv* meta, const int32_t* meta_indices, int32_t n_meta_pages,
+                      int32_t meta_last_page_len, const void* q, int32_t num_qo_heads, void* o,
+                      int64_t o_stride, void* stream);
+
+/*
  * RMSNorm: out[r, :] = x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * weight, fp32 math.
  * Replaces rms_norm_forward (bsk_ops.h:29-32, tidal/ops/csrc/rms_norm.cu:160-212).
  */

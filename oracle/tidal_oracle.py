@@ -75,6 +75,26 @@ def stable_topk(scores: torch.Tensor, k: int) -> torch.Tensor:
     return torch.sort(order, dim=-1).values
 
 
+def page_score_bound(q: torch.Tensor, k: torch.Tensor, page_size: int) -> torch.Tensor:
+    """Page-level upper bound of the logits from per-page element-wise key max / min (the
+    estimator of the reference's ancestor: compute_max_possible,
+    kernels/include/decode/decode_attn.cuh:142-172; test loop kernels/src/test/test_max_possible.cu:81-100):
+    bound[h, p] = sum_d max(q[h, d] * max_p[d], q[h, d] * min_p[d]), unscaled.
+    q [H_q, D], k [N, H_kv, D]; pages are the full and partial groups of page_size tokens.
+    Returns [H_q, ceil(N / page_size)]."""
+    q, k = q.float(), k.float()
+    n, hkv, d = k.shape
+    hq = q.shape[0]
+    n_pages = (n + page_size - 1) // page_size
+    out = torch.empty((hq, n_pages))
+    for pg in range(n_pages):
+        rows = k[pg * page_size: (pg + 1) * page_size]          # [<=P, H_kv, D]
+        mx = rows.max(0).values.repeat_interleave(hq // hkv, 0)  # [H_q, D]
+        mn = rows.min(0).values.repeat_interleave(hq // hkv, 0)
+        out[:, pg] = torch.maximum(q * mx, q * mn).sum(-1)
+    return out
+
+
 def head_sum_scores(logits: torch.Tensor, rows: int = 1) -> torch.Tensor:
     """Softmax probabilities summed over the query heads of each of `rows` equal groups:
     [H_q, N] -> [rows, N] (rows=1: all heads; rows=H_kv: per KV head)."""

@@ -105,8 +105,10 @@ def test_python_surface_rejects_cpu_tensors_and_bad_shapes():
                                 torch.zeros((2, 4), dtype=torch.int32), None, 4)
     with pytest.raises(RuntimeError, match="Invalid layout"):
         _kernels.BatchDecodeWithPagedKVCachePyTorchWrapper(7)
-    with pytest.raises(NotImplementedError):
-        _kernels.estimate_attn_score()
+    with pytest.raises(RuntimeError, match="CUDA"):
+        _kernels.estimate_attn_score(q, torch.zeros((32, 4), dtype=torch.float16),
+                                     torch.zeros((2, 2, 16, 32, 128), dtype=torch.float16),
+                                     torch.zeros(1, dtype=torch.int32), None, 5, 0, 0)
     w = _kernels.BatchDecodeWithPagedKVCachePyTorchWrapper(0)
     with pytest.raises(RuntimeError, match="BeginForward"):
         w.forward(q, q, q, q, None, 1, 0, None)

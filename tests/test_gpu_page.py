@@ -209,3 +209,40 @@ def test_rms_norm(cuda, dtype, rows, cols):
     _kernels.rms_norm_forward(x.to(dtype).to(cuda), w.to(dtype).to(cuda), out, 1e-5)
     torch.cuda.synchronize()
     assert ((out.float().cpu() - want).abs() <= ULP[dtype] * 1.01 * want.abs() + 1e-6).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("hq,hkv,d,page,layout", [(32, 32, 128, 16, "NHD"), (8, 2, 64, 4, "HND"),
+                                                  (4, 4, 256, 7, "NHD"), (32, 8, 128, 32, "NHD")])
+def test_page_score_estimator(cuda, dtype, hq, hkv, d, page, layout):
+    """decode_estimate over the metadata the append kernels keep (prefill append, then decode
+    appends) against the oracle's bound on the same rounded keys; sequence lengths of the
+    reference's estimator test (kernels/src/test/test_max_possible.cu:158)."""
+    from oracle import tidal_oracle as orc
+    from tidaldecode_amd import utils as ops
+    from tidaldecode_amd.utils import InferenceController
+
+    for n in (65, 213, 1110):
+        c = InferenceController(1, hq, d, page, 64, 4096, dtype, cuda, num_kv_heads=hkv,
+                                kv_layout=layout, with_metadata=True, page_order_seed=2)
+        gk = torch.Generator().manual_seed(n)
+        k = torch.randn((n + 3, hkv, d), generator=gk).to(dtype)
+        v = torch.randn((n + 3, hkv, d), generator=gk).to(dtype)
+        c.prepare_metadata(n)
+        c.begin_forward(n)
+        ops.append_kv(k[:n].to(cuda), v[:n].to(cuda), c, 0)
+        c.end_forward()
+        for i in range(n, n + 3):
+            c.prepare_metadata(1)
+            c.begin_forward(1)
+            ops.append_kv(k[i:i + 1].to(cuda), v[i:i + 1].to(cuda), c, 0)
+            c.end_forward()
+        q = torch.randn((1, hq, d), generator=gk).to(dtype)
+        got = ops.decode_estimate(q.to(cuda), c, 0)
+        torch.cuda.synchronize()
+        want = orc.page_score_bound(q[0].float(), k.float(), page)
+        n_pages = (n + 3 + page - 1) // page
+        assert got.shape == (hq, n_pages - 1)            # the page being filled is left out
+        want = want[:, : n_pages - 1]
+        tol = (2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7) * want.abs().clamp(min=1.0) + 1e-3
+        assert ((got.float().cpu() - want).abs() <= tol).all()

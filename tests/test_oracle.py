@@ -305,3 +305,26 @@ def test_paged_selected_attention_equals_dense_on_the_same_tokens(layout):
     slots = table[pos // p] * p + pos % p
     got2, _ = orc.paged_selected_attention(q.numpy(), pool, slots.numpy(), 0, 0, layout, "slots")
     assert np.abs(got2 - want.numpy()).max() < 1e-5
+
+
+def test_page_score_bound_properties():
+    """The page estimator is an upper bound of every q.k inside the page, is tight for one-token
+    pages, and equals the closed form q.(max+min)/2 + |q|.(max-min)/2."""
+    g = torch.Generator().manual_seed(4)
+    q = torch.randn((8, 32), generator=g)
+    k = torch.randn((100, 4, 32), generator=g)
+    for page in (1, 3, 16, 100):
+        b = orc.page_score_bound(q, k, page)
+        raw = orc.attn_logits(q, k) * math.sqrt(32)          # unscaled q.k, [8, 100]
+        n_pages = (100 + page - 1) // page
+        assert b.shape == (8, n_pages)
+        for pg in range(n_pages):
+            inside = raw[:, pg * page: (pg + 1) * page]
+            assert (b[:, pg] >= inside.max(-1).values - 1e-4).all()
+            if page == 1:
+                assert (b[:, pg] - inside[:, 0]).abs().max() < 1e-4
+            rows = k[pg * page: (pg + 1) * page]
+            mx = rows.max(0).values.repeat_interleave(2, 0)
+            mn = rows.min(0).values.repeat_interleave(2, 0)
+            closed = (q * (mx + mn) / 2).sum(-1) + (q.abs() * (mx - mn) / 2).sum(-1)
+            assert (b[:, pg] - closed).abs().max() < 1e-4

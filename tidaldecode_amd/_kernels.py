@@ -225,13 +225,32 @@ def topk_workspace_bytes(rows: int) -> int:
     return int(lib.td_topk_workspace_bytes(int(rows)))
 
 
-def estimate_attn_score(*args, **kwargs):
-    """bsk_ops.h:41-48.  Page-level upper-bound estimator inherited from Quest; no TidalDecode
-    model code calls it (only tidal/utils/__init__.py:176-214 wraps it).  Not part of the
-    decode-attention path: raises."""
-    raise NotImplementedError(
-        "estimate_attn_score (Quest page estimator) is not used by TidalDecode's decode path and "
-        "is not provided by tidaldecode_amd")
+def estimate_attn_score(q: torch.Tensor, o: torch.Tensor, metadata_data: torch.Tensor,
+                        metadata_indices: torch.Tensor, metadata_indptr: Optional[torch.Tensor],
+                        metadata_last_page_len: int, metadata_last_page_idx: int,
+                        layout: int) -> None:
+    """bsk_ops.h:41-48 / estimate.cu:6-88.  Page-level upper bound of the logits (the estimator
+    TidalDecode inherited from Quest): ``o[h, e] = sum_d max(q*max_e, q*min_e)`` over the
+    metadata entries of ``metadata_indices`` except the newest one; ``q [1, H, D]``,
+    ``o [H, entries]``.  ``metadata_indptr`` and ``metadata_last_page_idx`` are accepted for
+    signature parity (all pages of ``metadata_indices`` are used, the last one is its last)."""
+    _check_input(q, "q")
+    _check_dim(3, q, "q")
+    _check_input(o, "o")
+    _check_dim(2, o, "o")
+    _check_input(metadata_indices, "metadata_indices")
+    _check_i32(metadata_indices, "metadata_indices")
+    pool = _pool(metadata_data, int(layout), "metadata_data")
+    if q.size(0) != 1 or q.size(2) != pool.head_dim or q.dtype != metadata_data.dtype \
+            or o.dtype != q.dtype or o.size(0) != q.size(1):
+        raise RuntimeError("estimate_attn_score: q / o do not fit the metadata pool")
+    n_pages = metadata_indices.numel()
+    n_entries = (n_pages - 1) * pool.page_size + int(metadata_last_page_len) - 1
+    if o.size(1) < n_entries:
+        raise RuntimeError(f"estimate_attn_score: o holds {o.size(1)} entries, {n_entries} needed")
+    check(lib.td_estimate_score(pool, metadata_indices.data_ptr(), n_pages,
+                                int(metadata_last_page_len), q.data_ptr(), q.size(1),
+                                o.data_ptr(), o.stride(0), _stream()))
 
 
 def _append(k, v, kv_data, kv_indices, kv_indptr, kv_last_page_len, metadata_data,

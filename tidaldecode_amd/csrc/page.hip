@@ -195,6 +195,42 @@ __global__ void append_meta_kernel(PoolGeom kvg, PoolGeom mg, const uint16_t* k,
   mrow[mg.v_offset + d] = from_float<T>(mn);
 }
 
+// Upper bound of q.k over the keys of a page from the page's element-wise max / min metadata:
+// o[h, e] = sum_d max(q[h, d] * max[e, d], q[h, d] * min[e, d]).  A 16-byte lane group per
+// metadata entry; grid: (ceil(entries / entries per workgroup), query heads).
+template <typename T, int D>
+__global__ __launch_bounds__(256) void estimate_kernel(PoolGeom mg, const int32_t* meta_indices,
+                                                       int n_entries, const uint16_t* q,
+                                                       int q_per_kv, uint16_t* o, int64_t o_stride) {
+  constexpr int LPR = D / 8;
+  constexpr int EPB = 256 / LPR;  // entries per workgroup
+  const int tid = threadIdx.x;
+  const int li = tid % LPR;
+  const int e = blockIdx.x * EPB + tid / LPR;
+  const int h = blockIdx.y;
+  const int ec = e < n_entries ? e : n_entries - 1;  // clamped: loads stay unconditional
+  const uint32_t page = (uint32_t)meta_indices[ec / mg.page_size];
+  const uint16_t* row = reinterpret_cast<const uint16_t*>(mg.data) +
+                        k_offset(mg, page, ec % mg.page_size, h / q_per_kv) + li * 8;
+  const u32x4 mx = *reinterpret_cast<const u32x4*>(row);
+  const u32x4 mn = *reinterpret_cast<const u32x4*>(row + mg.v_offset);
+  const u32x4 qv = *reinterpret_cast<const u32x4*>(q + (int64_t)h * D + li * 8);
+  const uint32_t mxw[4] = {mx.x, mx.y, mx.z, mx.w}, mnw[4] = {mn.x, mn.y, mn.z, mn.w},
+                 qw[4] = {qv.x, qv.y, qv.z, qv.w};
+  float acc = 0.f;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    float q0, q1, a0, a1, b0, b1;
+    unpack2<T>(qw[c], q0, q1);
+    unpack2<T>(mxw[c], a0, a1);
+    unpack2<T>(mnw[c], b0, b1);
+    acc += fmaxf(q0 * a0, q0 * b0);
+    acc += fmaxf(q1 * a1, q1 * b1);
+  }
+  acc = group_sum<LPR>(acc);
+  if (li == 0 && e < n_entries) o[(int64_t)h * o_stride + e] = from_float<T>(acc);
+}
+
 // RMSNorm, one 256-thread workgroup per row, fp32 accumulation
 template <typename T>
 __global__ __launch_bounds__(256) void rms_norm_kernel(const uint16_t* x, const uint16_t* w,
@@ -355,6 +391,50 @@ extern "C" int td_rope_table(const int32_t* positions, int32_t batch, int32_t he
   hipLaunchKernelGGL(rope_table_kernel, dim3(batch), dim3(head_dim / 2), 0,
                      reinterpret_cast<hipStream_t>(stream), positions, head_dim,
                      1.0 / (double)rope_scale, log2((double)rope_theta), cos, sin);
+  TD_HIP_CHECK(hipGetLastError());
+  return TD_OK;
+}
+
+extern "C" int td_estimate_score(const td_paged_kv* meta, const int32_t* meta_indices,
+                                 int32_t n_meta_pages, int32_t meta_last_page_len, const void* q,
+                                 int32_t num_qo_heads, void* o, int64_t o_stride, void* stream) {
+  int rc = check_pool(meta, "td_estimate_score");
+  if (rc) return rc;
+  TD_REQUIRE(meta_indices && q && o, "td_estimate_score: NULL argument");
+  TD_REQUIRE(num_qo_heads >= meta->num_kv_heads && num_qo_heads % meta->num_kv_heads == 0,
+             "td_estimate_score: num_qo_heads %d is not a multiple of num_kv_heads %d",
+             num_qo_heads, meta->num_kv_heads);
+  TD_REQUIRE(n_meta_pages >= 1 && meta_last_page_len >= 1 && meta_last_page_len <= meta->page_size,
+             "td_estimate_score: %d pages, last page length %d", n_meta_pages, meta_last_page_len);
+  // the newest entry describes the page still being filled and is left out, as in the reference
+  const int n_entries = (n_meta_pages - 1) * meta->page_size + meta_last_page_len - 1;
+  TD_REQUIRE(o_stride >= n_entries, "td_estimate_score: o_stride %lld < %d entries",
+             (long long)o_stride, n_entries);
+  if (n_entries == 0) return TD_OK;
+  const PoolGeom mg = geom_of(meta);
+  const int D = meta->head_dim;
+  const int qpk = num_qo_heads / meta->num_kv_heads;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const uint16_t* qp = reinterpret_cast<const uint16_t*>(q);
+  uint16_t* op = reinterpret_cast<uint16_t*>(o);
+#define TD_EST(T, DD)                                                                            \
+  hipLaunchKernelGGL((estimate_kernel<T, DD>), dim3((n_entries + 2048 / DD - 1) / (2048 / DD),   \
+                                                    num_qo_heads),                               \
+                     dim3(256), 0, st, mg, meta_indices, n_entries, qp, qpk, op, o_stride)
+  if (meta->dtype == TD_F16) {
+    if (D == 64) TD_EST(F16, 64);
+    else if (D == 128) TD_EST(F16, 128);
+    else if (D == 256) TD_EST(F16, 256);
+    else return fail(TD_ERR_UNSUPPORTED, "estimate_attn_score failed to dispatch with head_dim %d", D);
+  } else if (meta->dtype == TD_BF16) {
+    if (D == 64) TD_EST(BF16, 64);
+    else if (D == 128) TD_EST(BF16, 128);
+    else if (D == 256) TD_EST(BF16, 256);
+    else return fail(TD_ERR_UNSUPPORTED, "estimate_attn_score failed to dispatch with head_dim %d", D);
+  } else {
+    return fail(TD_ERR_UNSUPPORTED, "estimate_attn_score failed to dispatch with dtype %d", meta->dtype);
+  }
+#undef TD_EST
   TD_HIP_CHECK(hipGetLastError());
   return TD_OK;
 }

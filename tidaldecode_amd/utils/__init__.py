@@ -86,9 +86,20 @@ def prefill_forward(q: torch.Tensor, iController: InferenceController, layer_idx
         1.0 if rope_scale is None else rope_scale, 1e4 if rope_theta is None else rope_theta)
 
 
-def decode_estimate(q: torch.Tensor, iController: InferenceController, layer_idx: int):
-    """Page-score estimator of the reference's ancestor; dead code in TidalDecode."""
-    return _kernels.estimate_attn_score(q, iController, layer_idx)
+def decode_estimate(q: torch.Tensor, iController: InferenceController, layer_idx: int
+                    ) -> torch.Tensor:
+    """Page-score estimator of the reference's ancestor (tidal/utils/__init__.py:176-214): upper
+    bound of the logits per KV page from the page metadata, ``[H, pages - 1]`` (the page being
+    filled is left out).  Needs a controller built ``with_metadata=True``; TidalDecode's own
+    layers never call it."""
+    c = iController
+    if c.metadata_cache is None:
+        raise RuntimeError("decode_estimate needs InferenceController(..., with_metadata=True)")
+    o = torch.empty((q.size(1), c.metadata_cache.seqlen - 1), dtype=q.dtype, device=q.device)
+    _kernels.estimate_attn_score(q, o, c.metadata_cache.buf_layer(layer_idx), c.metadata_indices,
+                                 c.metadata_indptr_for_append, c.metadata_cache.last_page_len,
+                                 c.metadata_last_page_idx, c.layout)
+    return o
 
 
 def decode_topk(iController: InferenceController):
