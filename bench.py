@@ -54,6 +54,10 @@ def parse():
                     help="profile helper: run only the sparse-layer launches")
     ap.add_argument("--no-e2e", action="store_true",
                     help="skip the end-to-end decoder leg (Llama-2-7B shape, random weights)")
+    ap.add_argument("--sweep", action="store_true",
+                    help="instead of the benchmark line: attention-path latency for token budgets "
+                         "{256,1024,2048,4096} x contexts {10240,32768,102400} against full "
+                         "attention (the grid of the reference's latency figure), one JSON object")
     ap.add_argument("--no-prefill", action="store_true",
                     help="skip the prefill-attention leg (one layer, causal, whole context)")
     ap.add_argument("--e2e-ctx", type=str, default="32768,102400",
@@ -100,6 +104,7 @@ class Workload:
         page = c.kv_cache.indicies[pos // self.P]
         self.dst_slot = torch.tensor([page * self.P + pos % self.P], dtype=torch.int32,
                                      device=self.dev)
+        self._probe_out = None
         self.fuse = (not args.no_fuse) and c.fused_step_ok
         from tidaldecode_amd import _kernels
         self.cos, self.sin = _kernels.rope_table(self.positions, self.D)
@@ -141,6 +146,17 @@ class Workload:
 
         return ops.decode_sparse_attn(self.q[layer], self.c, layer,
                                       self.c.topk_dindices_buffer, False, fresh=fresh)
+
+    def gather_probe(self, layer):
+        """memory side of sparse_attn(layer) alone (no arithmetic, no merge)"""
+        from tidaldecode_amd import _kernels
+
+        if self._probe_out is None:
+            self._probe_out = self.torch.empty(self.H * 64 * 8, dtype=self.torch.int32,
+                                               device=self.dev)
+        return _kernels.gather_probe(self.c._decode_handler._wrapper,
+                                     self.c.kv_cache.buf_layer(layer), self.c.topk_dindices_buffer,
+                                     self._probe_out)
 
     def step(self):
         """attention path of one decode step; with fusion RoPE + append ride inside the attention
@@ -305,6 +321,44 @@ def prefill_leg(args):
             "shape": f"{n} tokens, {hq}/{hkv} heads x {d}, page {page}, {args.dtype}"}
 
 
+def sweep(args):
+    """Attention-only latency of one decode step (all layers, hipGraph) for every budget x context
+    of the reference's latency evaluation (README llama_latency_eval figure; tidal/models/llama.py:
+    616-656 sets the budget), with the ratio to full attention in every layer."""
+    import copy
+
+    import torch
+
+    out = {"shape": f"{args.layers} layers, {args.heads}/{args.kv_heads} heads x 128, {args.dtype}, "
+                    f"page 16, {args.select_mode} lists, selection layers 0 and 2", "rows": []}
+    for ctx in (10240, 32768, 102400):
+        full_ms = None
+        for budget in (256, 1024, 2048, 4096):
+            a = copy.copy(args)
+            a.ctx, a.top_k = ctx, budget
+            w = Workload(a, args.select_mode)
+            w.step()
+            torch.cuda.synchronize()
+            r_step, _ = capture(torch, w.step, not args.no_graph)
+            ms = time_events(torch, r_step, 20)
+            if full_ms is None:
+                def full_step():
+                    if w.fuse:
+                        w.rope_table()
+                    for layer in range(w.L):
+                        if not w.fuse:
+                            w.rope_append(layer)
+                        w.full_attn(layer, w.fresh(layer) if w.fuse else None)
+
+                r_full, _ = capture(torch, full_step, not args.no_graph)
+                full_ms = time_events(torch, r_full, 5, warm=1)
+            out["rows"].append({"ctx": ctx, "budget": budget, "tidal_ms": round(ms, 4),
+                                "full_ms": round(full_ms, 4), "ratio": round(ms / full_ms, 4)})
+            del w
+            torch.cuda.empty_cache()
+    return out
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -318,6 +372,9 @@ def main():
         sys.exit(1)
 
     use_graph = not args.no_graph
+    if args.sweep:
+        print(json.dumps(sweep(args)))
+        return
     if args.calibrate_copy:
         src = torch.ones(64 << 20, dtype=torch.float32, device="cuda:0")  # 256 MiB
         dst = torch.empty_like(src)
@@ -351,6 +408,16 @@ def main():
             r_plain, _ = capture(torch, run_sparse_plain, use_graph)
             entry["sparse_unfused_us_per_layer"] = (time_events(torch, r_plain, max(args.steps, 20))
                                                     * 1e3 / len(sparse))
+        if w.H == w.HKV and w.c.index_rows == w.H and args.layout == "NHD" and not args.waves \
+                and not args.chunk and not args.rows:
+            # the same lists gathered by a kernel that does nothing else: the memory floor of the launch
+            def run_probe():
+                for layer in sparse:
+                    w.gather_probe(layer)
+
+            r_probe, _ = capture(torch, run_probe, use_graph)
+            entry["gather_only_us_per_layer"] = (time_events(torch, r_probe, max(args.steps, 20))
+                                                 * 1e3 / len(sparse))
         if not args.only_sparse:
             def run_select():
                 for layer in w.sel_layers:

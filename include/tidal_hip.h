@@ -277,6 +277,18 @@ int td_rms_norm(const void* x, const void* weight, void* out, int32_t rows, int3
                 float eps, int32_t dtype, void* stream);
 
 /*
+ * Measurement aid without a counterpart in the reference: the memory side of a sparse layer
+ * alone.  Same grid and the same list -> slot -> K / V row loads as td_decode_attn for
+ * token-slot lists (the launch that replaces BatchDecodeWithPagedKVCacheKernel,
+ * kernels/include/decode/decode_attn.cuh:432-658), no arithmetic and no merge; one word per
+ * wavefront is written to out (batch * head rows * plan->max_splits * 8 words).  bench.py times
+ * it next to the attention launch.
+ */
+int td_gather_probe(const td_paged_kv* kv, const td_index_list* list, const td_decode_plan* plan,
+                    int32_t batch, int32_t num_qo_heads, void* out, int64_t out_bytes,
+                    void* stream);
+
+/*
  * Prefill: attention of the n_q newest tokens of one sequence (q, o: [n_q, num_qo_heads, head_dim])
  * over its kv_len cached tokens, whose pages are page_table[0 .. n_pages) in order (K/V of the
  * new tokens already appended).  causal != 0: query row i sees positions <= kv_len - n_q + i.

@@ -557,6 +557,30 @@ class BatchDecodeWithPagedKVCachePyTorchWrapper:
                                  ws.numel() if ws is not None else 0, _stream()))
 
 
+def gather_probe(wrapper: "BatchDecodeWithPagedKVCachePyTorchWrapper", paged_kv_data: torch.Tensor,
+                 slots: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Measurement aid: only the memory side of ``wrapper.forward(..., slots, index_kind="slots")``
+    (same grid, same list -> K/V row loads, no arithmetic, no merge).  Returns the word-per-wave
+    output tensor, which is of no use except that it keeps the loads alive."""
+    _check_rows(slots, "slots")
+    _check_i32(slots, "slots")
+    pool = _pool(paged_kv_data, wrapper._layout, "paged_kv_data")
+    hq, hkv, d, page, dtype = wrapper._geom
+    rows, budget = slots.shape
+    lst = IndexList()
+    lst.idx = _ptr(slots)
+    lst.idx_rows = rows
+    lst.idx_row_stride = slots.stride(0)
+    lst.kind = TD_IDX_SLOTS
+    lst.n_list_host = budget
+    plan = wrapper._plan(1, rows, budget)
+    words = hq * int(plan.max_splits) * 8
+    if out is None:
+        out = torch.empty(words, dtype=torch.int32, device=slots.device)
+    check(lib.td_gather_probe(pool, lst, plan, 1, hq, out.data_ptr(), out.numel() * 4, _stream()))
+    return out
+
+
 def score_reduce(logits: torch.Tensor, lse: torch.Tensor, num_kv_heads: int, n: int,
                  mode: str = "head_sum", out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Extension: sum of softmax probabilities over query heads.  logits float32 ``[H_q, stride]``,

@@ -119,6 +119,11 @@ SIGNATURES = {
          c_int32, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p],
     ),
     "td_topk_workspace_bytes": (c_int64, [c_int32]),
+    "td_gather_probe": (
+        c_int32,
+        [POINTER(PagedKV), POINTER(IndexList), POINTER(DecodePlan), c_int32, c_int32, c_void_p,
+         c_int64, c_void_p],
+    ),
     "td_estimate_score": (
         c_int32,
         [POINTER(PagedKV), c_void_p, c_int32, c_int32, c_void_p, c_int32, c_void_p, c_int64,

@@ -97,12 +97,12 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
   return TD_OK;
 }
 
-extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
-                              const td_decode_plan* plan, const void* q, void* o, int32_t batch,
-                              int32_t num_qo_heads, float sm_scale, void* scores,
-                              int32_t scores_dtype, int64_t score_stride, float* lse,
-                              const td_fresh_token* fresh, void* workspace,
-                              int64_t workspace_bytes, void* stream) {
+// Argument checks and the kernel parameter block shared by td_decode_attn and td_gather_probe.
+static int build_params(const td_paged_kv* kv, const td_index_list* list, const td_decode_plan* plan,
+                        const void* q, void* o, int32_t batch, int32_t num_qo_heads, float sm_scale,
+                        void* scores, int32_t scores_dtype, int64_t score_stride, float* lse,
+                        const td_fresh_token* fresh, void* workspace, int64_t workspace_bytes,
+                        DecodeParams& p, int& qpg_out, int& n_hrows_out) {
   TD_REQUIRE(kv && list && plan && q && o, "td_decode_attn: NULL argument");
   TD_REQUIRE(kv->data != nullptr, "td_decode_attn: kv->data is NULL");
   TD_REQUIRE(batch >= 1, "td_decode_attn: batch %d < 1", batch);
@@ -157,6 +157,8 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
 
   const int qpg = qpg_for(num_qo_heads, Hkv, list->idx_rows, D);
   const int n_hrows = num_qo_heads / qpg;
+  qpg_out = qpg;
+  n_hrows_out = n_hrows;
 
   const int64_t n_part = (int64_t)batch * num_qo_heads * plan->max_splits;
   const int64_t off_o = kTicketBytes;
@@ -174,7 +176,6 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
                   (long long)workspace_bytes, (long long)need);
   }
 
-  DecodeParams p;
   p.q = q;
   p.o = o;
   p.kv = kv->data;
@@ -239,6 +240,21 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
   p.ws_o = reinterpret_cast<float*>(ws ? ws + off_o : nullptr);
   p.ws_ml = reinterpret_cast<float*>(ws ? ws + off_ml : nullptr);
 
+  return TD_OK;
+}
+
+extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
+                              const td_decode_plan* plan, const void* q, void* o, int32_t batch,
+                              int32_t num_qo_heads, float sm_scale, void* scores,
+                              int32_t scores_dtype, int64_t score_stride, float* lse,
+                              const td_fresh_token* fresh, void* workspace,
+                              int64_t workspace_bytes, void* stream) {
+  DecodeParams p;
+  int qpg, n_hrows;
+  const int prc = build_params(kv, list, plan, q, o, batch, num_qo_heads, sm_scale, scores, scores_dtype,
+                               score_stride, lse, fresh, workspace, workspace_bytes, p, qpg, n_hrows);
+  if (prc != TD_OK) return prc;
+  const int D = kv->head_dim;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const bool page_mode = list->kind == TD_IDX_PAGES;
   dim3 grid(n_hrows, plan->max_splits, batch);
@@ -251,6 +267,80 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
     rc = launch_decode_bf16(p, D, qpg, plan->waves_per_block, plan->tile_rows, page_mode, scores != nullptr,
                             merge_kernel, grid, st);
   if (rc != TD_OK) return rc;
+  TD_HIP_CHECK(hipGetLastError());
+  return TD_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Measurement aid: the memory side of a sparse layer alone.  Same grid, same interleaved tiles,
+// same list -> slot -> K row / V row non-temporal 16-byte loads as decode_attn_kernel for token
+// -slot lists, but no arithmetic, no merge: every wave folds what it loaded into one word and
+// stores it.  Its duration is the floor that the attention launch is compared with.
+// ---------------------------------------------------------------------------------------------
+template <int D, int U, int NW>
+__global__ __launch_bounds__(NW * 64) void gather_probe_kernel(const DecodeParams p, uint32_t* out) {
+  constexpr int LPR = D / 8, TPI = 64 / LPR, TILE = U * TPI;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int g = lane / LPR, li = lane % LPR;
+  const int hrow = blockIdx.x, split = blockIdx.y, b = blockIdx.z;
+  const int kv_head = hrow / p.q_per_kv;
+  SeqList s;
+  int list_beg;
+  const int n_splits = seq_items(p, b, s, list_beg);
+  if (split >= n_splits) return;
+  const int idx_row = p.idx_per_kv ? kv_head : hrow;
+  s.row = p.idx + (int64_t)idx_row * p.idx_row_stride + list_beg;
+  const int c1 = s.n_list;  // listed slots only
+  const char* kbase = reinterpret_cast<const char*>(p.kv);
+  const char* vbase = kbase + p.v_offset * 2;
+  const uint32_t head_byte_off = (uint32_t)(kv_head * p.head_stride + li * 8) * 2u;
+  const int STEP = n_splits * NW * TILE;
+  u32x4 fold = {0u, 0u, 0u, 0u};
+  for (int t = (split * NW + wave) * TILE; t < c1; t += STEP) {
+    u32x4 kb[U], vb[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      int i = t + u * TPI + g;
+      i = i < c1 ? i : c1 - 1;
+      uint32_t slot = (uint32_t)s.row[i];
+      slot = slot > p.max_slot ? p.max_slot : slot;
+      const uint32_t page = slot >> p.page_shift, entry = slot & ((1u << p.page_shift) - 1u);
+      const uint32_t off = page * p.page_stride_b + entry * p.entry_stride_b + head_byte_off;
+      kb[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kbase + off));
+      vb[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vbase + off));
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) fold ^= kb[u] ^ vb[u];
+  }
+  uint32_t w = fold.x ^ fold.y ^ fold.z ^ fold.w;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) w ^= (uint32_t)__shfl_xor((int)w, off, 64);
+  if (lane == 0)
+    out[(((int64_t)b * gridDim.x + hrow) * gridDim.y + split) * NW + wave] = w;
+}
+
+extern "C" int td_gather_probe(const td_paged_kv* kv, const td_index_list* list,
+                               const td_decode_plan* plan, int32_t batch, int32_t num_qo_heads,
+                               void* out, int64_t out_bytes, void* stream) {
+  TD_REQUIRE(out != nullptr, "td_gather_probe: NULL out");
+  DecodeParams p;
+  int qpg, n_hrows;
+  const int prc = build_params(kv, list, plan, out, out, batch, num_qo_heads, 1.f, nullptr, TD_F32, 0,
+                               nullptr, nullptr, out, (int64_t)1 << 40, p, qpg, n_hrows);
+  if (prc != TD_OK) return prc;
+  if (!(list->kind == TD_IDX_SLOTS && p.lean && qpg == 1 && kv->head_dim == 128 &&
+        plan->waves_per_block == 8 && plan->tile_rows == 4 && list->last_page_len == 0 &&
+        !list->last_page_len_arr))
+    return fail(TD_ERR_UNSUPPORTED,
+                "td_gather_probe: token-slot lists without a forced last page, one query head per "
+                "row, head_dim 128, power-of-two pages, pool below 4 GiB, 8 waves x 4 rows only");
+  TD_REQUIRE(out_bytes >= (int64_t)batch * n_hrows * plan->max_splits * 8 * 4,
+             "td_gather_probe: out holds %lld bytes, %lld needed", (long long)out_bytes,
+             (long long)batch * n_hrows * plan->max_splits * 8 * 4);
+  hipLaunchKernelGGL((gather_probe_kernel<128, 4, 8>), dim3(n_hrows, plan->max_splits, batch),
+                     dim3(512), 0, reinterpret_cast<hipStream_t>(stream), p,
+                     reinterpret_cast<uint32_t*>(out));
   TD_HIP_CHECK(hipGetLastError());
   return TD_OK;
 }
