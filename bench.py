@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the TidalDecode decode-attention path on one MI355X.
 
-Workload (BASELINE.json configs[1], Llama-2-7B shape): 32 layers, 32 query / 32 KV heads,
+Workload (benchmark configuration 1, Llama-2-7B shape): 32 layers, 32 query / 32 KV heads,
 head_dim 128, bf16 paged KV with page size 16 (pages scattered in the pool), context 32768
 tokens, top_k = 2048, token selection (full attention + logits + top-k) at layers 0 and 2, sparse
 attention over the persisted tokens in the other 30 layers.  One *step* is the attention path of
@@ -359,6 +359,52 @@ def sweep(args):
     return out
 
 
+def batch8_leg(args):
+    """Sparse decode attention for a ragged batch of 8 sequences (benchmark configuration 3:
+    lengths randint(8192, 65537) seed 0, fp16, page 16, 1024 selected tokens per sequence and
+    head, pages scattered in one pool): one launch for the whole batch, several pools in rotation
+    so that the data is cold."""
+    import torch
+
+    from tidaldecode_amd import _kernels
+
+    dev = torch.device("cuda:0")
+    h, d, page, k, nb, n_pools = 32, 128, 16, 1024, 8, 4
+    g = torch.Generator().manual_seed(0)
+    lens = torch.randint(8192, 65537, (nb,), generator=g).tolist()
+    pages = [(n + page - 1) // page for n in lens]
+    total = sum(pages)
+    perm = torch.randperm(total, generator=g)
+    rows, used = [], 0
+    for b_, n in enumerate(lens):
+        table = perm[used: used + pages[b_]]
+        used += pages[b_]
+        pos = torch.stack([torch.randperm(n, generator=g)[:k] for _ in range(h)])
+        rows.append((table[pos // page] * page + pos % page).to(torch.int32))
+    idx = torch.cat(rows, dim=1).contiguous().to(dev)
+    indptr = torch.arange(0, (nb + 1) * k, k, dtype=torch.int32, device=dev)
+    zeros = torch.zeros(nb, dtype=torch.int32, device=dev)
+    pools = [torch.randn((total, 2, page, h, d), device=dev, dtype=torch.float16) for _ in range(n_pools)]
+    q = torch.randn((nb, h, d), device=dev, dtype=torch.float16)
+    o = torch.empty_like(q)
+    w = _kernels.BatchDecodeWithPagedKVCachePyTorchWrapper(0)
+    w.begin_forward(None, h, h, d, page, torch.empty(0, dtype=torch.float16))
+
+    def run():
+        for pool in pools:
+            w.forward(q, o, pool, idx, indptr, zeros, zeros, None, index_kind="slots", n_list=k)
+
+    r, how = capture(torch, run, not args.no_graph)
+    us = time_events(torch, r, 20) * 1e3 / n_pools
+    algo = nb * k * h * d * 2 * 2 + nb * k * h * 4 + 2 * nb * h * d * 2
+    del pools
+    torch.cuda.empty_cache()
+    return {"us_per_launch": round(us, 3), "algorithmic_bytes": algo,
+            "achieved_gbs": round(algo / us / 1e3, 1), "frac": round(algo / us / 1e3 / HBM_PEAK_GBS, 4),
+            "launch": how, "shape": f"batch {nb}, lengths {lens}, {h}/{h} heads x {d}, fp16, "
+                                    f"page {page}, {k} tokens per sequence and head"}
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -518,6 +564,7 @@ def main():
         line["attention_path_tokens_per_s"] = round(1e3 / e["ms_per_step"], 1)
     if not args.no_prefill and not args.only_sparse:
         line["prefill_attn"] = prefill_leg(args)
+        line["batch8_sparse_attn"] = batch8_leg(args)
     if not args.no_e2e and not args.only_sparse:
         line["e2e_decode_llama2_7b_shape"] = e2e_leg(args)
     if not args.no_cpu and not args.only_sparse:

@@ -9,7 +9,7 @@ HIP path is compared against them.
 
     python tests/golden/make_fixtures.py
 
-cfg0.npz      BASELINE configuration 0: 32/32 heads, head_dim 128, 4096 tokens, top_k 256.
+cfg0.npz      benchmark configuration 0: 32/32 heads, head_dim 128, 4096 tokens, top_k 256.
               Inputs are regenerated from seeds (selection layer seed 0, sparse layer seed 1) and
               rounded to fp16, so only outputs are stored.
 small.npz     4 query / 2 KV heads, head_dim 64, 96 tokens, page size 4, top_k 16, fp16: inputs

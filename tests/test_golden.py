@@ -114,7 +114,7 @@ def test_gpu_small_fixture(cuda, mode):
 @pytest.mark.gpu
 @pytest.mark.parametrize("mode", ["per_head", "head_sum"])
 def test_gpu_cfg0(cuda, mode):
-    """BASELINE configuration 0 on the GPU in fp16 against the fixture."""
+    """benchmark configuration 0 on the GPU in fp16 against the fixture."""
     from oracle import tidal_oracle as orc
 
     f = _load("cfg0.npz")
