@@ -521,16 +521,25 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
         a = dot2<T>(qp[j][3], kb[u].w, a);
         a = group_sum<LPR>(a) * p.scale_log2;
         sc[j][u] = valid ? a : kNegBig;
-        if constexpr (EMIT) {
-          if (valid && li == 0) {
-            const int64_t at = ((int64_t)b * p.num_qo_heads + qh0 + j) * p.score_stride + i;
-            const float nat = a * kLn2;
-            if (p.scores_f32)
-              reinterpret_cast<float*>(p.scores)[at] = nat;
-            else
-              reinterpret_cast<uint16_t*>(p.scores)[at] = from_float<T>(nat);
-          }
-        }
+      }
+    }
+    if constexpr (EMIT) {
+      // one store per tile: lane L < TILE collects the logit of token base + L (row L / TPI of
+      // lane group L % TPI) and the TILE lanes write consecutive addresses
+      float e = 0.f;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const float v = __shfl(sc[0][u], (lane % TPI) * LPR, 64);
+        e = (lane / TPI == u) ? v : e;
+      }
+      const int i = base + lane;
+      if (lane < TILE && i < c1) {
+        const int64_t at = ((int64_t)b * p.num_qo_heads + qh0) * p.score_stride + i;
+        const float nat = e * kLn2;
+        if (p.scores_f32)
+          reinterpret_cast<float*>(p.scores)[at] = nat;
+        else
+          reinterpret_cast<uint16_t*>(p.scores)[at] = from_float<T>(nat);
       }
     }
 #pragma unroll
