@@ -37,8 +37,9 @@ __device__ __forceinline__ float wave_sum64(float x) {
   return x;
 }
 
-// R rows per wavefront, UN 16-byte chunks per lane and row in flight (R * UN loads per lane)
-template <typename T, int MODE, bool PAIR, int R, int UN>
+// R rows per wavefront, UN 16-byte chunks per lane and row in flight (R * UN loads per lane),
+// XR 16-byte chunks of x per thread (XR * 256 * 8 >= cols)
+template <typename T, int MODE, bool PAIR, int R, int UN, int XR>
 __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(const GemvParams p) {
   constexpr int kGemvRows = R, kGemvUnroll = UN;
   __shared__ uint32_t xs[kGemvMaxCols / 2];
@@ -47,57 +48,12 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(const GemvParams p) 
   const int cols = p.cols;
   const int chunks = cols / 8;
 
-  // ---- stage x (and what is folded into it) in LDS, as packed 16-bit pairs ----------------------
-  if constexpr (MODE == 0) {
-    for (int c = tid; c < chunks; c += kGemvThreads)
-      reinterpret_cast<u32x4*>(xs)[c] = reinterpret_cast<const u32x4*>(p.x)[c];
-  } else if constexpr (MODE == 1) {
-    // RMSNorm as the model computes it: fp32 statistics, the normalised value rounded to the
-    // storage type, then the weight applied in the storage type
-    float ss = 0.f;
-    for (int c = tid; c < chunks; c += kGemvThreads) {
-      const u32x4 v = reinterpret_cast<const u32x4*>(p.x)[c];
-      reinterpret_cast<u32x4*>(xs)[c] = v;
-      float a, b;
-      unpack2<T>(v.x, a, b); ss = fmaf(a, a, fmaf(b, b, ss));
-      unpack2<T>(v.y, a, b); ss = fmaf(a, a, fmaf(b, b, ss));
-      unpack2<T>(v.z, a, b); ss = fmaf(a, a, fmaf(b, b, ss));
-      unpack2<T>(v.w, a, b); ss = fmaf(a, a, fmaf(b, b, ss));
-    }
-    ss = wave_sum64(ss);
-    if (lane == 0) red[wave] = ss;
-    __syncthreads();
-    float tot = 0.f;
-#pragma unroll
-    for (int w = 0; w < kGemvWaves; ++w) tot += red[w];
-    const float inv = rsqrtf(tot / (float)cols + p.eps);
-    // (the barrier above also ordered the staging stores before these reads of other threads' dwords)
-    for (int c = tid; c < cols / 2; c += kGemvThreads) {
-      float a, b, wa, wb;
-      unpack2<T>(xs[c], a, b);
-      unpack2<T>(reinterpret_cast<const uint32_t*>(p.norm_weight)[c], wa, wb);
-      float na, nb;
-      unpack2<T>(pack2<T>(a * inv, b * inv), na, nb);
-      xs[c] = pack2<T>(na * wa, nb * wb);
-    }
-  } else {
-    // gated MLP input: silu(gate) rounded to the storage type, times up, rounded again
-    for (int c = tid; c < cols / 2; c += kGemvThreads) {
-      float ga, gb, ua, ub;
-      unpack2<T>(reinterpret_cast<const uint32_t*>(p.x)[c], ga, gb);
-      unpack2<T>(reinterpret_cast<const uint32_t*>(p.x + cols)[c], ua, ub);
-      float sa, sb;
-      unpack2<T>(pack2<T>(ga / (1.f + __expf(-ga)), gb / (1.f + __expf(-gb))), sa, sb);
-      xs[c] = pack2<T>(sa * ua, sb * ub);
-    }
-  }
-  __syncthreads();
-
-  // ---- rows ---------------------------------------------------------------------------------------
+  // ---- rows of this wavefront; the first batch of weight loads is issued before x is staged: the
+  // weights do not depend on x, so the staging (and the norm's reduction) hides behind them ------
   const int half = p.rows / 2;
   const int unit = blockIdx.x * kGemvWaves + wave;  // two consecutive rows, or a gate/up row pair
   const int n_units = PAIR ? (half + kGemvRows / 2 - 1) / (kGemvRows / 2) : (p.rows + kGemvRows - 1) / kGemvRows;
-  if (unit >= n_units) return;
+  const bool unit_live = unit < n_units;  // a wave without rows still helps staging x
   // PAIR: rows [unit * R/2, +R/2) of the gate block and the same rows of the up block
   constexpr int HR = kGemvRows > 1 ? kGemvRows / 2 : 1;
   int row_of[kGemvRows];
@@ -113,15 +69,93 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(const GemvParams p) 
     const int row = row_of[r] < p.rows ? row_of[r] : p.rows - 1;  // a clamped row is computed, not stored
     wrow[r] = reinterpret_cast<const u32x4*>(p.w + (int64_t)row * p.w_row_stride);
   }
-  for (int c0 = 0; c0 < chunks; c0 += 64 * kGemvUnroll) {
-    u32x4 wv[kGemvRows][kGemvUnroll];
+  // Program order of the loads matters (the wait counter retires in order): x first, then the
+  // weights, so that waiting for x does not wait for the weights.
+  u32x4 xr[XR], nr[XR];
+  if constexpr (MODE != 2) {
+#pragma unroll
+    for (int k = 0; k < XR; ++k) {
+      const int c = tid + k * kGemvThreads;
+      const int cc = c < chunks ? c : chunks - 1;
+      xr[k] = reinterpret_cast<const u32x4*>(p.x)[cc];
+      if constexpr (MODE == 1) nr[k] = reinterpret_cast<const u32x4*>(p.norm_weight)[cc];
+    }
+  }
+  u32x4 wv[kGemvRows][kGemvUnroll];
+  auto load_trip = [&](int c0) {
 #pragma unroll
     for (int u = 0; u < kGemvUnroll; ++u) {
       const int c = c0 + u * 64 + lane;
-      const int cc = c < chunks ? c : chunks - 1;  // unconditional loads; masked below
+      const int cc = c < chunks ? c : chunks - 1;  // unconditional loads; masked in the product
 #pragma unroll
       for (int r = 0; r < kGemvRows; ++r) wv[r][u] = __builtin_nontemporal_load(wrow[r] + cc);
     }
+  };
+  load_trip(0);
+
+  // ---- stage x (and what is folded into it) in LDS, as packed 16-bit pairs ----------------------
+  if constexpr (MODE == 0) {
+#pragma unroll
+    for (int k = 0; k < XR; ++k) {
+      const int c = tid + k * kGemvThreads;
+      if (c < chunks) reinterpret_cast<u32x4*>(xs)[c] = xr[k];
+    }
+  } else if constexpr (MODE == 1) {
+    // RMSNorm as the model computes it: fp32 statistics, the normalised value rounded to the
+    // storage type, then the weight applied in the storage type
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < XR; ++k) {
+      if (tid + k * kGemvThreads < chunks) {
+        const uint32_t w4[4] = {xr[k].x, xr[k].y, xr[k].z, xr[k].w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          float a, b;
+          unpack2<T>(w4[q], a, b);
+          ss = fmaf(a, a, fmaf(b, b, ss));
+        }
+      }
+    }
+    ss = wave_sum64(ss);
+    if (lane == 0) red[wave] = ss;
+    __syncthreads();
+    float tot = 0.f;
+#pragma unroll
+    for (int w = 0; w < kGemvWaves; ++w) tot += red[w];
+    const float inv = rsqrtf(tot / (float)cols + p.eps);
+#pragma unroll
+    for (int k = 0; k < XR; ++k) {
+      const int c = tid + k * kGemvThreads;
+      if (c < chunks) {
+        const uint32_t x4[4] = {xr[k].x, xr[k].y, xr[k].z, xr[k].w};
+        const uint32_t n4[4] = {nr[k].x, nr[k].y, nr[k].z, nr[k].w};
+        uint32_t o4[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          float a, b, wa, wb, na, nb;
+          unpack2<T>(x4[q], a, b);
+          unpack2<T>(n4[q], wa, wb);
+          unpack2<T>(pack2<T>(a * inv, b * inv), na, nb);
+          o4[q] = pack2<T>(na * wa, nb * wb);
+        }
+        reinterpret_cast<u32x4*>(xs)[c] = u32x4{o4[0], o4[1], o4[2], o4[3]};
+      }
+    }
+  } else {
+    // gated MLP input: silu(gate) rounded to the storage type, times up, rounded again
+    for (int c = tid; c < cols / 2; c += kGemvThreads) {
+      float ga, gb, ua, ub;
+      unpack2<T>(reinterpret_cast<const uint32_t*>(p.x)[c], ga, gb);
+      unpack2<T>(reinterpret_cast<const uint32_t*>(p.x + cols)[c], ua, ub);
+      float sa, sb;
+      unpack2<T>(pack2<T>(ga / (1.f + __expf(-ga)), gb / (1.f + __expf(-gb))), sa, sb);
+      xs[c] = pack2<T>(sa * ua, sb * ub);
+    }
+  }
+  __syncthreads();
+
+  if (!unit_live) return;
+  for (int c0 = 0;;) {
 #pragma unroll
     for (int u = 0; u < kGemvUnroll; ++u) {
       const int c = c0 + u * 64 + lane;
@@ -136,6 +170,9 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(const GemvParams p) 
         acc[r] = dot2<T>(wv[r][u].w, xv.w, acc[r]);
       }
     }
+    c0 += 64 * kGemvUnroll;
+    if (c0 >= chunks) break;
+    load_trip(c0);
   }
   float sum[kGemvRows];
 #pragma unroll
@@ -164,22 +201,33 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(const GemvParams p) 
   }
 }
 
-template <typename T, int R, int UN>
-static void launch_gemv_shape(const GemvParams& p, int mode, bool pair, hipStream_t st) {
+template <typename T, int R, int UN, int XR>
+static void launch_gemv_x(const GemvParams& p, int mode, bool pair, hipStream_t st) {
   const int units = pair ? (p.rows / 2 + R / 2 - 1) / (R / 2) : (p.rows + R - 1) / R;
   const dim3 grid((units + kGemvWaves - 1) / kGemvWaves), block(kGemvThreads);
   if (pair) {
     if (mode == 0)
-      hipLaunchKernelGGL((gemv_kernel<T, 0, true, R, UN>), grid, block, 0, st, p);
+      hipLaunchKernelGGL((gemv_kernel<T, 0, true, R, UN, XR>), grid, block, 0, st, p);
     else
-      hipLaunchKernelGGL((gemv_kernel<T, 1, true, R, UN>), grid, block, 0, st, p);
+      hipLaunchKernelGGL((gemv_kernel<T, 1, true, R, UN, XR>), grid, block, 0, st, p);
   } else if (mode == 0) {
-    hipLaunchKernelGGL((gemv_kernel<T, 0, false, R, UN>), grid, block, 0, st, p);
+    hipLaunchKernelGGL((gemv_kernel<T, 0, false, R, UN, XR>), grid, block, 0, st, p);
   } else if (mode == 1) {
-    hipLaunchKernelGGL((gemv_kernel<T, 1, false, R, UN>), grid, block, 0, st, p);
+    hipLaunchKernelGGL((gemv_kernel<T, 1, false, R, UN, XR>), grid, block, 0, st, p);
   } else {
-    hipLaunchKernelGGL((gemv_kernel<T, 2, false, R, UN>), grid, block, 0, st, p);
+    hipLaunchKernelGGL((gemv_kernel<T, 2, false, R, UN, 1>), grid, block, 0, st, p);
   }
+}
+
+template <typename T, int R, int UN>
+static void launch_gemv_shape(const GemvParams& p, int mode, bool pair, hipStream_t st) {
+  const int per_thread = (p.cols / 8 + kGemvThreads - 1) / kGemvThreads;  // x chunks per thread
+  if (per_thread <= 2)
+    launch_gemv_x<T, R, UN, 2>(p, mode, pair, st);
+  else if (per_thread <= 6)
+    launch_gemv_x<T, R, UN, 6>(p, mode, pair, st);
+  else
+    launch_gemv_x<T, R, UN, 8>(p, mode, pair, st);
 }
 
 // Tall matrices: four rows per wavefront (fewer, longer-lived waves stream better); short ones:
