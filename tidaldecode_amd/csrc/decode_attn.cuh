@@ -282,18 +282,29 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
   }
   // Rotation of q and of the new key, and the cache write; called once the first K/V tile of
   // the wave is in flight so that these few loads and shuffles hide behind it.
+  // rotate-half RoPE of 8 elements per lane; the partner dimension (+- D/2) sits LPR/2 lanes away
+  auto rotate = [&](uint32_t(&w)[4]) {
+    float x[8], y[8];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) unpack2<T>(w[c], x[2 * c], x[2 * c + 1]);
+#pragma unroll
+    for (int d = 0; d < 8; ++d) {
+      float partner;
+      if constexpr (LPR == 16)
+        partner = dpp_move<0x128>(x[d]);  // row_ror:8 == lane ^ 8 inside the 16-lane row
+      else if constexpr (LPR == 8)
+        partner = lane_xor16<4>(x[d]);
+      else
+        partner = __shfl_xor(x[d], LPR / 2, 64);
+      y[d] = x[d] * rcs[d] + partner * rsn[d];
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) w[c] = pack2<T>(y[2 * c], y[2 * c + 1]);
+  };
+  // (Rotating the new key lazily, only where the list meets the new slot, keeps cos/sin alive
+  // through the main loop and costs more registers than it saves instructions.)
   auto finish_fresh = [&]() {
     if constexpr (FRESH) {
-      constexpr int HALF = LPR / 2;
-      auto rotate = [&](uint32_t(&w)[4]) {
-        float x[8], y[8];
-#pragma unroll
-        for (int c = 0; c < 4; ++c) unpack2<T>(w[c], x[2 * c], x[2 * c + 1]);
-#pragma unroll
-        for (int d = 0; d < 8; ++d) y[d] = x[d] * rcs[d] + __shfl_xor(x[d], HALF, 64) * rsn[d];
-#pragma unroll
-        for (int c = 0; c < 4; ++c) w[c] = pack2<T>(y[2 * c], y[2 * c + 1]);
-      };
 #pragma unroll
       for (int j = 0; j < QPG; ++j) rotate(qp[j]);
       rotate(knew);
