@@ -265,7 +265,7 @@ def e2e_leg(args):
     cfg = TidalLlamaConfig.llama2_7b(top_k=args.top_k, sparse_layer_start=0, correction_layer=2,
                                      select_mode=args.select_mode)
     model = TidalLlama(cfg, "cuda:0", seed=0)
-    model.tidal_init(page_size=16, max_seq_len=max(ctxs) + 64, page_order_seed=0)
+    model.tidal_init(page_size=16, max_seq_len=max(ctxs) + 128, page_order_seed=0)
     out = {}
     for ctx in ctxs:
         row = {}
@@ -288,6 +288,20 @@ def e2e_leg(args):
                                    use_graph=not args.no_graph)
         model.use_gemv = True
         row["tidal_torch_linear_ms_per_token"] = round(dt * 1e3, 4)
+        # a real greedy loop: eager launches, the sequence grows by one token per step, one
+        # device synchronisation per token (decode_step)
+        model.tidal_clear()
+        model.synthetic_prefill(ctx)
+        tok = torch.zeros(1, dtype=torch.long, device="cuda:0")
+        for _ in range(3):
+            tok = model.decode_step(tok).argmax().view(1)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        n_gen = 32
+        for _ in range(n_gen):
+            tok = model.decode_step(tok).argmax().view(1)
+        torch.cuda.synchronize()
+        row["tidal_eager_generate_ms_per_token"] = round((time.perf_counter() - t0) / n_gen * 1e3, 4)
         out[str(ctx)] = row
     del model
     torch.cuda.empty_cache()
