@@ -128,10 +128,13 @@ __device__ __forceinline__ void merge_splits(const DecodeParams& p, int b, int q
   const int j = c / (D / 2), d2 = c % (D / 2);
   const int64_t part0 = ((int64_t)b * p.num_qo_heads + qh0 + j) * p.max_splits;
 
-  float ml_m = kNegBig, ml_l = 0.f;
+  // (m, l) of every split and head: one pair per thread; the load is unconditional (clamped
+  // thread index) so that it is in flight together with the partial loads below
+  float ml_m, ml_l;
   const bool has_ml = tid < n_splits * QPG;
-  if (has_ml) {
-    const int jj = tid / n_splits, ss = tid % n_splits;
+  {
+    const int tc = has_ml ? tid : 0;
+    const int jj = tc / n_splits, ss = tc % n_splits;
     load_coherent(p.ws_ml + (((int64_t)b * p.num_qo_heads + qh0 + jj) * p.max_splits + ss) * 2,
                   ml_m, ml_l);
   }
