@@ -468,7 +468,7 @@ def main():
             r_plain, _ = capture(torch, run_sparse_plain, use_graph)
             entry["sparse_unfused_us_per_layer"] = (time_events(torch, r_plain, max(args.steps, 20))
                                                     * 1e3 / len(sparse))
-        if w.H == w.HKV and w.c.index_rows == w.H and args.layout == "NHD" and not args.waves \
+        if w.H == w.HKV and w.c.index_rows in (1, w.H) and args.layout == "NHD" and not args.waves \
                 and not args.chunk and not args.rows:
             # the same lists gathered by a kernel that does nothing else: the memory floor of the launch
             def run_probe():
