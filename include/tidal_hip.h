@@ -292,7 +292,7 @@ int td_gather_probe(const td_paged_kv* kv, const td_index_list* list, const td_d
  * Prefill: attention of the n_q newest tokens of one sequence (q, o: [n_q, num_qo_heads, head_dim])
  * over its kv_len cached tokens, whose pages are page_table[0 .. n_pages) in order (K/V of the
  * new tokens already appended).  causal != 0: query row i sees positions <= kv_len - n_q + i.
- * head_dim 64 or 128, fp16 / bf16.  Replaces prefill_with_paged_kv_cache (bsk_ops.h:80-88,
+ * head_dim 64, 128 or 256, fp16 / bf16.  Replaces prefill_with_paged_kv_cache (bsk_ops.h:80-88,
  * tidal/ops/csrc/batch_prefill.cu:27-117, kernels/include/prefill/prefill.cuh:674-870).
  */
 int td_prefill_attn(const td_paged_kv* kv, const int32_t* page_table, int32_t n_pages,

@@ -60,7 +60,8 @@ def test_causal_prefill_matches_dense_attention(cuda, dtype, kv_len, n_q):
 @pytest.mark.parametrize("hq,hkv,d,page,layout,causal", [
     (32, 8, 128, 16, 0, True), (4, 2, 64, 4, 0, True), (4, 4, 64, 16, 1, True),
     (8, 2, 128, 1, 0, True), (8, 8, 128, 8, 1, True), (6, 3, 128, 5, 0, True),
-    (8, 8, 128, 16, 0, False), (4, 2, 64, 16, 1, False)])
+    (8, 8, 128, 16, 0, False), (4, 2, 64, 16, 1, False), (4, 2, 256, 16, 0, True),
+    (2, 2, 256, 8, 1, True), (4, 1, 256, 16, 0, False)])
 def test_head_layouts_page_sizes_and_non_causal(cuda, hq, hkv, d, page, layout, causal):
     dtype = torch.float16
     kv_len, n_q = 1500, 333
@@ -96,6 +97,11 @@ def test_prefill_errors(cuda):
     with pytest.raises(RuntimeError):   # 3 query heads over 2 KV heads
         _kernels.prefill_with_paged_kv_cache(q[:8, :3].contiguous(), pool, table, 16, True, 0,
                                              False, 1.0, 1e4)
+    with pytest.raises(RuntimeError, match="failed to dispatch"):   # head_dim without a kernel
+        _kernels.prefill_with_paged_kv_cache(
+            torch.zeros((4, 2, 32), dtype=torch.float16, device=cuda),
+            torch.zeros((4, 2, 16, 2, 32), dtype=torch.float16, device=cuda), table, 16, True, 0,
+            False, 1.0, 1e4)
     with pytest.raises(RuntimeError):   # dtype mismatch
         _kernels.prefill_with_paged_kv_cache(q[:8].bfloat16(), pool, table, 16, True, 0, False,
                                              1.0, 1e4)

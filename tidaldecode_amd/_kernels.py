@@ -345,44 +345,24 @@ def rope_table(positions: torch.Tensor, head_dim: int, rope_scale: float = 1.0,
 def prefill_with_paged_kv_cache(q, kv_data, kv_indices, kv_last_page_len, causal, layout,
                                 allow_fp16_qk_reduction, rope_scale, rope_theta) -> torch.Tensor:
     """bsk_ops.h:80-88 / batch_prefill.cu:27-117.  Attention of the ``q.size(0)`` newest tokens
-    over the paged cache (their K/V already appended), causal or not.  head_dim 64 / 128 run the
-    library's matrix-core kernel (``td_prefill_attn``); other head dimensions gather the pages
-    and call torch's fused SDPA on the GPU."""
+    over the paged cache (their K/V already appended), causal or not, on the matrix cores
+    (``td_prefill_attn``; head_dim 64, 128 or 256).  ``allow_fp16_qk_reduction``, ``rope_scale``
+    and ``rope_theta`` are accepted for signature parity: RoPE is applied before the cache is
+    written (RotaryMode::kNone in the reference's call, batch_prefill.cu:95)."""
     _check_input(q, "q")
     _check_dim(3, q, "q")
+    _check_input(kv_indices, "kv_indices")
+    _check_i32(kv_indices, "kv_indices")
     pool = _pool(kv_data, int(layout))
     n_pages = kv_indices.numel()
     kv_len = (n_pages - 1) * pool.page_size + int(kv_last_page_len)
-    if pool.head_dim in (64, 128):
-        _check_input(kv_indices, "kv_indices")
-        _check_i32(kv_indices, "kv_indices")
-        if q.size(2) != pool.head_dim or q.dtype != kv_data.dtype:
-            raise RuntimeError("prefill_with_paged_kv_cache: q does not fit the cache")
-        o = torch.empty_like(q)
-        check(lib.td_prefill_attn(pool, kv_indices.data_ptr(), n_pages, kv_len, q.data_ptr(),
-                                  o.data_ptr(), q.size(0), q.size(1),
-                                  1.0 / math.sqrt(pool.head_dim), int(bool(causal)), _stream()))
-        return o
-    pages = kv_data.index_select(0, kv_indices.long())  # [n, 2, P, H, D] or [n, 2, H, P, D]
-    if int(layout) == TD_HND:
-        pages = pages.permute(0, 1, 3, 2, 4)
-    kk = pages[:, 0].reshape(n_pages * pool.page_size, pool.num_kv_heads, pool.head_dim)[:kv_len]
-    vv = pages[:, 1].reshape(n_pages * pool.page_size, pool.num_kv_heads, pool.head_dim)[:kv_len]
-    hq = q.size(1)
-    group = hq // pool.num_kv_heads
-    qq = q.transpose(0, 1).unsqueeze(0)  # [1, Hq, N, D]
-    kk = kk.transpose(0, 1).repeat_interleave(group, 0).unsqueeze(0)
-    vv = vv.transpose(0, 1).repeat_interleave(group, 0).unsqueeze(0)
-    n = q.size(0)
-    if causal and n == kv_len:
-        o = torch.nn.functional.scaled_dot_product_attention(qq, kk, vv, is_causal=True)
-    else:
-        mask = None
-        if causal and n > 1:
-            qpos = torch.arange(kv_len - n, kv_len, device=q.device).unsqueeze(1)
-            mask = torch.arange(kv_len, device=q.device).unsqueeze(0) <= qpos
-        o = torch.nn.functional.scaled_dot_product_attention(qq, kk, vv, attn_mask=mask)
-    return o.squeeze(0).transpose(0, 1).contiguous()
+    if q.size(2) != pool.head_dim or q.dtype != kv_data.dtype:
+        raise RuntimeError("prefill_with_paged_kv_cache: q does not fit the cache")
+    o = torch.empty_like(q)
+    check(lib.td_prefill_attn(pool, kv_indices.data_ptr(), n_pages, kv_len, q.data_ptr(),
+                              o.data_ptr(), q.size(0), q.size(1),
+                              1.0 / math.sqrt(pool.head_dim), int(bool(causal)), _stream()))
+    return o
 
 
 # ------------------------------------------------------------------------------------------

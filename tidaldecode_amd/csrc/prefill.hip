@@ -3,7 +3,8 @@
 // (kernels/include/prefill/prefill.cuh:674-870, bound in tidal/ops/csrc/batch_prefill.cu:27-117).
 //
 // One 256-thread workgroup per (64 MT query rows, query head); a wavefront owns 16 MT query rows
-// as MT = 2 16-row tiles: every K/V operand read from LDS feeds two matrix instructions.  The loop walks the keys in tiles of 64 tokens that the workgroup stages once
+// as MT = 2 16-row tiles: every K/V operand read from LDS feeds two matrix instructions
+// (head_dim 256: 64 query rows per workgroup, MT = 1, key tiles of 32 tokens).  The loop walks the keys in tiles of 64 tokens that the workgroup stages once
 // in LDS (rows padded to 272 bytes: conflict-free 16-byte reads) while the global loads of the
 // next tile are already in flight.  Per 16 tokens and query tile:
 //   S^T = K Q^T   mfma_f32_16x16x32, A = K rows from LDS, B = Q rows kept in registers: an operand
@@ -22,7 +23,6 @@
 namespace tidal {
 
 constexpr int kPfThreads = 256;
-constexpr int kPfBN = 64;   // tokens per key tile
 
 struct PrefillParams {
   const uint16_t* kv;
@@ -38,7 +38,8 @@ struct PrefillParams {
   int32_t causal;
 };
 
-template <typename T, int D, int MT>
+// BN tokens per key tile (a multiple of 32)
+template <typename T, int D, int MT, int BN>
 __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kernel(const PrefillParams p) {
   constexpr int kPfBM = 64 * MT;    // query rows per workgroup
   constexpr int WR = 16 * MT;       // query rows per wavefront
@@ -46,8 +47,11 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
   constexpr int DC = D / 16;        // head dimensions per lane in the P.V product
   constexpr int PITCH = D + 8;      // LDS row pitch in elements: +16 bytes
   constexpr int CPR = D / 8;        // 16-byte chunks per row
+  constexpr int kPfBN = BN;
+  constexpr int NSUB = BN / 16;     // 16-token sub-tiles per key tile
   constexpr int CPT = kPfBN * CPR / kPfThreads;  // chunks a thread stages per tile and matrix
-  static_assert(D == 64 || D == 128, "head dimensions of the prefill kernel");
+  static_assert(D == 64 || D == 128 || D == 256, "head dimensions of the prefill kernel");
+  static_assert(BN % 32 == 0 && CPT >= 1, "key tile");
   __shared__ __attribute__((aligned(16))) uint16_t ks[kPfBN * PITCH];
   __shared__ __attribute__((aligned(16))) uint16_t vs[kPfBN * PITCH];
 
@@ -136,9 +140,9 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
     for (int mt = 0; mt < MT; ++mt) act[mt] = !p.causal || kt <= wave_first_pos + mt * 16 + 15;
     if (act[MT - 1]) {
       // ---- S^T: each K operand is read once and used by every active query tile -----------------
-      f32x4 st[MT][4];
+      f32x4 st[MT][NSUB];
 #pragma unroll
-      for (int sub = 0; sub < 4; ++sub) {
+      for (int sub = 0; sub < NSUB; ++sub) {
         u32x4 ka[NS];
         const uint16_t* krow = &ks[(sub * 16 + r) * PITCH + 8 * g];
 #pragma unroll
@@ -153,7 +157,7 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
         }
       }
       // ---- online softmax of query row r (lanes r, r+16, r+32, r+48 share the row) ---------------
-      uint32_t pa[MT][4][2];
+      uint32_t pa[MT][NSUB][2];
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         if (!act[mt]) continue;
@@ -162,7 +166,7 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
             (p.causal && kt + kPfBN - 1 > wave_first_pos + mt * 16) || kt + kPfBN > p.kv_len;
         if (need_mask) {
 #pragma unroll
-          for (int sub = 0; sub < 4; ++sub)
+          for (int sub = 0; sub < NSUB; ++sub)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               const int tpos = kt + sub * 16 + 4 * g + i;
@@ -172,7 +176,7 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
         }
         float mt_max = kNegBig;
 #pragma unroll
-        for (int sub = 0; sub < 4; ++sub)
+        for (int sub = 0; sub < NSUB; ++sub)
 #pragma unroll
           for (int i = 0; i < 4; ++i) mt_max = fmaxf(mt_max, st[mt][sub][i]);
         mt_max = fmaxf(mt_max, __shfl_xor(mt_max, 16, 64));
@@ -184,7 +188,7 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
         m_run[mt] = m_new;
         float psum = 0.f;
 #pragma unroll
-        for (int sub = 0; sub < 4; ++sub) {
+        for (int sub = 0; sub < NSUB; ++sub) {
           float pr[4];
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
@@ -207,13 +211,18 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
       }
       // ---- O += P V, 32 tokens (two sub-tiles) per matrix instruction ------------------------------
 #pragma unroll
-      for (int pair = 0; pair < 2; ++pair) {
+      for (int pair = 0; pair < NSUB / 2; ++pair) {
         uint32_t vw[8][DC / 2];  // rows 4g + u of sub-tile 2 pair (u < 4) and of sub-tile 2 pair + 1
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
           const int row = (2 * pair + u / 4) * 16 + 4 * g + (u % 4);
           const uint16_t* vrow = &vs[row * PITCH + DC * r];
-          if constexpr (DC == 8) {
+          if constexpr (DC == 16) {
+            const u32x4 v = *reinterpret_cast<const u32x4*>(vrow);
+            const u32x4 v2 = *reinterpret_cast<const u32x4*>(vrow + 8);
+            vw[u][0] = v.x; vw[u][1] = v.y; vw[u][2] = v.z; vw[u][3] = v.w;
+            vw[u][4] = v2.x; vw[u][5] = v2.y; vw[u][6] = v2.z; vw[u][7] = v2.w;
+          } else if constexpr (DC == 8) {
             const u32x4 v = *reinterpret_cast<const u32x4*>(vrow);
             vw[u][0] = v.x; vw[u][1] = v.y; vw[u][2] = v.z; vw[u][3] = v.w;
           } else {
@@ -263,44 +272,46 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
       const int row = q0 + wave * WR + mt * 16 + 4 * g + i;
       if (row < p.n_q) {
         uint16_t* dst = p.o + ((int64_t)row * p.num_qo_heads + qh) * D + DC * r;
-        if constexpr (DC == 8) {
-          u32x4 out;
-          out.x = pack2<T>(oacc[mt][0][i] * inv, oacc[mt][1][i] * inv);
-          out.y = pack2<T>(oacc[mt][2][i] * inv, oacc[mt][3][i] * inv);
-          out.z = pack2<T>(oacc[mt][4][i] * inv, oacc[mt][5][i] * inv);
-          out.w = pack2<T>(oacc[mt][6][i] * inv, oacc[mt][7][i] * inv);
-          *reinterpret_cast<u32x4*>(dst) = out;
+        uint32_t ow[DC / 2];
+#pragma unroll
+        for (int c = 0; c < DC / 2; ++c)
+          ow[c] = pack2<T>(oacc[mt][2 * c][i] * inv, oacc[mt][2 * c + 1][i] * inv);
+        if constexpr (DC == 4) {
+          *reinterpret_cast<u32x2*>(dst) = u32x2{ow[0], ow[1]};
         } else {
-          u32x2 out;
-          out.x = pack2<T>(oacc[mt][0][i] * inv, oacc[mt][1][i] * inv);
-          out.y = pack2<T>(oacc[mt][2][i] * inv, oacc[mt][3][i] * inv);
-          *reinterpret_cast<u32x2*>(dst) = out;
+#pragma unroll
+          for (int c = 0; c < DC / 8; ++c)
+            *reinterpret_cast<u32x4*>(dst + 8 * c) =
+                u32x4{ow[4 * c], ow[4 * c + 1], ow[4 * c + 2], ow[4 * c + 3]};
         }
       }
     }
   }
 }
 
-template <typename T, int MT>
-static int launch_prefill_mt(const PrefillParams& p, int head_dim, hipStream_t st) {
-  const dim3 grid((p.n_q + 64 * MT - 1) / (64 * MT), p.num_qo_heads), block(kPfThreads);
-  if (head_dim == 128)
-    hipLaunchKernelGGL((prefill_attn_kernel<T, 128, MT>), grid, block, 0, st, p);
-  else if (head_dim == 64)
-    hipLaunchKernelGGL((prefill_attn_kernel<T, 64, MT>), grid, block, 0, st, p);
-  else
-    return fail(TD_ERR_UNSUPPORTED, "BatchPrefillWithPagedKVCache failed to dispatch with head_dim %d",
-                head_dim);
-  return TD_OK;
-}
-
 template <typename T>
 static int launch_prefill(const PrefillParams& p, int head_dim, hipStream_t st) {
-  // Two query tiles per wavefront keep the kernel at 256 registers, i.e. two workgroups per
-  // compute unit: one computes while the other waits for its next K/V tile.  Four tiles per
-  // wavefront halve the LDS traffic per flop but run one workgroup per compute unit with every
-  // memory and barrier latency exposed (measured: 2.5x slower).
-  return launch_prefill_mt<T, 2>(p, head_dim, st);
+  // Two query tiles per wavefront and 64-token key tiles keep the kernel at 256 registers, i.e.
+  // two workgroups per compute unit: one computes while the other waits for its next K/V tile.
+  // (Four query tiles per wavefront halve the LDS traffic per flop but run one workgroup per
+  // compute unit with every memory and barrier latency exposed: 2.5x slower.)  head_dim 256 has
+  // twice the accumulators and twice the LDS per token: one query tile per wavefront, 32-token
+  // key tiles.
+  const dim3 block(kPfThreads);
+  if (head_dim == 128)
+    hipLaunchKernelGGL((prefill_attn_kernel<T, 128, 2, 64>), dim3((p.n_q + 127) / 128, p.num_qo_heads),
+                       block, 0, st, p);
+  else if (head_dim == 64)
+    hipLaunchKernelGGL((prefill_attn_kernel<T, 64, 2, 64>), dim3((p.n_q + 127) / 128, p.num_qo_heads),
+                       block, 0, st, p);
+  else if (head_dim == 256)
+    hipLaunchKernelGGL((prefill_attn_kernel<T, 256, 1, 32>), dim3((p.n_q + 63) / 64, p.num_qo_heads),
+                       block, 0, st, p);
+  else
+    return fail(TD_ERR_UNSUPPORTED,
+                "BatchPrefillWithPagedKVCache failed to dispatch with head_dim %d (supported: 64, 128, 256)",
+                head_dim);
+  return TD_OK;
 }
 
 }  // namespace tidal
