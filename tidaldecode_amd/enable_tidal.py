@@ -9,7 +9,7 @@ The reference replaces ``forward`` of every attention module by a closure that c
 library's kernels over a paged KV cache that is shared by all layers through one state object
 on the model, and the persisted selection is the token list inside that state:
 
-    prefill (q_len > 1)            causal attention (torch SDPA), K/V appended to the paged cache
+    prefill (q_len > 1)            K/V appended to the paged cache, causal attention kernel over it
     decode, layer < sparse_layer_start                 full attention kernel
     decode, layer == sparse_layer_start / correction   full attention + logits -> top-k
     decode, other layers                               sparse attention over the persisted list
