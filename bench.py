@@ -152,7 +152,7 @@ class Workload:
         from tidaldecode_amd import _kernels
 
         if self._probe_out is None:
-            self._probe_out = self.torch.empty(self.H * 64 * 8, dtype=self.torch.int32,
+            self._probe_out = self.torch.empty(self.H * 64 * 16, dtype=self.torch.int32,
                                                device=self.dev)
         return _kernels.gather_probe(self.c._decode_handler._wrapper,
                                      self.c.kv_cache.buf_layer(layer), self.c.topk_dindices_buffer,
@@ -468,8 +468,7 @@ def main():
             r_plain, _ = capture(torch, run_sparse_plain, use_graph)
             entry["sparse_unfused_us_per_layer"] = (time_events(torch, r_plain, max(args.steps, 20))
                                                     * 1e3 / len(sparse))
-        if w.H == w.HKV and w.c.index_rows in (1, w.H) and args.layout == "NHD" and not args.waves \
-                and not args.chunk and not args.rows:
+        if w.H == w.HKV and w.c.index_rows in (1, w.H) and args.layout == "NHD":
             # the same lists gathered by a kernel that does nothing else: the memory floor of the launch
             def run_probe():
                 for layer in sparse:

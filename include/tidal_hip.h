@@ -281,7 +281,7 @@ int td_rms_norm(const void* x, const void* weight, void* out, int32_t rows, int3
  * alone.  Same grid and the same list -> slot -> K / V row loads as td_decode_attn for
  * token-slot lists (the launch that replaces BatchDecodeWithPagedKVCacheKernel,
  * kernels/include/decode/decode_attn.cuh:432-658), no arithmetic and no merge; one word per
- * wavefront is written to out (batch * head rows * plan->max_splits * 8 words).  bench.py times
+ * wavefront is written to out (batch * head rows * plan->max_splits * plan->waves_per_block words).  bench.py times
  * it next to the attention launch.
  */
 int td_gather_probe(const td_paged_kv* kv, const td_index_list* list, const td_decode_plan* plan,

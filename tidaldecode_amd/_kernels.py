@@ -554,7 +554,7 @@ def gather_probe(wrapper: "BatchDecodeWithPagedKVCachePyTorchWrapper", paged_kv_
     lst.kind = TD_IDX_SLOTS
     lst.n_list_host = budget
     plan = wrapper._plan(1, rows, budget)
-    words = hq * int(plan.max_splits) * 8
+    words = hq * int(plan.max_splits) * int(plan.waves_per_block)
     if out is None:
         out = torch.empty(words, dtype=torch.int32, device=slots.device)
     check(lib.td_gather_probe(pool, lst, plan, 1, hq, out.data_ptr(), out.numel() * 4, _stream()))

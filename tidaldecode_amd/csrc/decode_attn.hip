@@ -329,18 +329,25 @@ extern "C" int td_gather_probe(const td_paged_kv* kv, const td_index_list* list,
   const int prc = build_params(kv, list, plan, out, out, batch, num_qo_heads, 1.f, nullptr, TD_F32, 0,
                                nullptr, nullptr, out, (int64_t)1 << 40, p, qpg, n_hrows);
   if (prc != TD_OK) return prc;
+  const int nw = plan->waves_per_block, rows = plan->tile_rows;
   if (!(list->kind == TD_IDX_SLOTS && p.lean && qpg == 1 && kv->head_dim == 128 &&
-        plan->waves_per_block == 8 && plan->tile_rows == 4 && list->last_page_len == 0 &&
-        !list->last_page_len_arr))
+        ((nw == 8 && (rows == 4 || rows == 2)) || (nw == 16 && rows == 4)) &&
+        list->last_page_len == 0 && !list->last_page_len_arr))
     return fail(TD_ERR_UNSUPPORTED,
                 "td_gather_probe: token-slot lists without a forced last page, one query head per "
-                "row, head_dim 128, power-of-two pages, pool below 4 GiB, 8 waves x 4 rows only");
-  TD_REQUIRE(out_bytes >= (int64_t)batch * n_hrows * plan->max_splits * 8 * 4,
+                "row, head_dim 128, power-of-two pages, pool below 4 GiB only");
+  TD_REQUIRE(out_bytes >= (int64_t)batch * n_hrows * plan->max_splits * nw * 4,
              "td_gather_probe: out holds %lld bytes, %lld needed", (long long)out_bytes,
-             (long long)batch * n_hrows * plan->max_splits * 8 * 4);
-  hipLaunchKernelGGL((gather_probe_kernel<128, 4, 8>), dim3(n_hrows, plan->max_splits, batch),
-                     dim3(512), 0, reinterpret_cast<hipStream_t>(stream), p,
-                     reinterpret_cast<uint32_t*>(out));
+             (long long)batch * n_hrows * plan->max_splits * nw * 4);
+  const dim3 grid(n_hrows, plan->max_splits, batch);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  uint32_t* outw = reinterpret_cast<uint32_t*>(out);
+  if (nw == 16)
+    hipLaunchKernelGGL((gather_probe_kernel<128, 4, 16>), grid, dim3(1024), 0, st, p, outw);
+  else if (rows == 2)
+    hipLaunchKernelGGL((gather_probe_kernel<128, 2, 8>), grid, dim3(512), 0, st, p, outw);
+  else
+    hipLaunchKernelGGL((gather_probe_kernel<128, 4, 8>), grid, dim3(512), 0, st, p, outw);
   TD_HIP_CHECK(hipGetLastError());
   return TD_OK;
 }
