@@ -60,6 +60,9 @@ def parse():
                          "attention (the grid of the reference's latency figure), one JSON object")
     ap.add_argument("--no-prefill", action="store_true",
                     help="skip the prefill-attention leg (one layer, causal, whole context)")
+    ap.add_argument("--e2e-shape", default="llama2_7b", choices=["llama2_7b", "llama3_8b"],
+                    help="decoder shape of the end-to-end leg (llama3_8b: GQA 32/8, selection at "
+                         "layers 0 and 13)")
     ap.add_argument("--e2e-ctx", type=str, default="32768,102400",
                     help="context lengths of the end-to-end leg")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -262,8 +265,12 @@ def e2e_leg(args):
     from tidaldecode_amd.llama import TidalLlama, TidalLlamaConfig
 
     ctxs = [int(x) for x in args.e2e_ctx.split(",") if x]
-    cfg = TidalLlamaConfig.llama2_7b(top_k=args.top_k, sparse_layer_start=0, correction_layer=2,
-                                     select_mode=args.select_mode)
+    if args.e2e_shape == "llama3_8b":
+        cfg = TidalLlamaConfig.llama3_8b(top_k=args.top_k, sparse_layer_start=0, correction_layer=13,
+                                         select_mode=args.select_mode)
+    else:
+        cfg = TidalLlamaConfig.llama2_7b(top_k=args.top_k, sparse_layer_start=0, correction_layer=2,
+                                         select_mode=args.select_mode)
     model = TidalLlama(cfg, "cuda:0", seed=0)
     model.tidal_init(page_size=16, max_seq_len=max(ctxs) + 128, page_order_seed=0)
     out = {}
@@ -579,7 +586,7 @@ def main():
         line["prefill_attn"] = prefill_leg(args)
         line["batch8_sparse_attn"] = batch8_leg(args)
     if not args.no_e2e and not args.only_sparse:
-        line["e2e_decode_llama2_7b_shape"] = e2e_leg(args)
+        line[f"e2e_decode_{args.e2e_shape}_shape"] = e2e_leg(args)
     if not args.no_cpu and not args.only_sparse:
         line["cpu_baseline"] = cpu_baseline(args)
     print(json.dumps(line))
