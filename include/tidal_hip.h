@@ -305,7 +305,7 @@ int td_prefill_attn(const td_paged_kv* kv, const int32_t* page_table, int32_t n_
  * (eps); 2: f(x) = silu(x[:cols]) * x[cols:2 cols] (gated MLP).  residual (or NULL) is added to
  * the result and may alias y.  pair_gated != 0: rows is even and y has rows/2 entries,
  * y[i] = silu(W[i] . f(x)) * (W[i + rows/2] . f(x)) (gate and up projections stacked in W).
- * cols: multiple of 8, at most 16384; w and x 16-byte aligned.
+ * cols: multiple of 8, at most 30720; w and x 16-byte aligned.
  * Serves the decoder harness around the attention path, where the reference calls torch's
  * nn.Linear, LlamaRMSNorm and act_fn one by one (tidal/models/SparseAttention.py:122-124,216,
  * tidal/models/llama.py:99,108-122,563-578).

@@ -34,7 +34,7 @@ def _ref(w, x, norm_weight, eps, gated, residual, dtype):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("rows,cols,mode", [(4096, 4096, "plain"), (12288, 4096, "norm"),
                                             (4096, 11008, "gated"), (22016, 4096, "norm"),
-                                            (37, 4096, "plain"), (5, 8, "plain"), (129, 16384, "gated"),
+                                            (37, 4096, "plain"), (5, 8, "plain"), (129, 16384, "gated"), (64, 28672, "plain"), (32, 30720, "norm"),
                                             (32000, 4096, "norm"), (1000, 2056, "norm")])
 @pytest.mark.parametrize("with_residual", [False, True])
 def test_gemv_matches_fp32_reference(cuda, dtype, rows, cols, mode, with_residual):
@@ -101,4 +101,4 @@ def test_gemv_errors(cuda):
         _kernels.gemv(w, torch.zeros(24, dtype=torch.float16, device=cuda))
     with pytest.raises(RuntimeError):
         _kernels.gemv(torch.zeros((4, 32768), dtype=torch.bfloat16, device=cuda),
-                      torch.zeros(32768, dtype=torch.bfloat16, device=cuda))
+                      torch.zeros(32768, dtype=torch.bfloat16, device=cuda))    # cols > 30720

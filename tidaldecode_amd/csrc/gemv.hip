@@ -17,7 +17,7 @@ namespace tidal {
 
 constexpr int kGemvThreads = 256;
 constexpr int kGemvWaves = kGemvThreads / 64;
-constexpr int kGemvMaxCols = 16384; // x in LDS: 32 KiB
+constexpr int kGemvMaxCols = 30720; // x in LDS: 60 KiB (covers the 28672-wide MLP of 70B-class models)
 
 struct GemvParams {
   const uint16_t* w;
@@ -226,8 +226,10 @@ static void launch_gemv_shape(const GemvParams& p, int mode, bool pair, hipStrea
     launch_gemv_x<T, R, UN, 2>(p, mode, pair, st);
   else if (per_thread <= 6)
     launch_gemv_x<T, R, UN, 6>(p, mode, pair, st);
-  else
+  else if (per_thread <= 8)
     launch_gemv_x<T, R, UN, 8>(p, mode, pair, st);
+  else
+    launch_gemv_x<T, R, UN, 15>(p, mode, pair, st);
 }
 
 // Tall matrices: four rows per wavefront (fewer, longer-lived waves stream better); short ones:
