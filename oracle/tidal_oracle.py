@@ -86,13 +86,13 @@ def page_score_bound(q: torch.Tensor, k: torch.Tensor, page_size: int) -> torch.
     n, hkv, d = k.shape
     hq = q.shape[0]
     n_pages = (n + page_size - 1) // page_size
-    out = torch.empty((hq, n_pages))
-    for pg in range(n_pages):
-        rows = k[pg * page_size: (pg + 1) * page_size]          # [<=P, H_kv, D]
-        mx = rows.max(0).values.repeat_interleave(hq // hkv, 0)  # [H_q, D]
-        mn = rows.min(0).values.repeat_interleave(hq // hkv, 0)
-        out[:, pg] = torch.maximum(q * mx, q * mn).sum(-1)
-    return out
+    pad = n_pages * page_size - n
+    inf = torch.full((pad, hkv, d), float("inf"))
+    mx = torch.cat([k, -inf]).view(n_pages, page_size, hkv, d).max(1).values  # [pages, H_kv, D]
+    mn = torch.cat([k, inf]).view(n_pages, page_size, hkv, d).min(1).values
+    mx = mx.repeat_interleave(hq // hkv, 1)                                    # [pages, H_q, D]
+    mn = mn.repeat_interleave(hq // hkv, 1)
+    return torch.maximum(q[None] * mx, q[None] * mn).sum(-1).t().contiguous()  # [H_q, pages]
 
 
 def head_sum_scores(logits: torch.Tensor, rows: int = 1) -> torch.Tensor:

@@ -246,3 +246,42 @@ def test_page_score_estimator(cuda, dtype, hq, hkv, d, page, layout):
         want = want[:, : n_pages - 1]
         tol = (2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7) * want.abs().clamp(min=1.0) + 1e-3
         assert ((got.float().cpu() - want).abs() <= tol).all()
+
+
+@pytest.mark.parametrize("head_dim", [64, 128])
+@pytest.mark.parametrize("page_size", [1, 3, 7, 16, 32])
+def test_page_score_estimator_reference_grid(cuda, head_dim, page_size):
+    """The reference's estimator test grid (kernels/src/test/test_max_possible.cu:158-165: ten
+    sequence lengths x five page sizes x two head dims, 32 heads, fp16) at the kernel boundary:
+    the metadata pool is filled with the brute-force per-page key max / min."""
+    from oracle import tidal_oracle as orc
+    from tidaldecode_amd import _kernels
+
+    h, dtype = 32, torch.float16
+    for n in (65, 127, 213, 1110, 2000, 4099, 8192, 8222, 12345, 28837):
+        g = torch.Generator().manual_seed(n * 31 + page_size)
+        k = torch.randn((n, h, head_dim), generator=g).to(dtype)
+        q = torch.randn((1, h, head_dim), generator=g).to(dtype)
+        n_kv_pages = (n + page_size - 1) // page_size            # one metadata entry per KV page
+        n_meta_pages = (n_kv_pages + page_size - 1) // page_size
+        pad = n_kv_pages * page_size - n
+        kf = k.float()
+        mx = torch.cat([kf, torch.full((pad, h, head_dim), -65504.0)]).view(n_kv_pages, page_size, h, head_dim).max(1).values
+        mn = torch.cat([kf, torch.full((pad, h, head_dim), 65504.0)]).view(n_kv_pages, page_size, h, head_dim).min(1).values
+        table = torch.randperm(n_meta_pages + 2, generator=g)[:n_meta_pages]
+        meta = torch.full((n_meta_pages + 2, 2, page_size, h, head_dim), 7.0)
+        epad = n_meta_pages * page_size - n_kv_pages
+        meta[table, 0] = torch.cat([mx, torch.zeros(epad, h, head_dim)]).view(n_meta_pages, page_size, h, head_dim)
+        meta[table, 1] = torch.cat([mn, torch.zeros(epad, h, head_dim)]).view(n_meta_pages, page_size, h, head_dim)
+        last_len = (n_kv_pages - 1) % page_size + 1
+        n_out = n_kv_pages - 1
+        o = torch.full((h, max(n_out, 1)), float("nan"), dtype=dtype, device=cuda)
+        _kernels.estimate_attn_score(q.to(cuda), o, meta.to(dtype).to(cuda),
+                                     table.to(torch.int32).to(cuda), None, last_len,
+                                     int(table[-1]), 0)
+        torch.cuda.synchronize()
+        if n_out == 0:
+            continue
+        want = orc.page_score_bound(q[0].float(), kf, page_size)[:, :n_out]
+        tol = 2.0 ** -10 * want.abs().clamp(min=1.0) + 1e-3
+        assert ((o[:, :n_out].float().cpu() - want).abs() <= tol).all(), (n, page_size, head_dim)
