@@ -72,6 +72,28 @@ def test_head_layouts_page_sizes_and_non_causal(cuda, hq, hkv, d, page, layout, 
     assert ((got.float().cpu() - want).abs() <= ATOL[dtype] * want.abs().clamp(min=1.0)).all()
 
 
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("head_dim", [64, 128])
+@pytest.mark.parametrize("page_size", [1, 8, 16])
+@pytest.mark.parametrize("hq,hkv", [(32, 4), (32, 8), (32, 32), (8, 1), (8, 2), (8, 8)])
+def test_reference_prefill_grid(cuda, hq, hkv, page_size, head_dim, causal):
+    """The reference's prefill test grid (kernels/src/test/test_prefill.cu:408-467): its three
+    families of lengths -- a few queries over a short cache (q in [1, 15), kv in [15, 257)), a fresh
+    short prompt (q = kv in [1, 64)) and 63 queries over 2047 cached tokens -- with seeded draws."""
+    dtype = torch.float16
+    g = torch.Generator().manual_seed(hq * 1000 + hkv * 100 + page_size * 10 + head_dim + causal)
+    q1 = int(torch.randint(1, 15, (1,), generator=g))
+    kv1 = int(torch.randint(15, 257, (1,), generator=g))
+    q2 = int(torch.randint(1, 64, (1,), generator=g))
+    for n_q, kv_len in ((q1, kv1), (q2, q2), (63, 2047)):
+        case = PagedCase(kv_len, hkv, head_dim, page_size, dtype, seed=kv_len + n_q + hkv)
+        q = randn((n_q, hq, head_dim), n_q * 7 + kv_len, dtype)
+        want = _dense(q, case.k, case.v, causal)
+        got = _run(cuda, case, q, causal, dtype)
+        assert ((got.float().cpu() - want).abs() <= ATOL[dtype] * want.abs().clamp(min=1.0)).all(), \
+            (n_q, kv_len)
+
+
 def test_prefill_at_benchmark_length(cuda):
     """32768 tokens, Llama-2-7B head shape (4 of the 32 heads, GQA 4/2): checked on sampled rows
     against the oracle's single-query attention over the row's causal prefix."""
