@@ -141,6 +141,14 @@ def test_kv_pool_and_cache_bookkeeping():
     assert hnd.pool.buf.shape == (1, 2, 2, 4, 16, 8)
     hnd.append_seq(32)
     assert sorted(hnd.indicies) == [0, 1]
+    assert TensorLayout.FORMAT2STR == {0: "NHD", 1: "HND"}
+    with pytest.raises(KeyError, match="Invalide kv_layout"):
+        TensorLayout.parse("nhd")
+    page = hnd.pool.alloc_block() if hnd.pool.num_free_blocks else None
+    assert page is None                                         # both pages are held
+    hnd.pool.free_block(hnd.indicies[0])
+    with pytest.raises(AssertionError):                         # returning a page twice
+        hnd.pool.free_block(hnd.indicies[0])
 
 
 @pytest.mark.parametrize("scope", ["all", "exclude_last_page"])

@@ -11,9 +11,7 @@ import torch
 
 from .. import _kernels
 from .controller import InferenceController
-from .decode_wrapper import BatchDecodeWithPagedKVCacheWrapper
-from .kv_cache import KvCache, KvPool
-from .utils import TensorLayout
+from .paged import BatchDecodeWithPagedKVCacheWrapper, KvCache, KvPool, TensorLayout
 
 __all__ = [
     "TensorLayout",

@@ -21,9 +21,7 @@ from typing import Optional
 
 import torch
 
-from .decode_wrapper import BatchDecodeWithPagedKVCacheWrapper
-from .kv_cache import KvCache
-from .utils import TensorLayout
+from .paged import BatchDecodeWithPagedKVCacheWrapper, KvCache, TensorLayout
 
 _SELECT_MODES = ("per_head", "group_sum", "head_sum")
 _SELECT_SCOPES = ("all", "exclude_last_page")
@@ -41,7 +39,7 @@ class InferenceController:
         num_kv_heads = num_heads if num_kv_heads is None else num_kv_heads
         if num_heads % num_kv_heads != 0:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
-        self.layout = getattr(TensorLayout, kv_layout)
+        self.layout = TensorLayout.parse(kv_layout)
         self.kv_cache = KvCache(num_layers=num_layers, num_heads=num_kv_heads, head_dim=head_dim,
                                 max_seq_len=max_seq_len, page_size=page_size, dtype=dtype,
                                 device=device, layout=self.layout,

@@ -1,7 +1,2 @@
-class TensorLayout:
-    """Layout of the last three page dimensions (tidal/utils/utils.py:1-5 of the reference)."""
-
-    NHD = 0
-    HND = 1
-
-    FORMAT2STR = {0: "NHD", 1: "HND"}
+"""Import path of the reference's tidal.utils.utils; the enum is defined in ``paged``."""
+from .paged import TensorLayout  # noqa: F401
