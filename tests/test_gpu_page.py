@@ -198,7 +198,8 @@ def test_fused_rope_append_equals_the_two_calls(cuda, dtype, layout):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("rows,cols", [(1, 4096), (7, 5120), (300, 128), (2, 33)])
+@pytest.mark.parametrize("rows,cols", [(1, 4096), (7, 5120), (300, 128), (2, 33), (1, 8), (5, 2056),
+                                       (3, 8192), (2, 16384), (2, 16392), (3, 20000)])
 def test_rms_norm(cuda, dtype, rows, cols):
     from tidaldecode_amd import _kernels
 
@@ -209,6 +210,14 @@ def test_rms_norm(cuda, dtype, rows, cols):
     _kernels.rms_norm_forward(x.to(dtype).to(cuda), w.to(dtype).to(cuda), out, 1e-5)
     torch.cuda.synchronize()
     assert ((out.float().cpu() - want).abs() <= ULP[dtype] * 1.01 * want.abs() + 1e-6).all()
+    # the same rows at an address that is not 16-byte aligned (2-byte access path)
+    flat = torch.zeros(rows * cols + 8, dtype=dtype, device=cuda)
+    flat[4:4 + rows * cols] = x.to(dtype).to(cuda).flatten()
+    out2 = torch.empty_like(out)
+    _kernels.rms_norm_forward(flat[4:4 + rows * cols].view(1, rows, cols), w.to(dtype).to(cuda), out2,
+                              1e-5)
+    torch.cuda.synchronize()
+    assert ((out2.float().cpu() - want).abs() <= ULP[dtype] * 1.01 * want.abs() + 1e-6).all()
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])

@@ -231,7 +231,67 @@ __global__ __launch_bounds__(256) void estimate_kernel(PoolGeom mg, const int32_
   if (li == 0 && e < n_entries) o[(int64_t)h * o_stride + e] = from_float<T>(acc);
 }
 
-// RMSNorm, one 256-thread workgroup per row, fp32 accumulation
+// RMSNorm, one 256-thread workgroup per row, fp32 accumulation.
+// Sum of squares over the workgroup: every wave reduces by butterfly, four partials through LDS.
+__device__ __forceinline__ float rms_block_sum(float ss) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+  __shared__ float part[4];
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  return part[0] + part[1] + part[2] + part[3];
+}
+
+// Rows of up to CH*2048 elements with 16-byte alignment: the row is read once, as CH independent
+// 16-byte loads per thread issued back to back, and stays in registers between the two passes.
+// Threads past the end of the row reload the row's last chunk (an unconditional load keeps all
+// loads in flight together; a predicated one is waited for inside its branch) and drop it.
+template <typename T, int CH>
+__global__ __launch_bounds__(256) void rms_norm_vec_kernel(const uint16_t* x, const uint16_t* w,
+                                                           uint16_t* out, int cols, float eps) {
+  const int64_t base = (int64_t)blockIdx.x * cols;
+  uint4 xv[CH], wv[CH];
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    const int c = min((i * 256 + (int)threadIdx.x) * 8, cols - 8);
+    xv[i] = *reinterpret_cast<const uint4*>(x + base + c);
+  }
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    const int c = min((i * 256 + (int)threadIdx.x) * 8, cols - 8);
+    wv[i] = *reinterpret_cast<const uint4*>(w + c);
+  }
+  float xf[CH][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    const uint32_t xw[4] = {xv[i].x, xv[i].y, xv[i].z, xv[i].w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) unpack2<T>(xw[j], xf[i][2 * j], xf[i][2 * j + 1]);
+    if ((i * 256 + (int)threadIdx.x) * 8 < cols) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss = fmaf(xf[i][j], xf[i][j], ss);
+    }
+  }
+  const float inv = rsqrtf(rms_block_sum(ss) / (float)cols + eps);
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    const int c = (i * 256 + (int)threadIdx.x) * 8;
+    if (c < cols) {
+      const uint32_t ww[4] = {wv[i].x, wv[i].y, wv[i].z, wv[i].w};
+      uint32_t ow[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float w0, w1;
+        unpack2<T>(ww[j], w0, w1);
+        ow[j] = pack2<T>(xf[i][2 * j] * inv * w0, xf[i][2 * j + 1] * inv * w1);
+      }
+      *reinterpret_cast<uint4*>(out + base + c) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+    }
+  }
+}
+
+// Any other row length or alignment: two passes of 2-byte accesses.
 template <typename T>
 __global__ __launch_bounds__(256) void rms_norm_kernel(const uint16_t* x, const uint16_t* w,
                                                        uint16_t* out, int cols, float eps) {
@@ -239,19 +299,33 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const uint16_t* x, const 
   const uint16_t* xr = x + (int64_t)row * cols;
   uint16_t* orow = out + (int64_t)row * cols;
   float ss = 0.f;
+#pragma unroll 4
   for (int c = threadIdx.x; c < cols; c += 256) {
     const float f = to_float<T>(xr[c]);
     ss = fmaf(f, f, ss);
   }
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
-  __shared__ float part[4];
-  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
-  __syncthreads();
-  const float total = part[0] + part[1] + part[2] + part[3];
-  const float inv = rsqrtf(total / (float)cols + eps);
+  const float inv = rsqrtf(rms_block_sum(ss) / (float)cols + eps);
+#pragma unroll 4
   for (int c = threadIdx.x; c < cols; c += 256)
     orow[c] = from_float<T>(to_float<T>(xr[c]) * inv * to_float<T>(w[c]));
+}
+
+template <typename T>
+static void launch_rms_norm(const void* x, const void* weight, void* out, int rows, int cols,
+                            float eps, hipStream_t st) {
+  const uint16_t* xp = (const uint16_t*)x;
+  const uint16_t* wp = (const uint16_t*)weight;
+  uint16_t* op = (uint16_t*)out;
+  const bool vec = cols % 8 == 0 && cols <= 8 * 2048 &&
+                   (((uintptr_t)x | (uintptr_t)weight | (uintptr_t)out) & 15) == 0;
+#define TD_RMS(CH) \
+  hipLaunchKernelGGL((rms_norm_vec_kernel<T, CH>), dim3(rows), dim3(256), 0, st, xp, wp, op, cols, eps)
+  if (!vec) hipLaunchKernelGGL(rms_norm_kernel<T>, dim3(rows), dim3(256), 0, st, xp, wp, op, cols, eps);
+  else if (cols <= 2048) TD_RMS(1);
+  else if (cols <= 2 * 2048) TD_RMS(2);
+  else if (cols <= 4 * 2048) TD_RMS(4);
+  else TD_RMS(8);
+#undef TD_RMS
 }
 
 static int check_pool(const td_paged_kv* kv, const char* who) {
@@ -446,11 +520,9 @@ extern "C" int td_rms_norm(const void* x, const void* weight, void* out, int32_t
   if (rows == 0) return TD_OK;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   if (dtype == TD_F16)
-    hipLaunchKernelGGL(rms_norm_kernel<F16>, dim3(rows), dim3(256), 0, st, (const uint16_t*)x,
-                       (const uint16_t*)weight, (uint16_t*)out, cols, eps);
+    launch_rms_norm<F16>(x, weight, out, rows, cols, eps, st);
   else if (dtype == TD_BF16)
-    hipLaunchKernelGGL(rms_norm_kernel<BF16>, dim3(rows), dim3(256), 0, st, (const uint16_t*)x,
-                       (const uint16_t*)weight, (uint16_t*)out, cols, eps);
+    launch_rms_norm<BF16>(x, weight, out, rows, cols, eps, st);
   else
     return fail(TD_ERR_UNSUPPORTED, "rms_norm_forward failed to dispatch with dtype %d", dtype);
   TD_HIP_CHECK(hipGetLastError());
