@@ -87,15 +87,11 @@ __device__ __forceinline__ uint32_t pack2<F16>(float lo, float hi) {
   h.y = (_Float16)hi;
   return __builtin_bit_cast(uint32_t, h);
 }
-__device__ __forceinline__ uint32_t bf16_bits_rne(float f) {
-  uint32_t u = __builtin_bit_cast(uint32_t, f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;  // quiet NaN
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return u >> 16;
-}
+// gfx950 converts in hardware (v_cvt_pk_bf16_f32: round to nearest even, NaN stays NaN)
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 template <>
 __device__ __forceinline__ uint32_t pack2<BF16>(float lo, float hi) {
-  return bf16_bits_rne(lo) | (bf16_bits_rne(hi) << 16);
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, bf16x2));
 }
 
 // scalar conversions (used by the small kernels)
@@ -117,7 +113,7 @@ __device__ __forceinline__ uint16_t from_float<F16>(float f) {
 }
 template <>
 __device__ __forceinline__ uint16_t from_float<BF16>(float f) {
-  return (uint16_t)bf16_bits_rne(f);
+  return __builtin_bit_cast(uint16_t, (__bf16)f);
 }
 
 // ---------------------------------------------------------------------------------------------
