@@ -24,6 +24,15 @@ namespace tidal {
 
 constexpr int kPfThreads = 256;
 
+// LDS read with transpose (gfx950): within every 16 lanes, lane 4a + b receives element b of the
+// four 8-byte pieces addressed by lanes a, a + 4, a + 8, a + 12.
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x2 lds_read_tr16(const uint16_t* at) {
+  const i16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (__attribute__((address_space(3))) i16x4*)(at));
+  return __builtin_bit_cast(u32x2, v);
+}
+
 struct PrefillParams {
   const uint16_t* kv;
   int64_t page_stride, v_offset;  // elements
@@ -45,13 +54,15 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
   constexpr int WR = 16 * MT;       // query rows per wavefront
   constexpr int NS = D / 32;        // 16-byte pieces of a Q/K row per lane (one MFMA each)
   constexpr int DC = D / 16;        // head dimensions per lane in the P.V product
-  constexpr int PITCH = D + 8;      // LDS row pitch in elements: +16 bytes
+  constexpr int PITCH = D + 16;     // LDS row pitch in elements: +32 bytes (see the layout note)
   constexpr int CPR = D / 8;        // 16-byte chunks per row
   constexpr int kPfBN = BN;
   constexpr int NSUB = BN / 16;     // 16-token sub-tiles per key tile
-  constexpr int CPT = kPfBN * CPR / kPfThreads;  // chunks a thread stages per tile and matrix
+  constexpr int RPT = BN / 32;      // staging: rows per thread (row = tid / 8 + 32 jr)
+  constexpr int CCT = CPR / 8;      // staging: chunks per thread and row (chunk = tid % 8 + 8 jc)
+  constexpr int CPT = RPT * CCT;    // chunks a thread stages per tile and matrix
   static_assert(D == 64 || D == 128 || D == 256, "head dimensions of the prefill kernel");
-  static_assert(BN % 32 == 0 && CPT >= 1, "key tile");
+  static_assert(BN % 32 == 0 && CPT * kPfThreads == BN * CPR, "key tile");
   __shared__ __attribute__((aligned(16))) uint16_t ks[kPfBN * PITCH];
   __shared__ __attribute__((aligned(16))) uint16_t vs[kPfBN * PITCH];
 
@@ -93,13 +104,14 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
   const int kv_end = p.causal ? (q_off + last_row + 1) : p.kv_len;
 
   // ---- staging: thread -> CPT chunks of K and of V per tile --------------------------------------
+  // eight adjacent lanes move 128 contiguous bytes of one row (one cache line in, one conflict-free
+  // LDS write out); a thread looks up the page of each of its RPT rows once
   u32x4 kreg[CPT], vreg[CPT];
+  const int srow = tid >> 3, sl8 = tid & 7;
   auto fetch = [&](int kt) {
 #pragma unroll
-    for (int j = 0; j < CPT; ++j) {
-      const int c = tid + j * kPfThreads;
-      const int row = c / CPR, cc = c % CPR;
-      int tok = kt + row;
+    for (int jr = 0; jr < RPT; ++jr) {
+      int tok = kt + srow + 32 * jr;
       tok = tok < p.kv_len ? tok : p.kv_len - 1;
       int pg_i, entry;
       if (p.page_shift >= 0) {
@@ -111,20 +123,24 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
       }
       uint32_t page = (uint32_t)p.page_table[pg_i];
       page = page > p.max_page ? p.max_page : page;
-      const int64_t off = (int64_t)page * p.page_stride + (int64_t)entry * p.entry_stride +
-                          (int64_t)kvh * p.head_stride + cc * 8;
-      kreg[j] = *reinterpret_cast<const u32x4*>(p.kv + off);
-      vreg[j] = *reinterpret_cast<const u32x4*>(p.kv + off + p.v_offset);
+      const uint16_t* src = p.kv + ((int64_t)page * p.page_stride + (int64_t)entry * p.entry_stride +
+                                    (int64_t)kvh * p.head_stride + sl8 * 8);
+#pragma unroll
+      for (int jc = 0; jc < CCT; ++jc) {
+        kreg[jr * CCT + jc] = *reinterpret_cast<const u32x4*>(src + jc * 64);
+        vreg[jr * CCT + jc] = *reinterpret_cast<const u32x4*>(src + jc * 64 + p.v_offset);
+      }
     }
   };
   auto stash = [&]() {
 #pragma unroll
-    for (int j = 0; j < CPT; ++j) {
-      const int c = tid + j * kPfThreads;
-      const int row = c / CPR, cc = c % CPR;
-      *reinterpret_cast<u32x4*>(&ks[row * PITCH + cc * 8]) = kreg[j];
-      *reinterpret_cast<u32x4*>(&vs[row * PITCH + cc * 8]) = vreg[j];
-    }
+    for (int jr = 0; jr < RPT; ++jr)
+#pragma unroll
+      for (int jc = 0; jc < CCT; ++jc) {
+        const int at = (srow + 32 * jr) * PITCH + (sl8 + 8 * jc) * 8;
+        *reinterpret_cast<u32x4*>(&ks[at]) = kreg[jr * CCT + jc];
+        *reinterpret_cast<u32x4*>(&vs[at]) = vreg[jr * CCT + jc];
+      }
   };
 
   const int wave_first_pos = q_off + q0 + wave * WR;  // position of the wave's first query row
@@ -210,44 +226,24 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
         }
       }
       // ---- O += P V, 32 tokens (two sub-tiles) per matrix instruction ------------------------------
+      // B operand of head dimensions [16 a, 16 a + 16): lane (r, g) needs dimension 16 a + r of the
+      // tokens 4g..4g+3 of both sub-tiles.  ds_read_b64_tr_b16 transposes a 4 token x 16 dimension
+      // block inside every 16 lanes: lane r points at the 8-byte piece r % 4 of token row r / 4
+      // and receives dimension r of the four rows.
+      const uint16_t* vlane = &vs[(4 * g + (r >> 2)) * PITCH + 4 * (r & 3)];
 #pragma unroll
       for (int pair = 0; pair < NSUB / 2; ++pair) {
-        uint32_t vw[8][DC / 2];  // rows 4g + u of sub-tile 2 pair (u < 4) and of sub-tile 2 pair + 1
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int row = (2 * pair + u / 4) * 16 + 4 * g + (u % 4);
-          const uint16_t* vrow = &vs[row * PITCH + DC * r];
-          if constexpr (DC == 16) {
-            const u32x4 v = *reinterpret_cast<const u32x4*>(vrow);
-            const u32x4 v2 = *reinterpret_cast<const u32x4*>(vrow + 8);
-            vw[u][0] = v.x; vw[u][1] = v.y; vw[u][2] = v.z; vw[u][3] = v.w;
-            vw[u][4] = v2.x; vw[u][5] = v2.y; vw[u][6] = v2.z; vw[u][7] = v2.w;
-          } else if constexpr (DC == 8) {
-            const u32x4 v = *reinterpret_cast<const u32x4*>(vrow);
-            vw[u][0] = v.x; vw[u][1] = v.y; vw[u][2] = v.z; vw[u][3] = v.w;
-          } else {
-            const u32x2 v = *reinterpret_cast<const u32x2*>(vrow);
-            vw[u][0] = v.x; vw[u][1] = v.y;
-          }
-        }
-#pragma unroll
-        for (int c = 0; c < DC / 2; ++c) {
-          u32x4 lo, hi;
-          lo.x = __builtin_amdgcn_perm(vw[1][c], vw[0][c], 0x05040100u);
-          lo.y = __builtin_amdgcn_perm(vw[3][c], vw[2][c], 0x05040100u);
-          lo.z = __builtin_amdgcn_perm(vw[5][c], vw[4][c], 0x05040100u);
-          lo.w = __builtin_amdgcn_perm(vw[7][c], vw[6][c], 0x05040100u);
-          hi.x = __builtin_amdgcn_perm(vw[1][c], vw[0][c], 0x07060302u);
-          hi.y = __builtin_amdgcn_perm(vw[3][c], vw[2][c], 0x07060302u);
-          hi.z = __builtin_amdgcn_perm(vw[5][c], vw[4][c], 0x07060302u);
-          hi.w = __builtin_amdgcn_perm(vw[7][c], vw[6][c], 0x07060302u);
+        for (int a = 0; a < DC; ++a) {
+          const u32x2 t0 = lds_read_tr16(vlane + (32 * pair) * PITCH + 16 * a);
+          const u32x2 t1 = lds_read_tr16(vlane + (32 * pair + 16) * PITCH + 16 * a);
+          const u32x4 vb = {t0.x, t0.y, t1.x, t1.y};
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) {
             if (!act[mt]) continue;
             const u32x4 pp = {pa[mt][2 * pair][0], pa[mt][2 * pair][1], pa[mt][2 * pair + 1][0],
                               pa[mt][2 * pair + 1][1]};
-            oacc[mt][2 * c] = mfma_16x16x32<T>(pp, lo, oacc[mt][2 * c]);
-            oacc[mt][2 * c + 1] = mfma_16x16x32<T>(pp, hi, oacc[mt][2 * c + 1]);
+            oacc[mt][a] = mfma_16x16x32<T>(pp, vb, oacc[mt][a]);
           }
         }
       }
@@ -259,7 +255,7 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
     }
   }
 
-  // ---- normalise and store: lane holds rows 4g + i, dimensions [DC r, DC r + DC) ------------------
+  // ---- normalise and store: lane holds rows 4g + i, dimensions 16 a + r ---------------------------
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     float l = l_run[mt];
@@ -271,19 +267,9 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
       const float inv = li > 0.f ? 1.f / li : 0.f;
       const int row = q0 + wave * WR + mt * 16 + 4 * g + i;
       if (row < p.n_q) {
-        uint16_t* dst = p.o + ((int64_t)row * p.num_qo_heads + qh) * D + DC * r;
-        uint32_t ow[DC / 2];
+        uint16_t* dst = p.o + ((int64_t)row * p.num_qo_heads + qh) * D + r;
 #pragma unroll
-        for (int c = 0; c < DC / 2; ++c)
-          ow[c] = pack2<T>(oacc[mt][2 * c][i] * inv, oacc[mt][2 * c + 1][i] * inv);
-        if constexpr (DC == 4) {
-          *reinterpret_cast<u32x2*>(dst) = u32x2{ow[0], ow[1]};
-        } else {
-#pragma unroll
-          for (int c = 0; c < DC / 8; ++c)
-            *reinterpret_cast<u32x4*>(dst + 8 * c) =
-                u32x4{ow[4 * c], ow[4 * c + 1], ow[4 * c + 2], ow[4 * c + 3]};
-        }
+        for (int a = 0; a < DC; ++a) dst[16 * a] = from_float<T>(oacc[mt][a][i] * inv);
       }
     }
   }
