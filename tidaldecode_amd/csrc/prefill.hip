@@ -63,8 +63,10 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
   constexpr int CPT = RPT * CCT;    // chunks a thread stages per tile and matrix
   static_assert(D == 64 || D == 128 || D == 256, "head dimensions of the prefill kernel");
   static_assert(BN % 32 == 0 && CPT * kPfThreads == BN * CPR, "key tile");
-  __shared__ __attribute__((aligned(16))) uint16_t ks[kPfBN * PITCH];
-  __shared__ __attribute__((aligned(16))) uint16_t vs[kPfBN * PITCH];
+  // two buffers per matrix: tile t + 1 is written while tile t is still being read
+  constexpr int TILE = kPfBN * PITCH;
+  __shared__ __attribute__((aligned(16))) uint16_t ks[2 * TILE];
+  __shared__ __attribute__((aligned(16))) uint16_t vs[2 * TILE];
 
   // the wave index is made scalar: the per-tile activity tests below must be real branches, because
   // matrix instructions do not honour the EXEC mask of a masked-off region
@@ -132,12 +134,12 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
       }
     }
   };
-  auto stash = [&]() {
+  auto stash = [&](int buf) {
 #pragma unroll
     for (int jr = 0; jr < RPT; ++jr)
 #pragma unroll
       for (int jc = 0; jc < CCT; ++jc) {
-        const int at = (srow + 32 * jr) * PITCH + (sl8 + 8 * jc) * 8;
+        const int at = buf * TILE + (srow + 32 * jr) * PITCH + (sl8 + 8 * jc) * 8;
         *reinterpret_cast<u32x4*>(&ks[at]) = kreg[jr * CCT + jc];
         *reinterpret_cast<u32x4*>(&vs[at]) = vreg[jr * CCT + jc];
       }
@@ -145,27 +147,29 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
 
   const int wave_first_pos = q_off + q0 + wave * WR;  // position of the wave's first query row
   fetch(0);
-  stash();
-  __syncthreads();
-  for (int kt = 0; kt < kv_end; kt += kPfBN) {
+  stash(0);
+  int buf = 0;
+  for (int kt = 0; kt < kv_end; kt += kPfBN, buf ^= 1) {
+    // one barrier per tile: tile kt is visible in buffer buf, and every wave has finished reading
+    // the other buffer (tile kt - BN), which the end of this iteration overwrites
+    __syncthreads();
     const bool more = kt + kPfBN < kv_end;
     if (more) fetch(kt + kPfBN);
-    // a query tile whose last row lies before the key tile sees none of it (causal)
-    bool act[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) act[mt] = !p.causal || kt <= wave_first_pos + mt * 16 + 15;
-    if (act[MT - 1]) {
+    // A wave whose last query row lies before the key tile sees none of it (causal).  Inside an
+    // active wave every query tile is computed: a tile that lies wholly before the key tile is
+    // masked to zero weight below, which happens once per wave, and the loop body stays free of
+    // branches around the matrix instructions.
+    if (!p.causal || kt <= wave_first_pos + WR - 1) {
       // ---- S^T: each K operand is read once and used by every active query tile -----------------
       f32x4 st[MT][NSUB];
 #pragma unroll
       for (int sub = 0; sub < NSUB; ++sub) {
         u32x4 ka[NS];
-        const uint16_t* krow = &ks[(sub * 16 + r) * PITCH + 8 * g];
+        const uint16_t* krow = &ks[buf * TILE + (sub * 16 + r) * PITCH + 8 * g];
 #pragma unroll
         for (int s = 0; s < NS; ++s) ka[s] = *reinterpret_cast<const u32x4*>(krow + 32 * s);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-          if (!act[mt]) continue;
           f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int s = 0; s < NS; ++s) acc = mfma_16x16x32<T>(ka[s], qb[mt][s], acc);
@@ -176,7 +180,6 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
       uint32_t pa[MT][NSUB][2];
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        if (!act[mt]) continue;
         const int qpos = wave_first_pos + mt * 16 + r;  // position of this lane's query row
         const bool need_mask =
             (p.causal && kt + kPfBN - 1 > wave_first_pos + mt * 16) || kt + kPfBN > p.kv_len;
@@ -230,7 +233,7 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
       // tokens 4g..4g+3 of both sub-tiles.  ds_read_b64_tr_b16 transposes a 4 token x 16 dimension
       // block inside every 16 lanes: lane r points at the 8-byte piece r % 4 of token row r / 4
       // and receives dimension r of the four rows.
-      const uint16_t* vlane = &vs[(4 * g + (r >> 2)) * PITCH + 4 * (r & 3)];
+      const uint16_t* vlane = &vs[buf * TILE + (4 * g + (r >> 2)) * PITCH + 4 * (r & 3)];
 #pragma unroll
       for (int pair = 0; pair < NSUB / 2; ++pair) {
 #pragma unroll
@@ -240,7 +243,6 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
           const u32x4 vb = {t0.x, t0.y, t1.x, t1.y};
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) {
-            if (!act[mt]) continue;
             const u32x4 pp = {pa[mt][2 * pair][0], pa[mt][2 * pair][1], pa[mt][2 * pair + 1][0],
                               pa[mt][2 * pair + 1][1]};
             oacc[mt][a] = mfma_16x16x32<T>(pp, vb, oacc[mt][a]);
@@ -248,11 +250,7 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
         }
       }
     }
-    __syncthreads();  // every wave is done with the tile in LDS
-    if (more) {
-      stash();
-      __syncthreads();
-    }
+    if (more) stash(buf ^ 1);
   }
 
   // ---- normalise and store: lane holds rows 4g + i, dimensions 16 a + r ---------------------------
