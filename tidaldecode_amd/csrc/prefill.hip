@@ -110,21 +110,34 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
   // LDS write out); a thread looks up the page of each of its RPT rows once
   u32x4 kreg[CPT], vreg[CPT];
   const int srow = tid >> 3, sl8 = tid & 7;
-  auto fetch = [&](int kt) {
+  // page ids are looked up one tile ahead of the rows they address, so that a tile's K/V loads
+  // never wait for a page-table load issued in the same iteration
+  uint32_t pg[RPT];
+  auto split_tok = [&](int kt, int jr, int& pg_i, int& entry) {
+    int tok = kt + srow + 32 * jr;
+    tok = tok < p.kv_len ? tok : p.kv_len - 1;
+    if (p.page_shift >= 0) {
+      pg_i = tok >> p.page_shift;
+      entry = tok & (p.page_size - 1);
+    } else {
+      pg_i = tok / p.page_size;
+      entry = tok - pg_i * p.page_size;
+    }
+  };
+  auto lookup = [&](int kt) {
 #pragma unroll
     for (int jr = 0; jr < RPT; ++jr) {
-      int tok = kt + srow + 32 * jr;
-      tok = tok < p.kv_len ? tok : p.kv_len - 1;
       int pg_i, entry;
-      if (p.page_shift >= 0) {
-        pg_i = tok >> p.page_shift;
-        entry = tok & (p.page_size - 1);
-      } else {
-        pg_i = tok / p.page_size;
-        entry = tok - pg_i * p.page_size;
-      }
-      uint32_t page = (uint32_t)p.page_table[pg_i];
-      page = page > p.max_page ? p.max_page : page;
+      split_tok(kt, jr, pg_i, entry);
+      pg[jr] = (uint32_t)p.page_table[pg_i];
+    }
+  };
+  auto fetch = [&](int kt) {  // needs lookup(kt) before it
+#pragma unroll
+    for (int jr = 0; jr < RPT; ++jr) {
+      int pg_i, entry;
+      split_tok(kt, jr, pg_i, entry);
+      const uint32_t page = pg[jr] > p.max_page ? p.max_page : pg[jr];
       const uint16_t* src = p.kv + ((int64_t)page * p.page_stride + (int64_t)entry * p.entry_stride +
                                     (int64_t)kvh * p.head_stride + sl8 * 8);
 #pragma unroll
@@ -146,7 +159,9 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
   };
 
   const int wave_first_pos = q_off + q0 + wave * WR;  // position of the wave's first query row
+  lookup(0);
   fetch(0);
+  lookup(kPfBN);
   stash(0);
   int buf = 0;
   for (int kt = 0; kt < kv_end; kt += kPfBN, buf ^= 1) {
@@ -154,7 +169,10 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
     // the other buffer (tile kt - BN), which the end of this iteration overwrites
     __syncthreads();
     const bool more = kt + kPfBN < kv_end;
-    if (more) fetch(kt + kPfBN);
+    if (more) {
+      fetch(kt + kPfBN);
+      lookup(kt + 2 * kPfBN);
+    }
     // A wave whose last query row lies before the key tile sees none of it (causal).  Inside an
     // active wave every query tile is computed: a tile that lies wholly before the key tile is
     // masked to zero weight below, which happens once per wave, and the loop body stays free of
@@ -202,7 +220,11 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
         mt_max = fmaxf(mt_max, __shfl_xor(mt_max, 32, 64));
         // m_run is kept in the scaled base-2 domain.  A masked entry (kNegBig) gives exp2(-huge) = 0
         // by itself: every query row sees token 0 in its first tile, so m_new is a real maximum.
-        const float m_new = fmaxf(m_run[mt], mt_max * p.scale_log2);
+        // The running maximum only moves when the tile's maximum exceeds it by more than 2^8:
+        // softmax does not depend on the reference point, weights up to 256 are exact to the same
+        // relative precision, and the accumulator rescale below becomes rare.
+        const float m_tile = mt_max * p.scale_log2;
+        const float m_new = m_tile > m_run[mt] + 8.f ? m_tile : m_run[mt];
         const float alpha = fast_exp2(m_run[mt] - m_new);
         m_run[mt] = m_new;
         float psum = 0.f;
