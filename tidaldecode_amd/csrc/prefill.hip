@@ -72,8 +72,25 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
   // matrix instructions do not honour the EXEC mask of a masked-off region
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, g = lane >> 4;
-  const int qtile = gridDim.x - 1 - blockIdx.x;  // longest rows first
-  const int qh = blockIdx.y;
+  // Workgroups go to the eight XCDs round-robin by linear id, and each XCD has its own L2.  When
+  // the KV heads divide evenly, all query tiles of the heads that share a KV head are given to one
+  // XCD, so that its L2 streams one head's K/V instead of every head's.  (Placement only decides
+  // what the L2 holds; results do not depend on it.)  Longest rows first in either order.
+  int qtile, qh;
+  {
+    const int n_tiles = gridDim.x, n_heads = gridDim.y;
+    const int lin = blockIdx.x + n_tiles * blockIdx.y;
+    const int n_kv = n_heads / p.q_per_kv;
+    if (n_kv % 8 == 0) {
+      const int xcd = lin & 7, slot = lin >> 3;
+      const int idx = slot / n_tiles;  // which of this XCD's heads
+      qtile = n_tiles - 1 - slot % n_tiles;
+      qh = ((idx / p.q_per_kv) * 8 + xcd) * p.q_per_kv + idx % p.q_per_kv;
+    } else {
+      qtile = n_tiles - 1 - blockIdx.x;
+      qh = blockIdx.y;
+    }
+  }
   const int kvh = qh / p.q_per_kv;
   const int q0 = qtile * kPfBM;
   const int q_off = p.kv_len - p.n_q;  // position of query row 0
