@@ -125,7 +125,9 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
   // ---- staging: thread -> CPT chunks of K and of V per tile --------------------------------------
   // eight adjacent lanes move 128 contiguous bytes of one row (one cache line in, one conflict-free
   // LDS write out); a thread looks up the page of each of its RPT rows once
-  u32x4 kreg[CPT], vreg[CPT];
+  // Two register sets: the loads of tile t + 2 are issued while tile t + 1 still waits in the
+  // other set for its turn to be written to LDS, so a tile has two iterations to arrive.
+  u32x4 kreg_a[CPT], vreg_a[CPT], kreg_b[CPT], vreg_b[CPT];
   const int srow = tid >> 3, sl8 = tid & 7;
   // page ids are looked up one tile ahead of the rows they address, so that a tile's K/V loads
   // never wait for a page-table load issued in the same iteration
@@ -149,7 +151,7 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
       pg[jr] = (uint32_t)p.page_table[pg_i];
     }
   };
-  auto fetch = [&](int kt) {  // needs lookup(kt) before it
+  auto fetch = [&](int kt, u32x4 (&kreg)[CPT], u32x4 (&vreg)[CPT]) {  // needs lookup(kt) before it
 #pragma unroll
     for (int jr = 0; jr < RPT; ++jr) {
       int pg_i, entry;
@@ -164,7 +166,7 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
       }
     }
   };
-  auto stash = [&](int buf) {
+  auto stash = [&](int buf, const u32x4 (&kreg)[CPT], const u32x4 (&vreg)[CPT]) {
 #pragma unroll
     for (int jr = 0; jr < RPT; ++jr)
 #pragma unroll
@@ -176,20 +178,7 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
   };
 
   const int wave_first_pos = q_off + q0 + wave * WR;  // position of the wave's first query row
-  lookup(0);
-  fetch(0);
-  lookup(kPfBN);
-  stash(0);
-  int buf = 0;
-  for (int kt = 0; kt < kv_end; kt += kPfBN, buf ^= 1) {
-    // one barrier per tile: tile kt is visible in buffer buf, and every wave has finished reading
-    // the other buffer (tile kt - BN), which the end of this iteration overwrites
-    __syncthreads();
-    const bool more = kt + kPfBN < kv_end;
-    if (more) {
-      fetch(kt + kPfBN);
-      lookup(kt + 2 * kPfBN);
-    }
+  auto compute = [&](int kt, int buf) {
     // A wave whose last query row lies before the key tile sees none of it (causal).  Inside an
     // active wave every query tile is computed: a tile that lies wholly before the key tile is
     // masked to zero weight below, which happens once per wave, and the loop body stays free of
@@ -289,7 +278,35 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
         }
       }
     }
-    if (more) stash(buf ^ 1);
+  };
+
+  // tile 0 into buffer 0, tile 1 into register set a
+  lookup(0);
+  fetch(0, kreg_a, vreg_a);
+  lookup(kPfBN);
+  stash(0, kreg_a, vreg_a);
+  if (kPfBN < kv_end) {
+    fetch(kPfBN, kreg_a, vreg_a);
+    lookup(2 * kPfBN);
+  }
+  // One barrier per tile: it makes tile kt visible in its buffer, and it tells that every wave has
+  // finished reading the other buffer, which the end of the step overwrites with tile kt + BN.
+  for (int kt = 0; kt < kv_end; kt += 2 * kPfBN) {
+    __syncthreads();
+    if (kt + 2 * kPfBN < kv_end) {
+      fetch(kt + 2 * kPfBN, kreg_b, vreg_b);
+      lookup(kt + 3 * kPfBN);
+    }
+    compute(kt, 0);
+    if (kt + kPfBN >= kv_end) break;
+    stash(1, kreg_a, vreg_a);
+    __syncthreads();
+    if (kt + 3 * kPfBN < kv_end) {
+      fetch(kt + 3 * kPfBN, kreg_a, vreg_a);
+      lookup(kt + 4 * kPfBN);
+    }
+    compute(kt + kPfBN, 1);
+    if (kt + 2 * kPfBN < kv_end) stash(0, kreg_b, vreg_b);
   }
 
   // ---- normalise and store: lane holds rows 4g + i, dimensions 16 a + r ---------------------------
