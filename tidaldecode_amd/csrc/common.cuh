@@ -116,6 +116,47 @@ __device__ __forceinline__ uint16_t from_float<BF16>(float f) {
   return __builtin_bit_cast(uint16_t, (__bf16)f);
 }
 
+// Maximum / sum over the four 16-lane rows of a wavefront (lanes l, l ^ 16, l ^ 32, l ^ 48), result
+// in every lane.  gfx950's v_permlane16_swap / v_permlane32_swap exchange rows between two
+// registers in the vector pipeline: given the same value twice, the first result holds the even
+// row (lower half) of each pair in both of its rows (halves), the second result the odd row
+// (upper half).
+// The instruction swaps in place between two different registers; the copy below is made opaque
+// so that the two operands are never allocated to one register (a swap of a register with itself
+// exchanges nothing).
+typedef unsigned int u32pair __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t opaque_copy(uint32_t u) {
+  uint32_t c = u;
+  asm volatile("" : "+v"(c));
+  return c;
+}
+__device__ __forceinline__ void swap_rows16(float v, float& even, float& odd) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, v);
+  const u32pair a = __builtin_amdgcn_permlane16_swap(u, opaque_copy(u), false, false);
+  const uint32_t lo = a.x, hi = a.y;  // elements are copied out before the bit cast
+  even = __builtin_bit_cast(float, lo);
+  odd = __builtin_bit_cast(float, hi);
+}
+__device__ __forceinline__ void swap_halves32(float v, float& lower, float& upper) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, v);
+  const u32pair a = __builtin_amdgcn_permlane32_swap(u, opaque_copy(u), false, false);
+  const uint32_t lo = a.x, hi = a.y;
+  lower = __builtin_bit_cast(float, lo);
+  upper = __builtin_bit_cast(float, hi);
+}
+__device__ __forceinline__ float rows_max(float v) {
+  float a, b;
+  swap_rows16(v, a, b);
+  swap_halves32(fmaxf(a, b), a, b);
+  return fmaxf(a, b);
+}
+__device__ __forceinline__ float rows_sum(float v) {
+  float a, b;
+  swap_rows16(v, a, b);
+  swap_halves32(a + b, a, b);
+  return a + b;
+}
+
 // ---------------------------------------------------------------------------------------------
 // Cross-lane sums inside a group of W adjacent lanes (W = 8, 16 or 32) of a 64-wide wavefront,
 // result in every lane of the group.  DPP modifiers fold into the v_add_f32.

@@ -205,8 +205,11 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         const int qpos = wave_first_pos + mt * 16 + r;  // position of this lane's query row
+        // the test of the wave's first query tile covers the second: masking a tile that does
+        // not need it changes nothing, and one rare branch keeps the position arithmetic out of
+        // the common path
         const bool need_mask =
-            (p.causal && kt + kPfBN - 1 > wave_first_pos + mt * 16) || kt + kPfBN > p.kv_len;
+            (p.causal && kt + kPfBN - 1 > wave_first_pos) || kt + kPfBN > p.kv_len;
         if (need_mask) {
 #pragma unroll
           for (int sub = 0; sub < NSUB; ++sub)
@@ -222,8 +225,7 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
         for (int sub = 0; sub < NSUB; ++sub)
 #pragma unroll
           for (int i = 0; i < 4; ++i) mt_max = fmaxf(mt_max, st[mt][sub][i]);
-        mt_max = fmaxf(mt_max, __shfl_xor(mt_max, 16, 64));
-        mt_max = fmaxf(mt_max, __shfl_xor(mt_max, 32, 64));
+        mt_max = rows_max(mt_max);
         // m_run is kept in the scaled base-2 domain.  A masked entry (kNegBig) gives exp2(-huge) = 0
         // by itself: every query row sees token 0 in its first tile, so m_new is a real maximum.
         // The running maximum only moves when the tile's maximum exceeds it by more than 2^8:
@@ -312,9 +314,7 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
   // ---- normalise and store: lane holds rows 4g + i, dimensions 16 a + r ---------------------------
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    float l = l_run[mt];
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
+    const float l = rows_sum(l_run[mt]);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const float li = __shfl(l, 4 * g + i, 64);
