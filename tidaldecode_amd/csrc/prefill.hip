@@ -185,6 +185,10 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
     // branches around the matrix instructions.
     if (!p.causal || kt <= wave_first_pos + WR - 1) {
       // ---- S^T: each K operand is read once and used by every active query tile -----------------
+      // (the two matrix phases run at raised wave priority: while one wave of a SIMD is in its
+      // softmax arithmetic, the other's matrix instructions are issued first and keep the matrix
+      // pipeline busy)
+      __builtin_amdgcn_s_setprio(2);
       f32x4 st[MT][NSUB];
 #pragma unroll
       for (int sub = 0; sub < NSUB; ++sub) {
@@ -200,6 +204,7 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
           st[mt][sub] = acc;  // raw q.k; the softmax scale is folded into the exponent below
         }
       }
+      __builtin_amdgcn_s_setprio(0);
       // ---- online softmax of query row r (lanes r, r+16, r+32, r+48 share the row) ---------------
       uint32_t pa[MT][NSUB][2];
 #pragma unroll
@@ -258,6 +263,7 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
           }
         }
       }
+      __builtin_amdgcn_s_setprio(2);
       // ---- O += P V, 32 tokens (two sub-tiles) per matrix instruction ------------------------------
       // B operand of head dimensions [16 a, 16 a + 16): lane (r, g) needs dimension 16 a + r of the
       // tokens 4g..4g+3 of both sub-tiles.  ds_read_b64_tr_b16 transposes a 4 token x 16 dimension
@@ -279,6 +285,7 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
           }
         }
       }
+      __builtin_amdgcn_s_setprio(0);
     }
   };
 
