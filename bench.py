@@ -65,6 +65,9 @@ def parse():
                          "layers 0 and 13)")
     ap.add_argument("--e2e-ctx", type=str, default="32768,102400",
                     help="context lengths of the end-to-end leg")
+    ap.add_argument("--no-real-prompt", action="store_true",
+                    help="end-to-end leg: skip the real prompt (prefill of random tokens through "
+                         "the decoder, then greedy decoding)")
     ap.add_argument("--extra-only", action="store_true",
                     help="profile helper: run only the prefill, batch-8 and end-to-end legs and "
                          "print their JSON object")
@@ -312,6 +315,25 @@ def e2e_leg(args):
             tok = model.decode_step(tok).argmax().view(1)
         torch.cuda.synchronize()
         row["tidal_eager_generate_ms_per_token"] = round((time.perf_counter() - t0) / n_gen * 1e3, 4)
+        if not args.no_real_prompt:
+            # the configuration as written: a random-token prompt runs through the decoder (paged
+            # prefill attention, K/V appended to the cache), then greedy decoding, every step real
+            model.tidal_clear()
+            g = torch.Generator().manual_seed(0)
+            ids = torch.randint(0, cfg.vocab_size, (ctx,), generator=g)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            tok = model.prefill(ids).argmax().view(1)
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            n_gen = 256 if ctx <= 32768 else 128
+            for _ in range(n_gen):
+                tok = model.decode_step(tok).argmax().view(1)
+            torch.cuda.synchronize()
+            row["real_prompt"] = {"prompt_tokens": ctx, "prefill_s": round(t1 - t0, 3),
+                                  "prefill_tokens_per_s": round(ctx / (t1 - t0), 1),
+                                  "greedy_steps": n_gen,
+                                  "greedy_ms_per_token": round((time.perf_counter() - t1) / n_gen * 1e3, 4)}
         out[str(ctx)] = row
     del model
     torch.cuda.empty_cache()
