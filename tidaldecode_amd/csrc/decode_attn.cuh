@@ -443,7 +443,7 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
       }
     }
     if constexpr (QPG > 1) {
-      float sv[U];
+      float sv[U], xe[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         float a[QPG];
@@ -455,23 +455,37 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
           a[j] = dot2<T>(qp[j][3], kb[u].w, a[j]);
         }
         const float x = reduce_scatter16<QPG>(a, li) * p.scale_log2;  // head li % QPG
-        const int i = base + u * TPI + g;
-        const bool valid = i < c1;
-        if constexpr (EMIT) {
-          if (valid && li < QPG) {
-            const int64_t at = ((int64_t)b * p.num_qo_heads + qh0 + li) * p.score_stride + i;
-            const float nat = x * kLn2;
+        xe[u] = x;
+        sv[u] = (base + u * TPI + g < c1) ? x : kNegBig;
+      }
+      if constexpr (EMIT) {
+        // One store per four heads and tile: lane L collects the logit of (head L / 16, token
+        // base + L % 16), which lane group (L % 16) % TPI holds in its lane of that head for row
+        // (L % 16) / TPI, so that a head's 16 logits of the tile leave as 64 contiguous bytes.
+        static_assert(TPI == 4 && U == 4, "logit transposition of the grouped-query tile");
+#pragma unroll
+        for (int hb = 0; hb < (QPG + 3) / 4; ++hb) {
+          const int src = (lane & 3) * 16 + hb * 4 + (lane >> 4);
+          float e = 0.f;
+#pragma unroll
+          for (int u = 0; u < U; ++u) {
+            const float v = __shfl(xe[u], src, 64);
+            e = (((lane >> 2) & 3) == u) ? v : e;
+          }
+          const int head = hb * 4 + (lane >> 4);
+          const int i = base + (lane & 15);
+          if (head < QPG && i < c1) {
+            const int64_t at = ((int64_t)b * p.num_qo_heads + qh0 + head) * p.score_stride + i;
+            const float nat = e * kLn2;
             if (p.scores_f32)
               reinterpret_cast<float*>(p.scores)[at] = nat;
             else
               reinterpret_cast<uint16_t*>(p.scores)[at] = from_float<T>(nat);
           }
         }
-        sv[u] = valid ? x : kNegBig;
       }
       float mt = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
-      mt = fmaxf(mt, __shfl_xor(mt, 16, 64));  // the tile's maximum over all four lane groups
-      mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+      mt = rows_max(mt);  // the tile's maximum over all four lane groups
       const float m_new = fmaxf(mh, mt);
       const float alpha = fast_exp2(mh - m_new);
       mh = m_new;
