@@ -390,25 +390,42 @@ __global__ __launch_bounds__(kTopkThreads) void topk_reg_kernel(const TopkParams
 // push a 32K-element row through the single-workgroup kernels above (the row costs ~40K wave
 // instructions); with a handful of rows that leaves the other 200+ compute units idle.
 //
-//   launch 1 (topk_coop_select_kernel, grid G x rows): every workgroup histograms the top 11 key
-//     bits of its slice in LDS and adds the non-empty bins to a per-row global histogram; the last
-//     workgroup of a row to arrive (ticket) locates the threshold bin, re-reads the row once to
-//     gather that bin's candidates into LDS (counting, per slice, what lies above the bin),
-//     finishes the radix select on the candidates, and publishes the threshold key T, the number
-//     r of ties to take and per-slice output / tie offsets.
-//   launch 2 (topk_coop_emit_kernel, grid G x rows): every workgroup emits its slice in index
+//   launch 1 (topk_coop_hist_kernel, grid G x rows): every workgroup histograms the top 11 key
+//     bits of its slice in LDS and adds the non-empty bins to a per-row global histogram.
+//   launch 2 (topk_coop_select_kernel, grid G x rows): every workgroup locates the threshold bin
+//     in the row histogram (the same scan, redundantly: it is cheap), counts what its slice holds
+//     above the bin and appends the slice's members of the bin (key, index) to the row's
+//     candidate list; the last workgroup of a row to arrive (ticket) loads the list (a few
+//     thousand entries instead of the row), finishes the radix select on it, and publishes the
+//     threshold key T, the number r of ties to take and per-slice output / tie offsets.
+//     A bin with more members than the list holds (most keys share 11 leading bits) is left to
+//     the last workgroup, which narrows it with streaming passes over the row.
+//   launch 3 (topk_coop_emit_kernel, grid G x rows): every workgroup emits its slice in index
 //     order at its published offset.
 //
 // Scratch per row (uint32): [0,2048) histogram, 2048 ticket, 2049 T, 2050 r, then per slice
-// (out_before, eq_before).  The histogram and ticket must be zero before the first call; launch 1
-// leaves them zero again.  Values are keyed as fp32 whatever the input type.
+// (out_before, eq_before), the candidate count, per slice the count above the bin, and the
+// candidate keys and indices.  Histogram, ticket and candidate count must be zero before the
+// first call; launch 2 leaves them zero again.  Values are keyed as fp32 whatever the input type.
 // ---------------------------------------------------------------------------------------------
 constexpr int kCoopIPT = 8;                       // keys per thread and slice
 constexpr int kCoopSlice = kCoopIPT * kTopkThreads;  // 8192 elements per workgroup
 constexpr int kCoopMaxSlices = 32;
 constexpr int kCoopBatch = 4;                     // slices per trip of the row pass
 constexpr int kCoopCand = 6144;                   // candidates kept in LDS
-constexpr int kCoopRowWords = 2048 + 3 + 2 * kCoopMaxSlices;
+constexpr int kCoopOffsets = 2051;                            // (out_before, eq_before) per slice
+constexpr int kCoopCandCount = kCoopOffsets + 2 * kCoopMaxSlices;
+constexpr int kCoopSliceGt = kCoopCandCount + 1;              // per slice: keys above the bin
+constexpr int kCoopCandKey = kCoopSliceGt + kCoopMaxSlices;
+constexpr int kCoopCandIdx = kCoopCandKey + kCoopCand;
+constexpr int kCoopRowWords = kCoopCandIdx + kCoopCand;
+
+__device__ __forceinline__ uint32_t load_agent(const uint32_t* at) {
+  return __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_agent(uint32_t* at, uint32_t v) {
+  __hip_atomic_store(at, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 template <typename T>
 __device__ __forceinline__ uint32_t coop_key(const void* base, int64_t i);
@@ -488,6 +505,33 @@ __device__ __forceinline__ void coop_level(const uint32_t* ckey, int n_cand, uin
 }
 
 template <typename T>
+__global__ __launch_bounds__(kTopkThreads) void topk_coop_hist_kernel(const TopkParams p,
+                                                                      uint32_t* scratch,
+                                                                      int n_slices, int rows) {
+  int slice, row;
+  if (!coop_decode(n_slices, rows, slice, row)) return;
+  const int tid = threadIdx.x;
+  const int len = p.len;
+  const void* vals = reinterpret_cast<const char*>(p.values) +
+                     (int64_t)row * p.values_stride * sizeof(typename ElemOf<T>::type);
+  uint32_t* rs = scratch + (int64_t)row * kCoopRowWords;
+  __shared__ uint32_t hist[2048];
+  for (int i = tid; i < 2048; i += kTopkThreads) hist[i] = 0;
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < kCoopIPT; ++j) {
+    const int i = slice * kCoopSlice + j * kTopkThreads + tid;
+    const uint32_t kv = coop_key<T>(vals, i < len ? i : len - 1);  // loads stay unconditional
+    if (i < len) atomicAdd(&hist[kv >> 21], 1u);
+  }
+  __syncthreads();
+  for (int i = tid; i < 2048; i += kTopkThreads) {
+    const uint32_t c = hist[i];
+    if (c) __hip_atomic_fetch_add(rs + i, c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+template <typename T>
 __global__ __launch_bounds__(kTopkThreads) void topk_coop_select_kernel(const TopkParams p,
                                                                         uint32_t* scratch,
                                                                         int n_slices, int rows) {
@@ -505,39 +549,20 @@ __global__ __launch_bounds__(kTopkThreads) void topk_coop_select_kernel(const To
   __shared__ uint32_t ckey[kCoopCand];
   __shared__ int32_t cidx[kCoopCand];
   __shared__ uint32_t slice_gt[kCoopMaxSlices], slice_eq[kCoopMaxSlices];
-  __shared__ uint32_t n_cand_sh;
+  __shared__ uint32_t n_cand_sh, n_above_sh, cand_base_sh;
 
-  // ---- phase 1: slice histogram of the top 11 bits -> global row histogram -------------------
-  for (int i = tid; i < 2048; i += kTopkThreads) hist[i] = 0;
-  __syncthreads();
+  // ---- every workgroup: its slice's keys (in flight while the histogram is scanned) ------------
+  uint32_t own[kCoopIPT];
 #pragma unroll
   for (int j = 0; j < kCoopIPT; ++j) {
     const int i = slice * kCoopSlice + j * kTopkThreads + tid;
-    const uint32_t kv = coop_key<T>(vals, i < len ? i : len - 1);  // loads stay unconditional
-    if (i < len) atomicAdd(&hist[kv >> 21], 1u);
+    const uint32_t kv = coop_key<T>(vals, i < len ? i : len - 1);
+    own[j] = i < len ? kv : 0u;  // 0 lies below every real key
   }
-  __syncthreads();
-  for (int i = tid; i < 2048; i += kTopkThreads) {
-    const uint32_t c = hist[i];
-    if (c) __hip_atomic_fetch_add(rs + i, c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this workgroup's additions are performed
-  __syncthreads();
-  if (tid == 0)
-    sh[2] = __hip_atomic_fetch_add(rs + 2048, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __syncthreads();
-  if (sh[2] != (uint32_t)(n_slices - 1)) return;
-
-  // ---- phase 2 (last workgroup of the row): threshold bin of level 1 ------------------------
-  for (int i = tid; i < 2048; i += kTopkThreads) {
-    hist[i] = __hip_atomic_load(rs + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(rs + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
+  // ---- threshold bin of level 1 from the row histogram of the launch before -------------------
+  for (int i = tid; i < 2048; i += kTopkThreads) hist[i] = load_agent(rs + i);
   if (tid < kCoopMaxSlices) slice_gt[tid] = slice_eq[tid] = 0;
-  if (tid == 0) {
-    __hip_atomic_store(rs + 2048, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    n_cand_sh = 0;
-  }
+  if (tid == 0) n_cand_sh = n_above_sh = 0;
   __syncthreads();
   uint32_t prefix = 0, mask = 0, krem = (uint32_t)p.k;
   {
@@ -563,11 +588,77 @@ __global__ __launch_bounds__(kTopkThreads) void topk_coop_select_kernel(const To
     krem = sh[1];
   }
   int n_in_bin = (int)sh[3];
+  const bool crowded = n_in_bin > kCoopCand;  // the same in every workgroup of the row
   __syncthreads();
 
-  // If the bin is too crowded for LDS, narrow it with streaming passes over the row
-  // (11 more bits, then 10): only pathological rows (most keys share 11 leading bits) get here.
+  // ---- every workgroup: count above the bin, append the slice's members of the bin -------------
+  if (!crowded) {
+    uint32_t n_above = 0, n_in = 0;
+    uint64_t cm[kCoopIPT];
+#pragma unroll
+    for (int j = 0; j < kCoopIPT; ++j) {
+      n_above += (uint32_t)__popcll(__ballot((own[j] & mask) > prefix));
+      cm[j] = __ballot(own[j] != 0u && (own[j] & mask) == prefix);
+      n_in += (uint32_t)__popcll(cm[j]);
+    }
+    uint32_t at = 0;
+    if (lane == 0) {
+      if (n_in) at = atomicAdd(&n_cand_sh, n_in);
+      if (n_above) atomicAdd(&n_above_sh, n_above);
+    }
+    at = __shfl(at, 0, 64);
+#pragma unroll
+    for (int j = 0; j < kCoopIPT; ++j) {
+      const uint32_t mine = at + lanes_below(cm[j]);
+      if ((cm[j] >> lane) & 1ull) {  // at most n_in_bin <= kCoopCand candidates in the whole row
+        ckey[mine] = own[j];
+        cidx[mine] = slice * kCoopSlice + j * kTopkThreads + tid;
+      }
+      at += (uint32_t)__popcll(cm[j]);
+    }
+    __syncthreads();
+    const uint32_t n_mine = n_cand_sh;
+    if (tid == 0) {
+      cand_base_sh = n_mine ? __hip_atomic_fetch_add(rs + kCoopCandCount, n_mine, __ATOMIC_RELAXED,
+                                                     __HIP_MEMORY_SCOPE_AGENT)
+                            : 0u;
+      store_agent(rs + kCoopSliceGt + slice, n_above_sh);
+    }
+    __syncthreads();
+    const uint32_t cbase = cand_base_sh;
+    for (uint32_t i = tid; i < n_mine; i += kTopkThreads) {
+      store_agent(rs + kCoopCandKey + cbase + i, ckey[i]);
+      store_agent(rs + kCoopCandIdx + cbase + i, (uint32_t)cidx[i]);
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this workgroup's stores are performed
+  __syncthreads();
+  if (tid == 0)
+    sh[2] = __hip_atomic_fetch_add(rs + 2048, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  if (sh[2] != (uint32_t)(n_slices - 1)) return;
+
+  // ---- last workgroup of the row: leave the scratch clean, then finish ---------------------------
+  for (int i = tid; i < 2048; i += kTopkThreads) store_agent(rs + i, 0u);
+  if (tid == 0) {
+    store_agent(rs + 2048, 0u);
+    store_agent(rs + kCoopCandCount, 0u);
+    n_cand_sh = 0;
+  }
   int shift = 21;
+  if (!crowded) {
+    // the row's candidates, from every slice
+    for (int i = tid; i < n_in_bin; i += kTopkThreads) {
+      ckey[i] = load_agent(rs + kCoopCandKey + i);
+      cidx[i] = (int32_t)load_agent(rs + kCoopCandIdx + i);
+    }
+    if (tid < n_slices) slice_gt[tid] = load_agent(rs + kCoopSliceGt + tid);
+    if (tid == 0) n_cand_sh = (uint32_t)n_in_bin;
+  }
+  __syncthreads();
+
+  // A bin too crowded for the list is narrowed with streaming passes over the row (11 more bits,
+  // then 10): only pathological rows (most keys share 11 leading bits) get here.
   while (n_in_bin > kCoopCand && shift > 0) {
     const int bits = shift > 10 ? 11 : 10;
     const int nb = 1 << bits;
@@ -608,9 +699,10 @@ __global__ __launch_bounds__(kTopkThreads) void topk_coop_select_kernel(const To
   // ---- phase 3: one pass over the row: count per slice what lies above the candidate range,
   //      gather the candidates (keys matching the prefix) unless the range is a single key -------
   const bool gather = shift > 0;  // shift == 0: all bits fixed, every candidate equals the threshold
-  // kCoopBatch slices per trip: a thread keeps 32 loads in flight, which is what it takes to
-  // cover the memory latency from one compute unit
-  for (int base0 = 0; base0 < len; base0 += kCoopBatch * kCoopSlice) {
+  // (crowded rows only; otherwise the slices have done this.)  kCoopBatch slices per trip: a
+  // thread keeps 32 loads in flight, which is what it takes to cover the memory latency from one
+  // compute unit
+  for (int base0 = 0; crowded && base0 < len; base0 += kCoopBatch * kCoopSlice) {
     uint32_t key[kCoopBatch][kCoopIPT];
 #pragma unroll
     for (int s = 0; s < kCoopBatch; ++s)
@@ -688,8 +780,8 @@ __global__ __launch_bounds__(kTopkThreads) void topk_coop_select_kernel(const To
     rs[2050] = r;
     uint32_t out_run = 0, eq_run = 0;
     for (int sl = 0; sl < n_slices; ++sl) {
-      rs[2051 + 2 * sl] = out_run;
-      rs[2052 + 2 * sl] = eq_run;
+      rs[kCoopOffsets + 2 * sl] = out_run;
+      rs[kCoopOffsets + 1 + 2 * sl] = eq_run;
       const uint32_t e = slice_eq[sl];
       const uint32_t room = r > eq_run ? r - eq_run : 0u;
       out_run += slice_gt[sl] + (e < room ? e : room);
@@ -710,7 +802,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_coop_emit_kernel(const Topk
   const elem_t* vals = reinterpret_cast<const elem_t*>(p.values) + (int64_t)row * p.values_stride;
   const uint32_t* rs = scratch + (int64_t)row * kCoopRowWords;
   const uint32_t thr = rs[2049], r = rs[2050];
-  const uint32_t slice_out = rs[2051 + 2 * slice], slice_eq = rs[2052 + 2 * slice];
+  const uint32_t slice_out = rs[kCoopOffsets + 2 * slice], slice_eq = rs[kCoopOffsets + 1 + 2 * slice];
 
   __shared__ uint32_t wave_tot[kTopkWaves];
   __shared__ uint32_t run_eq[kCoopIPT * kTopkWaves], run_out[kCoopIPT * kTopkWaves];
@@ -799,6 +891,8 @@ static void launch_topk(const TopkParams& p, int rows, hipStream_t st) {
 }
 
 // out[r, i] = sum_{h in row r} exp(logits[h, i] - lse[h])
+// A 256-thread workgroup covers 64 tokens: wave w sums heads w, w + 4, ... of the row (four
+// independent 256-byte row reads in flight per wave and trip), the four partial sums meet in LDS.
 __global__ __launch_bounds__(256) void score_reduce_kernel(const float* __restrict__ logits,
                                                            int64_t logits_stride,
                                                            const float* __restrict__ lse,
@@ -806,14 +900,28 @@ __global__ __launch_bounds__(256) void score_reduce_kernel(const float* __restri
                                                            float* __restrict__ out,
                                                            int64_t out_stride) {
   const int r = blockIdx.y;
-  const int i = blockIdx.x * 256 + threadIdx.x;
-  if (i >= n) return;
+  const int t = threadIdx.x & 63, hg = threadIdx.x >> 6;
+  const int i = blockIdx.x * 64 + t;
+  const int ic = i < n ? i : n - 1;  // loads stay unconditional
+  const float* base = logits + (int64_t)r * heads_per_row * logits_stride + ic;
+  const float* lrow = lse + r * heads_per_row;
   float acc = 0.f;
-  for (int j = 0; j < heads_per_row; ++j) {
-    const int h = r * heads_per_row + j;
-    acc += fast_exp2((logits[(int64_t)h * logits_stride + i] - lse[h]) * kLog2e);
+  int j = hg;
+  for (; j + 12 < heads_per_row; j += 16) {
+    const float x0 = base[(int64_t)j * logits_stride], x1 = base[(int64_t)(j + 4) * logits_stride],
+                x2 = base[(int64_t)(j + 8) * logits_stride], x3 = base[(int64_t)(j + 12) * logits_stride];
+    acc += fast_exp2((x0 - lrow[j]) * kLog2e);
+    acc += fast_exp2((x1 - lrow[j + 4]) * kLog2e);
+    acc += fast_exp2((x2 - lrow[j + 8]) * kLog2e);
+    acc += fast_exp2((x3 - lrow[j + 12]) * kLog2e);
   }
-  out[(int64_t)r * out_stride + i] = acc;
+  for (; j < heads_per_row; j += 4)
+    acc += fast_exp2((base[(int64_t)j * logits_stride] - lrow[j]) * kLog2e);
+  __shared__ float part[4][64];
+  part[hg][t] = acc;
+  __syncthreads();
+  if (hg == 0 && i < n)
+    out[(int64_t)r * out_stride + i] = (part[0][t] + part[1][t]) + (part[2][t] + part[3][t]);
 }
 
 }  // namespace tidal
@@ -856,12 +964,15 @@ extern "C" int td_topk(const void* values, int32_t values_dtype, int64_t values_
     uint32_t* ws = reinterpret_cast<uint32_t*>(workspace);
     const dim3 grid((rows + kXcds - 1) / kXcds * slices * kXcds), block(kTopkThreads);
     if (values_dtype == TD_F32) {
+      hipLaunchKernelGGL(topk_coop_hist_kernel<F32>, grid, block, 0, st, p, ws, slices, rows);
       hipLaunchKernelGGL(topk_coop_select_kernel<F32>, grid, block, 0, st, p, ws, slices, rows);
       hipLaunchKernelGGL(topk_coop_emit_kernel<F32>, grid, block, 0, st, p, ws, slices, rows);
     } else if (values_dtype == TD_F16) {
+      hipLaunchKernelGGL(topk_coop_hist_kernel<F16>, grid, block, 0, st, p, ws, slices, rows);
       hipLaunchKernelGGL(topk_coop_select_kernel<F16>, grid, block, 0, st, p, ws, slices, rows);
       hipLaunchKernelGGL(topk_coop_emit_kernel<F16>, grid, block, 0, st, p, ws, slices, rows);
     } else {
+      hipLaunchKernelGGL(topk_coop_hist_kernel<BF16>, grid, block, 0, st, p, ws, slices, rows);
       hipLaunchKernelGGL(topk_coop_select_kernel<BF16>, grid, block, 0, st, p, ws, slices, rows);
       hipLaunchKernelGGL(topk_coop_emit_kernel<BF16>, grid, block, 0, st, p, ws, slices, rows);
     }
@@ -898,7 +1009,7 @@ extern "C" int td_score_reduce(const float* logits, int64_t logits_stride, const
   TD_REQUIRE(rows == 1 || out_stride >= n, "td_score_reduce: out_stride %lld < n %d",
              (long long)out_stride, n);
   if (n == 0) return TD_OK;
-  hipLaunchKernelGGL(score_reduce_kernel, dim3((n + 255) / 256, rows), dim3(256), 0,
+  hipLaunchKernelGGL(score_reduce_kernel, dim3((n + 63) / 64, rows), dim3(256), 0,
                      reinterpret_cast<hipStream_t>(stream), logits, logits_stride, lse,
                      num_qo_heads / rows, n, out, out_stride);
   TD_HIP_CHECK(hipGetLastError());
