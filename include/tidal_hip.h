@@ -251,7 +251,8 @@ int td_topk(const void* values, int32_t values_dtype, int64_t values_stride, int
 
 /*
  * Bytes of device scratch that lets td_topk spread a row over several workgroups (rows of more
- * than 8192 elements; two launches).  The scratch must be zero-filled once before its first use;
+ * than 8192 elements; three launches; about 56 KiB per row).  The scratch must be zero-filled once
+ * before its first use;
  * every call leaves it ready for the next.  Without it (NULL) one workgroup handles each row.
  * Plays the part of the `buf` argument of topk_filtering (tidal/utils/controller.py:164-168).
  */
