@@ -4,18 +4,22 @@
 //
 // One 256-thread workgroup per (64 MT query rows, query head); a wavefront owns 16 MT query rows
 // as MT = 2 16-row tiles: every K/V operand read from LDS feeds two matrix instructions
-// (head_dim 256: 64 query rows per workgroup, MT = 1, key tiles of 32 tokens).  The loop walks the keys in tiles of 64 tokens that the workgroup stages once
-// in LDS (rows padded to 272 bytes: conflict-free 16-byte reads) while the global loads of the
-// next tile are already in flight.  Per 16 tokens and query tile:
+// (head_dim 256: 64 query rows per workgroup, MT = 1, key tiles of 32 tokens).  The loop walks
+// the keys in tiles of 64 tokens that the workgroup stages in LDS, two buffers per matrix (one
+// barrier per tile) and two tiles in flight in registers.  LDS rows are padded by 32 bytes
+// (288 for head_dim 128): gfx950 serves a 16-byte LDS read of lane 0 in one cycle with lanes
+// 1-3, 12-15 and 20-27 (measured), and with that grouping a pitch of 16 (4k + 2) bytes is free of
+// bank conflicts for the K operand reads and for the transposed V reads.  Per key tile:
 //   S^T = K Q^T   mfma_f32_16x16x32, A = K rows from LDS, B = Q rows kept in registers: an operand
 //                 is a 16-byte piece of a row;
 //   softmax       base-2, online; the result tile has the query row in lane % 16 and four
-//                 tokens per lane, which is the A-operand layout of the next product;
-//   O += P V      per 32 tokens: A = P (rounded to the KV type), B = V: a lane reads the rows of its
-//                 eight tokens (16 bytes each) and re-packs them with v_perm into one operand
-//                 per head dimension.
-// Pages are looked up per staged row; rows past the end of the sequence are clamped (never
-// out of the pool) and masked.
+//                 tokens per lane, which is the A-operand layout of the next product; the row
+//                 maximum crosses the four lane groups with v_permlane16/32_swap;
+//   O += P V      per 32 tokens: A = P (rounded to the KV type), B = V read with
+//                 ds_read_b64_tr_b16, which hands lane r dimension 16 a + r of four tokens.
+// Pages are looked up per staged row, one tile ahead; rows past the end of the sequence are
+// clamped (never out of the pool) and masked.  All query tiles of the heads that share a KV head
+// are placed on one XCD (see the block-index mapping in the kernel).
 
 #include "common.cuh"
 #include "../../include/tidal_hip.h"
