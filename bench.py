@@ -44,7 +44,7 @@ def parse():
     ap.add_argument("--waves", type=int, default=0, help="waves per workgroup (0 = default)")
     ap.add_argument("--chunk", type=int, default=0, help="tokens per workgroup (0 = default)")
     ap.add_argument("--merge", type=int, default=-1, help="1 fused / 0 second kernel / -1 default")
-    ap.add_argument("--rows", type=int, default=0, help="K/V loads per wave tile: 2 / 4 (0 = default)")
+    ap.add_argument("--rows", type=int, default=0, help="K/V loads per wave tile: 2 / 4 / 8 (0 = default)")
     ap.add_argument("--layout", default="NHD", choices=["NHD", "HND"], help="page layout")
     ap.add_argument("--no-fuse", action="store_true",
                     help="run RoPE + append as their own launch instead of inside attention")
@@ -524,9 +524,12 @@ def main():
                 for layer in sparse:
                     w.gather_probe(layer)
 
-            r_probe, _ = capture(torch, run_probe, use_graph)
-            entry["gather_only_us_per_layer"] = (time_events(torch, r_probe, max(args.steps, 20))
-                                                 * 1e3 / len(sparse))
+            try:
+                r_probe, _ = capture(torch, run_probe, use_graph)
+                entry["gather_only_us_per_layer"] = (time_events(torch, r_probe, max(args.steps, 20))
+                                                     * 1e3 / len(sparse))
+            except RuntimeError:   # the probe exists for the default tile shapes only
+                pass
         if not args.only_sparse:
             def run_select():
                 for layer in w.sel_layers:
