@@ -187,7 +187,8 @@ def test_topk_errors(cuda):
         _kernels.topk_filtering(v, None, None, big, None, 200)           # k > len
 
 
-@pytest.mark.parametrize("hq,hkv,n", [(32, 32, 4096), (32, 8, 5000), (40, 40, 33), (32, 8, 1)])
+@pytest.mark.parametrize("hq,hkv,n", [(32, 32, 4096), (32, 8, 5000), (40, 40, 33), (32, 8, 1),
+                                      (3, 1, 100), (64, 2, 777), (17, 17, 64), (20, 4, 65)])
 def test_score_reduce(cuda, hq, hkv, n):
     """sum over heads of softmax probabilities, from logits + lse, against the closed form."""
     from oracle import tidal_oracle as orc
