@@ -156,7 +156,7 @@ class Workload:
         return ops.decode_sparse_attn(self.q[layer], self.c, layer,
                                       self.c.topk_dindices_buffer, False, fresh=fresh)
 
-    def gather_probe(self, layer):
+    def gather_probe(self, layer, lists=None):
         """memory side of sparse_attn(layer) alone (no arithmetic, no merge)"""
         from tidaldecode_amd import _kernels
 
@@ -164,7 +164,8 @@ class Workload:
             self._probe_out = self.torch.empty(self.H * 64 * 16, dtype=self.torch.int32,
                                                device=self.dev)
         return _kernels.gather_probe(self.c._decode_handler._wrapper,
-                                     self.c.kv_cache.buf_layer(layer), self.c.topk_dindices_buffer,
+                                     self.c.kv_cache.buf_layer(layer),
+                                     self.c.topk_dindices_buffer if lists is None else lists,
                                      self._probe_out)
 
     def step(self):
@@ -528,6 +529,18 @@ def main():
                 r_probe, _ = capture(torch, run_probe, use_graph)
                 entry["gather_only_us_per_layer"] = (time_events(torch, r_probe, max(args.steps, 20))
                                                      * 1e3 / len(sparse))
+                # the same number of rows, but the first top_k slots of the pool for every head:
+                # what the launch costs when the rows are not scattered
+                dense = torch.arange(w.K, dtype=torch.int32, device=w.dev).repeat(
+                    w.c.topk_dindices_buffer.shape[0], 1).contiguous()
+
+                def run_probe_dense():
+                    for layer in sparse:
+                        w.gather_probe(layer, dense)
+
+                r_dense, _ = capture(torch, run_probe_dense, use_graph)
+                entry["gather_contiguous_us_per_layer"] = (
+                    time_events(torch, r_dense, max(args.steps, 20)) * 1e3 / len(sparse))
             except RuntimeError:   # the probe exists for the default tile shapes only
                 pass
         if not args.only_sparse:
