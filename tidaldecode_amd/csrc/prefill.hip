@@ -2,9 +2,9 @@
 // gfx950 (MI355X), on the matrix cores.  Replaces BatchPrefillWithPagedKVCache of the reference
 // (kernels/include/prefill/prefill.cuh:674-870, bound in tidal/ops/csrc/batch_prefill.cu:27-117).
 //
-// One 256-thread workgroup per (64 MT query rows, query head); a wavefront owns 16 MT query rows
-// as MT = 2 16-row tiles: every K/V operand read from LDS feeds two matrix instructions
-// (head_dim 256: 64 query rows per workgroup, MT = 1, key tiles of 32 tokens).  The loop walks
+// One workgroup of NW = 4 or 8 wavefronts per (16 MT NW query rows, query head); a wavefront owns
+// 16 MT query rows as MT = 2 16-row tiles: every K/V operand read from LDS feeds two matrix
+// instructions (head_dim 256: MT = 1, key tiles of 32 tokens).  The loop walks
 // the keys in tiles of 64 tokens that the workgroup stages in LDS, two buffers per matrix (one
 // barrier per tile) and two tiles in flight in registers.  LDS rows are padded by 32 bytes
 // (288 for head_dim 128): gfx950 serves a 16-byte LDS read of lane 0 in one cycle with lanes
@@ -26,7 +26,6 @@
 
 namespace tidal {
 
-constexpr int kPfThreads = 256;
 
 // LDS read with transpose (gfx950): within every 16 lanes, lane 4a + b receives element b of the
 // four 8-byte pieces addressed by lanes a, a + 4, a + 8, a + 12.
@@ -51,10 +50,12 @@ struct PrefillParams {
   int32_t causal;
 };
 
-// BN tokens per key tile (a multiple of 32)
-template <typename T, int D, int MT, int BN>
-__global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kernel(const PrefillParams p) {
-  constexpr int kPfBM = 64 * MT;    // query rows per workgroup
+// BN tokens per key tile (a multiple of 32), NW wavefronts per workgroup (4 or 8: a staged K/V
+// tile serves 16 MT NW query rows, so eight waves halve the global -> LDS traffic per flop)
+template <typename T, int D, int MT, int BN, int NW>
+__global__ __launch_bounds__(64 * NW, MT == 2 ? 2 : 1) void prefill_attn_kernel(const PrefillParams p) {
+  constexpr int kThreads = 64 * NW;
+  constexpr int kPfBM = 16 * MT * NW;  // query rows per workgroup
   constexpr int WR = 16 * MT;       // query rows per wavefront
   constexpr int NS = D / 32;        // 16-byte pieces of a Q/K row per lane (one MFMA each)
   constexpr int DC = D / 16;        // head dimensions per lane in the P.V product
@@ -62,11 +63,12 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
   constexpr int CPR = D / 8;        // 16-byte chunks per row
   constexpr int kPfBN = BN;
   constexpr int NSUB = BN / 16;     // 16-token sub-tiles per key tile
-  constexpr int RPT = BN / 32;      // staging: rows per thread (row = tid / 8 + 32 jr)
+  constexpr int SR = kThreads / 8;  // staging: rows per pass (8 lanes per row piece)
+  constexpr int RPT = BN / SR;      // staging: rows per thread (row = tid / 8 + SR jr)
   constexpr int CCT = CPR / 8;      // staging: chunks per thread and row (chunk = tid % 8 + 8 jc)
   constexpr int CPT = RPT * CCT;    // chunks a thread stages per tile and matrix
   static_assert(D == 64 || D == 128 || D == 256, "head dimensions of the prefill kernel");
-  static_assert(BN % 32 == 0 && CPT * kPfThreads == BN * CPR, "key tile");
+  static_assert(BN % 32 == 0 && RPT >= 1 && CPT * kThreads == BN * CPR, "key tile");
   // two buffers per matrix: tile t + 1 is written while tile t is still being read
   constexpr int TILE = kPfBN * PITCH;
   __shared__ __attribute__((aligned(16))) uint16_t ks[2 * TILE];
@@ -137,7 +139,7 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
   // never wait for a page-table load issued in the same iteration
   uint32_t pg[RPT];
   auto split_tok = [&](int kt, int jr, int& pg_i, int& entry) {
-    int tok = kt + srow + 32 * jr;
+    int tok = kt + srow + SR * jr;
     tok = tok < p.kv_len ? tok : p.kv_len - 1;
     if (p.page_shift >= 0) {
       pg_i = tok >> p.page_shift;
@@ -175,7 +177,7 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
     for (int jr = 0; jr < RPT; ++jr)
 #pragma unroll
       for (int jc = 0; jc < CCT; ++jc) {
-        const int at = buf * TILE + (srow + 32 * jr) * PITCH + (sl8 + 8 * jc) * 8;
+        const int at = buf * TILE + (srow + SR * jr) * PITCH + (sl8 + 8 * jc) * 8;
         *reinterpret_cast<u32x4*>(&ks[at]) = kreg[jr * CCT + jc];
         *reinterpret_cast<u32x4*>(&vs[at]) = vreg[jr * CCT + jc];
       }
@@ -340,258 +342,28 @@ __global__ __launch_bounds__(kPfThreads, MT == 2 ? 2 : 1) void prefill_attn_kern
   }
 }
 
-// head_dim 128 with power-of-two pages: the K/V tiles go from global memory straight into LDS
-// (global_load_lds_dwordx4: no staging registers, no LDS store instructions).  One such
-// instruction fills 1 KiB = four unpadded 256-byte rows, so bank conflicts are avoided by
-// position instead of padding: the 16-byte chunk c of row rho sits at chunk position
-// c ^ (2 rho mod 16).  With the lane grouping of gfx950's LDS (see the file header) that is
-// conflict-free for the K operand reads (row = lane % 16, chunk = lane / 16 + 4 s) and for the
-// transposed V reads (8 consecutive rows per 32 lanes land in 8 different 32-byte columns).  The
-// permutation is applied on the global side: lane L of instruction j of wave w fetches chunk
-// (L % 16) ^ (2 row mod 16) of row 16 w + 4 j + L / 16.
-template <typename T>
-__global__ __launch_bounds__(kPfThreads, 2) void prefill_attn_d128_kernel(const PrefillParams p) {
-  constexpr int D = 128, MT = 2, BN = 64;
-  constexpr int kPfBM = 64 * MT, WR = 16 * MT, NS = D / 32, DC = D / 16, NSUB = BN / 16;
-  constexpr int ROWB = 2 * D;          // bytes of an LDS row
-  constexpr int TILEB = BN * ROWB;     // bytes of one matrix tile
-  __shared__ __attribute__((aligned(1024))) uint8_t kl[2 * TILEB];
-  __shared__ __attribute__((aligned(1024))) uint8_t vl[2 * TILEB];
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int r = lane & 15, g = lane >> 4;
-  int qtile, qh;
-  {
-    const int n_tiles = gridDim.x, n_heads = gridDim.y;
-    const int lin = blockIdx.x + n_tiles * blockIdx.y;
-    const int n_kv = n_heads / p.q_per_kv;
-    if (n_kv % 8 == 0) {  // all query tiles of the heads of one KV head on one XCD (see above)
-      const int xcd = lin & 7, slot = lin >> 3;
-      const int idx = slot / n_tiles;
-      qtile = n_tiles - 1 - slot % n_tiles;
-      qh = ((idx / p.q_per_kv) * 8 + xcd) * p.q_per_kv + idx % p.q_per_kv;
-    } else {
-      qtile = n_tiles - 1 - blockIdx.x;
-      qh = blockIdx.y;
-    }
-  }
-  const int kvh = qh / p.q_per_kv;
-  const int q0 = qtile * kPfBM;
-  const int q_off = p.kv_len - p.n_q;
-
-  u32x4 qb[MT][NS];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    int row = q0 + wave * WR + mt * 16 + r;
-    row = row < p.n_q ? row : p.n_q - 1;
-    const u32x4* src =
-        reinterpret_cast<const u32x4*>(p.q + ((int64_t)row * p.num_qo_heads + qh) * D);
-#pragma unroll
-    for (int s = 0; s < NS; ++s) qb[mt][s] = src[4 * s + g];
-  }
-  f32x4 oacc[MT][DC];
-  float m_run[MT], l_run[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    m_run[mt] = kNegBig;
-    l_run[mt] = 0.f;
-#pragma unroll
-    for (int d = 0; d < DC; ++d) oacc[mt][d] = f32x4{0.f, 0.f, 0.f, 0.f};
-  }
-  int last_row = q0 + kPfBM - 1;
-  last_row = last_row < p.n_q ? last_row : p.n_q - 1;
-  const int kv_end = p.causal ? (q_off + last_row + 1) : p.kv_len;
-  const int wave_first_pos = q_off + q0 + wave * WR;
-
-  // ---- staging: wave w moves rows [16 w, 16 w + 16) of a tile, four per instruction ------------
-  const int lrow = lane >> 4;
-  uint32_t pg[4];  // page ids of this lane's four rows, looked up one tile ahead
-  auto row_tok = [&](int kt, int j) {
-    const int tok = kt + 16 * wave + 4 * j + lrow;
-    return tok < p.kv_len ? tok : p.kv_len - 1;
-  };
-  auto lookup = [&](int kt) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) pg[j] = (uint32_t)p.page_table[row_tok(kt, j) >> p.page_shift];
-  };
-  auto issue = [&](int kt, int stage) {  // needs lookup(kt) before it
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int tok = row_tok(kt, j);
-      const int entry = tok & (p.page_size - 1);
-      const uint32_t page = pg[j] > p.max_page ? p.max_page : pg[j];
-      const int chunk = (lane & 15) ^ ((8 * j + 2 * lrow) & 15);  // 2 (16 w + 4 j + lrow) mod 16
-      const uint16_t* src = p.kv + ((int64_t)page * p.page_stride + (int64_t)entry * p.entry_stride +
-                                    (int64_t)kvh * p.head_stride + chunk * 8);
-      const int at = stage * TILEB + (16 * wave + 4 * j) * ROWB;
-      __builtin_amdgcn_global_load_lds(src, (__attribute__((address_space(3))) void*)(kl + at), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds(src + p.v_offset,
-                                       (__attribute__((address_space(3))) void*)(vl + at), 16, 0, 0);
-    }
-  };
-
-  // ---- operand addresses (bytes inside a tile), fixed per lane ------------------------------------
-  int kaddr[NS];  // K: row r of a 16-row sub-tile, chunk g + 4 s at position (g + 4 s) ^ (2 r mod 16)
-#pragma unroll
-  for (int s = 0; s < NS; ++s) kaddr[s] = r * ROWB + (((g + 4 * s) ^ ((2 * r) & 15)) << 4);
-  // V: row 4 g + r / 4 of a 16-row block; the 32-byte column a of that row sits at column
-  // a ^ (row mod 8); inside it the 8-byte piece r % 4
-  int vaddr[DC];
-  {
-    const int vrow = 4 * g + (r >> 2);
-#pragma unroll
-    for (int a = 0; a < DC; ++a)
-      vaddr[a] = vrow * ROWB + ((a ^ (vrow & 7)) << 5) + ((r & 3) << 3);
-  }
-
-  auto compute = [&](int kt, int stage) {
-    if (!p.causal || kt <= wave_first_pos + WR - 1) {
-      __builtin_amdgcn_s_setprio(2);
-      f32x4 st[MT][NSUB];
-#pragma unroll
-      for (int sub = 0; sub < NSUB; ++sub) {
-        u32x4 ka[NS];
-#pragma unroll
-        for (int s = 0; s < NS; ++s)
-          ka[s] = *reinterpret_cast<const u32x4*>(kl + stage * TILEB + sub * 16 * ROWB + kaddr[s]);
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int s = 0; s < NS; ++s) acc = mfma_16x16x32<T>(ka[s], qb[mt][s], acc);
-          st[mt][sub] = acc;
-        }
-      }
-      __builtin_amdgcn_s_setprio(0);
-      uint32_t pa[MT][NSUB][2];
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const int qpos = wave_first_pos + mt * 16 + r;
-        const bool need_mask =
-            (p.causal && kt + BN - 1 > wave_first_pos) || kt + BN > p.kv_len;
-        if (need_mask) {
-#pragma unroll
-          for (int sub = 0; sub < NSUB; ++sub)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const int tpos = kt + sub * 16 + 4 * g + i;
-              const bool ok = tpos < p.kv_len && (!p.causal || tpos <= qpos);
-              st[mt][sub][i] = ok ? st[mt][sub][i] : kNegBig;
-            }
-        }
-        float mt_max = kNegBig;
-#pragma unroll
-        for (int sub = 0; sub < NSUB; ++sub)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) mt_max = fmaxf(mt_max, st[mt][sub][i]);
-        mt_max = rows_max(mt_max);
-        // the running maximum moves only on steps of more than 2^8 (see the general kernel)
-        const float m_tile = mt_max * p.scale_log2;
-        const float m_new = m_tile > m_run[mt] + 8.f ? m_tile : m_run[mt];
-        const float alpha = fast_exp2(m_run[mt] - m_new);
-        m_run[mt] = m_new;
-        float psum = 0.f;
-#pragma unroll
-        for (int sub = 0; sub < NSUB; ++sub) {
-          float pr[4];
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            pr[i] = fast_exp2(fmaf(st[mt][sub][i], p.scale_log2, -m_new));
-            psum += pr[i];
-          }
-          pa[mt][sub][0] = pack2<T>(pr[0], pr[1]);
-          pa[mt][sub][1] = pack2<T>(pr[2], pr[3]);
-        }
-        l_run[mt] = fmaf(l_run[mt], alpha, psum);
-        if (__ballot(alpha != 1.f)) {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const float f = __shfl(alpha, 4 * g + i, 64);
-#pragma unroll
-            for (int d = 0; d < DC; ++d) oacc[mt][d][i] *= f;
-          }
-        }
-      }
-      __builtin_amdgcn_s_setprio(2);
-#pragma unroll
-      for (int pair = 0; pair < NSUB / 2; ++pair) {
-#pragma unroll
-        for (int a = 0; a < DC; ++a) {
-          const uint8_t* vb0 = vl + stage * TILEB + (32 * pair) * ROWB + vaddr[a];
-          const u32x2 t0 = lds_read_tr16(reinterpret_cast<const uint16_t*>(vb0));
-          const u32x2 t1 = lds_read_tr16(reinterpret_cast<const uint16_t*>(vb0 + 16 * ROWB));
-          const u32x4 vb = {t0.x, t0.y, t1.x, t1.y};
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt) {
-            const u32x4 pp = {pa[mt][2 * pair][0], pa[mt][2 * pair][1], pa[mt][2 * pair + 1][0],
-                              pa[mt][2 * pair + 1][1]};
-            oacc[mt][a] = mfma_16x16x32<T>(pp, vb, oacc[mt][a]);
-          }
-        }
-      }
-      __builtin_amdgcn_s_setprio(0);
-    }
-  };
-
-  lookup(0);
-  issue(0, 0);
-  lookup(BN);
-  // One barrier per tile.  __syncthreads waits for this wave's outstanding loads (the tile's
-  // rows are in LDS when the counter is zero) before the barrier, and every wave reaches it only
-  // after its reads of the other stage, which is then refilled while this stage is computed on.
-  for (int kt = 0; kt < kv_end; kt += 2 * BN) {
-    __syncthreads();
-    if (kt + BN < kv_end) {
-      issue(kt + BN, 1);
-      lookup(kt + 2 * BN);
-    }
-    compute(kt, 0);
-    if (kt + BN >= kv_end) break;
-    __syncthreads();
-    if (kt + 2 * BN < kv_end) {
-      issue(kt + 2 * BN, 0);
-      lookup(kt + 3 * BN);
-    }
-    compute(kt + BN, 1);
-  }
-
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const float l = rows_sum(l_run[mt]);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float li = __shfl(l, 4 * g + i, 64);
-      const float inv = li > 0.f ? 1.f / li : 0.f;
-      const int row = q0 + wave * WR + mt * 16 + 4 * g + i;
-      if (row < p.n_q) {
-        uint16_t* dst = p.o + ((int64_t)row * p.num_qo_heads + qh) * D + r;
-#pragma unroll
-        for (int a = 0; a < DC; ++a) dst[16 * a] = from_float<T>(oacc[mt][a][i] * inv);
-      }
-    }
-  }
-}
-
 template <typename T>
 static int launch_prefill(const PrefillParams& p, int head_dim, hipStream_t st) {
-  // Two query tiles per wavefront and 64-token key tiles keep the kernel at 256 registers, i.e.
-  // two workgroups per compute unit: one computes while the other waits for its next K/V tile.
-  // (Four query tiles per wavefront halve the LDS traffic per flop but run one workgroup per
-  // compute unit with every memory and barrier latency exposed: 2.5x slower.)  head_dim 256 has
+  // Two query tiles per wavefront and 64-token key tiles keep the kernel within 256 registers
+  // (two waves per SIMD).  Staging a K/V tile (global loads, page lookups, LDS stores) costs a
+  // quarter of the kernel's time, so head_dim 128 runs eight waves per workgroup: one staged tile
+  // serves 256 query rows (8.9 -> 8.4 ms per layer at 32K x 32 heads); prompts of up to 128 rows
+  // keep four.  (Four query tiles per wavefront halve the LDS traffic per flop but need twice
+  // the registers: one wave per SIMD with every latency exposed, 2.5x slower.)  head_dim 256 has
   // twice the accumulators and twice the LDS per token: one query tile per wavefront, 32-token
   // key tiles.
-  const dim3 block(kPfThreads);
-  if (head_dim == 128 && p.page_shift >= 0)
-    hipLaunchKernelGGL(prefill_attn_d128_kernel<T>, dim3((p.n_q + 127) / 128, p.num_qo_heads), block,
-                       0, st, p);
+  const dim3 block(256);
+  if (head_dim == 128 && p.n_q > 128)
+    hipLaunchKernelGGL((prefill_attn_kernel<T, 128, 2, 64, 8>), dim3((p.n_q + 255) / 256, p.num_qo_heads),
+                       dim3(512), 0, st, p);
   else if (head_dim == 128)
-    hipLaunchKernelGGL((prefill_attn_kernel<T, 128, 2, 64>), dim3((p.n_q + 127) / 128, p.num_qo_heads),
+    hipLaunchKernelGGL((prefill_attn_kernel<T, 128, 2, 64, 4>), dim3((p.n_q + 127) / 128, p.num_qo_heads),
                        block, 0, st, p);
   else if (head_dim == 64)
-    hipLaunchKernelGGL((prefill_attn_kernel<T, 64, 2, 64>), dim3((p.n_q + 127) / 128, p.num_qo_heads),
+    hipLaunchKernelGGL((prefill_attn_kernel<T, 64, 2, 64, 4>), dim3((p.n_q + 127) / 128, p.num_qo_heads),
                        block, 0, st, p);
   else if (head_dim == 256)
-    hipLaunchKernelGGL((prefill_attn_kernel<T, 256, 1, 32>), dim3((p.n_q + 63) / 64, p.num_qo_heads),
+    hipLaunchKernelGGL((prefill_attn_kernel<T, 256, 1, 32, 4>), dim3((p.n_q + 63) / 64, p.num_qo_heads),
                        block, 0, st, p);
   else
     return fail(TD_ERR_UNSUPPORTED,
