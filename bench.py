@@ -279,7 +279,7 @@ def e2e_leg(args):
         cfg = TidalLlamaConfig.llama2_7b(top_k=args.top_k, sparse_layer_start=0, correction_layer=2,
                                          select_mode=args.select_mode)
     model = TidalLlama(cfg, "cuda:0", seed=0)
-    model.tidal_init(page_size=16, max_seq_len=max(ctxs) + 128, page_order_seed=0)
+    model.tidal_init(page_size=16, max_seq_len=max(ctxs) + 512, page_order_seed=0)
     out = {}
     for ctx in ctxs:
         row = {}
