@@ -380,7 +380,7 @@ def sweep(args):
                     f"page 16, {args.select_mode} lists, selection layers 0 and 2", "rows": []}
     for ctx in (10240, 32768, 102400):
         full_ms = None
-        for budget in (256, 1024, 2048, 4096):
+        for budget in (32, 64, 128, 256, 512, 1024, 2048, 4096):
             a = copy.copy(args)
             a.ctx, a.top_k = ctx, budget
             w = Workload(a, args.select_mode)
