@@ -459,22 +459,20 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
         sv[u] = (base + u * TPI + g < c1) ? x : kNegBig;
       }
       if constexpr (EMIT) {
-        // One store per four heads and tile: lane L collects the logit of (head L / 16, token
-        // base + L % 16), which lane group (L % 16) % TPI holds in its lane of that head for row
-        // (L % 16) / TPI, so that a head's 16 logits of the tile leave as 64 contiguous bytes.
-        static_assert(TPI == 4 && U == 4, "logit transposition of the grouped-query tile");
+        // The 16 / QPG lanes of a row that hold the same head hold the same sums, so no value has
+        // to move between lanes: copy c = li / QPG of head li % QPG stores the logit of the tile's
+        // row c (token base + c TPI + g).  Over the four lane groups a head's 16 logits of the
+        // tile are written as 64 contiguous bytes by one instruction (two for QPG = 8).
+        constexpr int COPIES = 16 / QPG;
+        const int head = li % QPG, c = li / QPG;
 #pragma unroll
-        for (int hb = 0; hb < (QPG + 3) / 4; ++hb) {
-          const int src = (lane & 3) * 16 + hb * 4 + (lane >> 4);
-          float e = 0.f;
+        for (int u0 = 0; u0 < U; u0 += COPIES) {
+          float e = xe[u0];
 #pragma unroll
-          for (int u = 0; u < U; ++u) {
-            const float v = __shfl(xe[u], src, 64);
-            e = (((lane >> 2) & 3) == u) ? v : e;
-          }
-          const int head = hb * 4 + (lane >> 4);
-          const int i = base + (lane & 15);
-          if (head < QPG && i < c1) {
+          for (int x = 1; x < COPIES; ++x)
+            if (u0 + x < U) e = (c == x) ? xe[u0 + x] : e;
+          const int i = base + (u0 + c) * TPI + g;
+          if (u0 + c < U && i < c1) {
             const int64_t at = ((int64_t)b * p.num_qo_heads + qh0 + head) * p.score_stride + i;
             const float nat = e * kLn2;
             if (p.scores_f32)
@@ -552,16 +550,15 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
       }
     }
     if constexpr (EMIT) {
-      // one store per tile: lane L < TILE collects the logit of token base + L (row L / TPI of
-      // lane group L % TPI) and the TILE lanes write consecutive addresses
-      float e = 0.f;
+      // every lane of a lane group holds the group's U logits, so lane li < U of group g stores
+      // row li (token base + li TPI + g): one instruction writes the tile's TILE consecutive
+      // logits and nothing moves between lanes
+      static_assert(U <= LPR, "one lane of the group per row of the tile");
+      float e = sc[0][0];
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const float v = __shfl(sc[0][u], (lane % TPI) * LPR, 64);
-        e = (lane / TPI == u) ? v : e;
-      }
-      const int i = base + lane;
-      if (lane < TILE && i < c1) {
+      for (int u = 1; u < U; ++u) e = (li == u) ? sc[0][u] : e;
+      const int i = base + li * TPI + g;
+      if (li < U && i < c1) {
         const int64_t at = ((int64_t)b * p.num_qo_heads + qh0) * p.score_stride + i;
         const float nat = e * kLn2;
         if (p.scores_f32)
