@@ -319,3 +319,57 @@ def test_error_paths(cuda):
     pool48 = torch.zeros((4, 2, 16, 32, 48), dtype=torch.float16, device=cuda)
     with pytest.raises(RuntimeError, match="head_dim"):
         w48.forward(q48, q48.clone(), pool48, idx, None, 1, 0, None)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_configurations(cuda, seed):
+    """Seeded random draws over what the grids above enumerate one axis at a time: head counts and
+    group sizes, head_dim, page size, layout, dtype, length, budget, list rows, duplicates-free
+    token lists (slots) and the selection-layer mode (whole page table + logits) on the same
+    case.  Every draw is checked against the oracle's gathered / dense attention."""
+    import random
+
+    from oracle import tidal_oracle as orc
+
+    rnd = random.Random(1000 + seed)
+    dtype = rnd.choice([torch.float16, torch.bfloat16])
+    d = rnd.choice([64, 128, 128, 256])
+    hkv = rnd.choice([1, 2, 4, 8])
+    group = rnd.choice([1, 1, 2, 4, 8]) if d == 128 else rnd.choice([1, 2, 4])
+    hq = hkv * group
+    page_size = rnd.choice([1, 2, 4, 8, 16, 16, 32])
+    layout = rnd.choice([0, 1])
+    n = rnd.choice([1, 7, 16, 33, 250, 1000, 2500, 6000])
+    case = PagedCase(n, hkv, d, page_size, dtype, layout=layout, seed=seed + 50)
+    q = randn((hq, d), seed + 99, dtype)
+    w = _wrapper(layout, hq, hkv, d, page_size, dtype)
+    qd = q.to(dtype).to(cuda).unsqueeze(0)
+    pool = case.pool.to(cuda)
+
+    # token lists: per query head, per KV head or shared
+    rows = rnd.choice(sorted({1, hkv, hq}))
+    k = rnd.randint(1, n)
+    g = torch.Generator().manual_seed(seed)
+    pos = torch.stack([torch.randperm(n, generator=g)[:k] for _ in range(rows)])
+    want = orc.sparse_layer_gather(q, case.k, case.v, pos)
+    od = torch.empty_like(qd)
+    w.forward(qd, od, pool, case.slots_of(pos).to(torch.int32).to(cuda), None, 0, 0, None,
+              index_kind="slots")
+    torch.cuda.synchronize()
+    assert tolerance_report(od[0], want) <= ATOL[dtype], ("slots", dtype, d, hq, hkv, page_size, layout, n, k, rows)
+
+    # selection-layer mode on the same cache
+    logits = orc.attn_logits(q, case.k)
+    want_full = orc.softmax_pv(logits, case.v)
+    stride = case.n_pages * page_size
+    scores = torch.full((hq, stride), float("nan"), dtype=torch.float32, device=cuda)
+    lse = torch.empty((1, hq), dtype=torch.float32, device=cuda)
+    table = case.page_table[:-1].to(torch.int32).unsqueeze(0)
+    od2 = torch.empty_like(qd)
+    w.forward(qd, od2, pool, table.to(cuda), None, case.last_page_len, int(case.page_table[-1]),
+              scores, lse=lse)
+    torch.cuda.synchronize()
+    assert tolerance_report(od2[0], want_full) <= ATOL[dtype], ("pages", dtype, d, hq, hkv, page_size, layout, n)
+    assert (scores[:, :n].cpu() - logits).abs().max() <= 2e-4 * max(1.0, logits.abs().max().item())
+    assert torch.isnan(scores[:, n:]).all()
+    assert (lse[0].cpu() - torch.logsumexp(logits, -1)).abs().max() <= 1e-3

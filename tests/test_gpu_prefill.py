@@ -127,3 +127,28 @@ def test_prefill_errors(cuda):
     with pytest.raises(RuntimeError):   # dtype mismatch
         _kernels.prefill_with_paged_kv_cache(q[:8].bfloat16(), pool, table, 16, True, 0, False,
                                              1.0, 1e4)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_configurations(cuda, seed):
+    """Seeded random draws over head counts (incl. the 8-KV-head placement path and the eight-wave
+    workgroups above 128 query rows), head_dim, page size, layout, dtype, causal, cache and query
+    lengths."""
+    import random
+
+    rnd = random.Random(500 + seed)
+    dtype = rnd.choice([torch.float16, torch.bfloat16])
+    d = rnd.choice([64, 128, 128, 128, 256])
+    hkv = rnd.choice([1, 2, 3, 8])
+    hq = hkv * rnd.choice([1, 2, 4])
+    page = rnd.choice([1, 3, 4, 8, 16, 16, 32])
+    layout = rnd.choice([0, 1])
+    causal = rnd.random() < 0.75
+    kv_len = rnd.choice([1, 31, 64, 129, 257, 700, 1500, 2100])
+    n_q = rnd.randint(1, kv_len)
+    case = PagedCase(kv_len, hkv, d, page, dtype, layout=layout, seed=seed + 7)
+    q = randn((n_q, hq, d), seed + 31, dtype)
+    want = _dense(q, case.k, case.v, causal)
+    got = _run(cuda, case, q, causal, dtype)
+    ok = (got.float().cpu() - want).abs() <= ATOL[dtype] * want.abs().clamp(min=1.0)
+    assert ok.all(), (dtype, d, hq, hkv, page, layout, causal, kv_len, n_q)
