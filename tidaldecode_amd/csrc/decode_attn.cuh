@@ -430,6 +430,46 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
             reinterpret_cast<const u32x4*>(kv16 + offs[u] + p.v_offset));
     }
   };
+  // ---- logits (EMIT) ------------------------------------------------------------------------------
+  // Vector stores and loads share one in-order completion counter, so a store issued per tile
+  // holds back the wait for every younger K/V or list load until its write is acknowledged.  The
+  // logits are therefore collected in a per-wave LDS strip and written EMIT_TILES tiles at a
+  // time: the stores enter the memory queue once per batch (once per launch for most shapes).
+  constexpr int EMIT_FLOATS = EMIT ? (NW == 16 ? 512 : 1024) : 1;  // per wave
+  constexpr int EMIT_TILES = EMIT ? EMIT_FLOATS / (QPG * TILE) : 1;
+  static_assert(EMIT_TILES >= 1, "logit strip too small for one tile");
+  __shared__ float emit_buf[EMIT ? NW * EMIT_FLOATS : 1];
+  int emit_n = 0;       // tiles waiting in the strip
+  int emit_first = 0;   // first token of the oldest waiting tile
+  const int emit_step = n_splits * NW * TILE;  // tokens between two tiles of this wave
+  auto emit_flush = [&]() {
+    if constexpr (EMIT) {
+      // a store instruction covers 64 / TILE tiles of one head: lane -> (tile, token)
+      constexpr int TPS = 64 / TILE >= 1 ? 64 / TILE : 1;  // tiles per store (TILE <= 64)
+      const int lt = lane / TILE, ltok = lane % TILE;
+      for (int n0 = 0; n0 < emit_n; n0 += TPS) {
+        const int n = n0 + lt;
+        const int i = emit_first + n * emit_step + ltok;
+#pragma unroll
+        for (int j = 0; j < QPG; ++j) {
+          if (n < emit_n && i < c1) {
+            const float nat = emit_buf[((wave * EMIT_TILES + n) * QPG + j) * TILE + ltok];
+            const int64_t at = ((int64_t)b * p.num_qo_heads + qh0 + j) * p.score_stride + i;
+            if (p.scores_f32)
+              reinterpret_cast<float*>(p.scores)[at] = nat;
+            else
+              reinterpret_cast<uint16_t*>(p.scores)[at] = from_float<T>(nat);
+          }
+        }
+      }
+      emit_n = 0;
+    }
+  };
+  auto emit_push = [&](int base) {  // the tile that starts at token `base` is in the strip
+    if (emit_n == 0) emit_first = base;
+    if (++emit_n == EMIT_TILES) emit_flush();
+  };
+
   auto reduce = [&](u32x4(&kb)[U], u32x4(&vb)[U], int base, uint32_t hit) {
     if constexpr (FRESH) {
       if (__ballot(hit != 0)) {  // rare: some lane group of this wave meets the new token
@@ -460,27 +500,21 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
       }
       if constexpr (EMIT) {
         // The 16 / QPG lanes of a row that hold the same head hold the same sums, so no value has
-        // to move between lanes: copy c = li / QPG of head li % QPG stores the logit of the tile's
-        // row c (token base + c TPI + g).  Over the four lane groups a head's 16 logits of the
-        // tile are written as 64 contiguous bytes by one instruction (two for QPG = 8).
+        // to move between lanes: copy c = li / QPG of head li % QPG keeps the logit of the tile's
+        // row c (token base + c TPI + g).  The logits wait in the wave's LDS strip, laid out
+        // [tile][head][token], and leave in batches (see emit_flush).
         constexpr int COPIES = 16 / QPG;
         const int head = li % QPG, c = li / QPG;
+        float* strip = emit_buf + (wave * EMIT_TILES + emit_n) * (QPG * TILE);
 #pragma unroll
         for (int u0 = 0; u0 < U; u0 += COPIES) {
           float e = xe[u0];
 #pragma unroll
           for (int x = 1; x < COPIES; ++x)
             if (u0 + x < U) e = (c == x) ? xe[u0 + x] : e;
-          const int i = base + (u0 + c) * TPI + g;
-          if (u0 + c < U && i < c1) {
-            const int64_t at = ((int64_t)b * p.num_qo_heads + qh0 + head) * p.score_stride + i;
-            const float nat = e * kLn2;
-            if (p.scores_f32)
-              reinterpret_cast<float*>(p.scores)[at] = nat;
-            else
-              reinterpret_cast<uint16_t*>(p.scores)[at] = from_float<T>(nat);
-          }
+          if (u0 + c < U) strip[head * TILE + (u0 + c) * TPI + g] = e * kLn2;
         }
+        emit_push(base);
       }
       float mt = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
       mt = rows_max(mt);  // the tile's maximum over all four lane groups
@@ -550,22 +584,15 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
       }
     }
     if constexpr (EMIT) {
-      // every lane of a lane group holds the group's U logits, so lane li < U of group g stores
-      // row li (token base + li TPI + g): one instruction writes the tile's TILE consecutive
-      // logits and nothing moves between lanes
+      // every lane of a lane group holds the group's U logits, so lane li < U of group g keeps
+      // row li (token base + li TPI + g) and nothing moves between lanes; the logits wait in the
+      // wave's LDS strip and leave in batches (see emit_flush)
       static_assert(U <= LPR, "one lane of the group per row of the tile");
       float e = sc[0][0];
 #pragma unroll
       for (int u = 1; u < U; ++u) e = (li == u) ? sc[0][u] : e;
-      const int i = base + li * TPI + g;
-      if (li < U && i < c1) {
-        const int64_t at = ((int64_t)b * p.num_qo_heads + qh0) * p.score_stride + i;
-        const float nat = e * kLn2;
-        if (p.scores_f32)
-          reinterpret_cast<float*>(p.scores)[at] = nat;
-        else
-          reinterpret_cast<uint16_t*>(p.scores)[at] = from_float<T>(nat);
-      }
+      if (li < U) emit_buf[(wave * EMIT_TILES + emit_n) * TILE + li * TPI + g] = e * kLn2;
+      emit_push(base);
     }
 #pragma unroll
     for (int j = 0; j < QPG; ++j) {
@@ -629,6 +656,7 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
   } else {
     finish_fresh();  // a wave without tokens still takes part in the shuffles and the write
   }
+  emit_flush();
 
   // ---- combine the TPI token slots of the wave (butterfly over lane groups) ---------------------
   if constexpr (QPG > 1) {  // the matrix product already summed the groups; only lh is per group
