@@ -814,6 +814,26 @@ __global__ __launch_bounds__(kTopkThreads) void topk_coop_emit_kernel(const Topk
     const uint32_t kv = coop_key<T>(vals, i < len ? i : len - 1);
     key[j] = i < len ? kv : 0u;  // 0 lies below every real key
   }
+  int32_t* out_idx = p.out_idx + (int64_t)row * p.out_stride;
+  elem_t* out_val =
+      p.out_values ? reinterpret_cast<elem_t*>(p.out_values) + (int64_t)row * p.out_stride : nullptr;
+  // Payloads and values of every element are fetched right away, unconditionally (they sit in
+  // L2): together with the keys they are one round trip, and no load follows a store (vector
+  // loads and stores complete in order on one counter).
+  int32_t payload[kCoopIPT];
+  elem_t val[kCoopIPT];
+#pragma unroll
+  for (int j = 0; j < kCoopIPT; ++j) {
+    int i = slice * kCoopSlice + j * kTopkThreads + tid;
+    i = i < len ? i : len - 1;
+    if (p.in_idx)
+      payload[j] = p.in_idx[(int64_t)row * p.in_idx_stride + i];
+    else if (p.page_table)
+      payload[j] = slot_of(p, i);
+    else
+      payload[j] = i;
+    if (out_val) val[j] = vals[i];
+  }
 #pragma unroll
   for (int j = 0; j < kCoopIPT; ++j) {
     const uint32_t n_gt = (uint32_t)__popcll(__ballot(key[j] > thr));
@@ -839,9 +859,6 @@ __global__ __launch_bounds__(kTopkThreads) void topk_coop_emit_kernel(const Topk
     }
   }
   __syncthreads();
-  int32_t* out_idx = p.out_idx + (int64_t)row * p.out_stride;
-  elem_t* out_val =
-      p.out_values ? reinterpret_cast<elem_t*>(p.out_values) + (int64_t)row * p.out_stride : nullptr;
 #pragma unroll
   for (int j = 0; j < kCoopIPT; ++j) {
     const bool gt = key[j] > thr;
@@ -852,16 +869,8 @@ __global__ __launch_bounds__(kTopkThreads) void topk_coop_emit_kernel(const Topk
     const uint64_t sel_mask = __ballot(sel);
     const uint32_t pos = run_out[j * kTopkWaves + wave] + lanes_below(sel_mask);
     if (sel && pos < (uint32_t)p.k) {
-      const int i = slice * kCoopSlice + j * kTopkThreads + tid;
-      int32_t payload;
-      if (p.in_idx)
-        payload = p.in_idx[(int64_t)row * p.in_idx_stride + i];
-      else if (p.page_table)
-        payload = slot_of(p, i);
-      else
-        payload = i;
-      out_idx[pos] = payload;
-      if (out_val) out_val[pos] = vals[i];
+      out_idx[pos] = payload[j];
+      if (out_val) out_val[pos] = val[j];
     }
   }
 }
