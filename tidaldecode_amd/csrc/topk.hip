@@ -638,13 +638,9 @@ __global__ __launch_bounds__(kTopkThreads) void topk_coop_select_kernel(const To
   __syncthreads();
   if (sh[2] != (uint32_t)(n_slices - 1)) return;
 
-  // ---- last workgroup of the row: leave the scratch clean, then finish ---------------------------
-  for (int i = tid; i < 2048; i += kTopkThreads) store_agent(rs + i, 0u);
-  if (tid == 0) {
-    store_agent(rs + 2048, 0u);
-    store_agent(rs + kCoopCandCount, 0u);
-    n_cand_sh = 0;
-  }
+  // ---- last workgroup of the row: finish (the scratch is cleaned at the very end: a store issued
+  // here would sit in front of the candidate loads in the in-order memory queue) -----------------
+  if (tid == 0) n_cand_sh = 0;
   int shift = 21;
   if (!crowded) {
     // the row's candidates, from every slice
@@ -787,7 +783,11 @@ __global__ __launch_bounds__(kTopkThreads) void topk_coop_select_kernel(const To
       out_run += slice_gt[sl] + (e < room ? e : room);
       eq_run += e;
     }
+    store_agent(rs + 2048, 0u);
+    store_agent(rs + kCoopCandCount, 0u);
   }
+  // leave the histogram zero for the next call
+  for (int i = tid; i < 2048; i += kTopkThreads) store_agent(rs + i, 0u);
 }
 
 template <typename T>
