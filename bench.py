@@ -259,6 +259,16 @@ def cpu_baseline(args, budget_s=20.0):
         ga_t.append(time.perf_counter() - t)
         if time.perf_counter() - t0 > budget_s / 4 or len(ga_t) >= 30:
             break
+    # the CPU-runnable configuration exactly as written: 4096 tokens, 256 selected by the summed
+    # softmax scores of all heads, one selection layer then one sparse layer with fresh inputs
+    c0 = []
+    q0, k0, v0 = (torch.randn(s_, generator=g) for s_ in ((h, d), (4096, h, d), (4096, h, d)))
+    q1, k1, v1 = (torch.randn(s_, generator=g) for s_ in ((h, d), (4096, h, d), (4096, h, d)))
+    for _ in range(10):
+        t = time.perf_counter()
+        _, idx0, _ = orc.select_layer(q0, k0, v0, 256, "head_sum")
+        orc.sparse_layer(q1, k1, v1, orc.mask_from_indices(idx0, h, 4096))
+        c0.append(time.perf_counter() - t)
     return {
         "value": round(statistics.median(sp_t) * 1e6, 1),
         "unit": "us/layer",
@@ -268,6 +278,7 @@ def cpu_baseline(args, budget_s=20.0):
                   f"32 heads x 128, fp32, torch-CPU; median; selection layer "
                   f"{statistics.median(sel_t) * 1e6:.0f} us",
         "selection_us_per_layer": round(statistics.median(sel_t) * 1e6, 1),
+        "configs0_selection_plus_sparse_us": round(statistics.median(c0) * 1e6, 1),
         "gather_variant_us_per_layer": round(statistics.median(ga_t) * 1e6, 1),
         "gather_variant_note": "index_select of the selected rows, then attention over them: not "
                                "the reference's path, shown for scale",
