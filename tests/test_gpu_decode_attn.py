@@ -373,3 +373,35 @@ def test_random_configurations(cuda, seed):
     assert (scores[:, :n].cpu() - logits).abs().max() <= 2e-4 * max(1.0, logits.abs().max().item())
     assert torch.isnan(scores[:, n:]).all()
     assert (lse[0].cpu() - torch.logsumexp(logits, -1)).abs().max() <= 1e-3
+
+
+@pytest.mark.parametrize("hq,hkv,d", [(4, 4, 128), (8, 2, 128), (4, 2, 128), (8, 1, 128), (2, 2, 64),
+                                      (2, 2, 256)])
+def test_logits_of_long_wave_runs(cuda, hq, hkv, d):
+    """One split for the whole sequence: every wave walks hundreds of tiles, so the logits leave
+    the per-wave staging strip several times in mid-loop (and once more, partly filled, at the
+    end).  All of them must land at their token, nothing past the sequence."""
+    from oracle import tidal_oracle as orc
+
+    dtype, page_size, n = torch.float16, 16, 20011
+    case = PagedCase(n, hkv, d, page_size, dtype, seed=hq + d)
+    q = randn((hq, d), 5, dtype)
+    logits = orc.attn_logits(q, case.k)
+    want = orc.softmax_pv(logits, case.v)
+    knob_sets = [dict(chunk_tokens=1 << 20)]
+    if hq == hkv:  # sixteen-wave workgroups exist for one query head per row
+        knob_sets.append(dict(chunk_tokens=1 << 20, waves_per_block=16))
+    for knobs in knob_sets:
+        w = _wrapper(0, hq, hkv, d, page_size, dtype, **knobs)
+        qd = q.to(dtype).to(cuda).unsqueeze(0)
+        od = torch.empty_like(qd)
+        stride = case.n_pages * page_size
+        scores = torch.full((hq, stride), float("nan"), dtype=torch.float32, device=cuda)
+        lse = torch.empty((1, hq), dtype=torch.float32, device=cuda)
+        table = case.page_table[:-1].to(torch.int32).unsqueeze(0)
+        w.forward(qd, od, case.pool.to(cuda), table.to(cuda), None, case.last_page_len,
+                  int(case.page_table[-1]), scores, lse=lse)
+        torch.cuda.synchronize()
+        assert tolerance_report(od[0], want) <= ATOL[dtype], knobs
+        assert (scores[:, :n].cpu() - logits).abs().max() <= 2e-4 * max(1.0, logits.abs().max().item())
+        assert torch.isnan(scores[:, n:]).all()
