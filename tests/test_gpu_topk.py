@@ -61,7 +61,7 @@ def _check(values, k, cuda):
 @pytest.mark.parametrize("rows,n,k", [(32, 4096, 256), (32, 32768, 2048), (1, 32768, 2048),
                                       (8, 102400, 4096), (32, 8192, 64), (3, 1000, 999),
                                       (5, 70, 70), (2, 1, 1), (4, 63, 1), (4, 65, 64),
-                                      (2, 1025, 512), (1, 131072, 4096)])
+                                      (2, 1025, 512), (1, 131072, 4096), (2, 262144, 5000), (64, 20000, 300)])
 def test_random_scores_fp32(cuda, rows, n, k):
     g = torch.Generator().manual_seed(rows * 1000003 + n + k)
     _check(torch.randn((rows, n), generator=g), k, cuda)
@@ -105,6 +105,24 @@ def test_long_rows_with_crowded_threshold_bins(cuda, dtype):
     _check(v.to(dtype), 20000, cuda)
     _check(v.to(dtype), 1, cuda)
     _check(v.to(dtype), n, cuda)
+
+
+def test_sorted_and_blocky_long_rows(cuda):
+    """Rows whose threshold bin sits in one slice only (sorted input), in the last partial slice, or
+    alternates between slices: the per-slice candidate lists and offsets of the several-workgroups
+    path must still add up."""
+    g = torch.Generator().manual_seed(21)
+    n = 100000 + 13
+    base = torch.randn((1, n), generator=g)
+    asc = torch.sort(base, dim=1).values
+    desc = torch.flip(asc, dims=[1])
+    blocky = base.clone()
+    blocky[:, 8192:16384] += 10.0          # one slice holds everything above the threshold
+    tail = base.clone()
+    tail[:, -100:] += 20.0                 # the winners start in the last, partial slice
+    v = torch.cat([asc, desc, blocky, tail])
+    for k in (1, 100, 4096, 8192, 50000):
+        _check(v, k, cuda)
 
 
 def test_payloads_on_long_rows(cuda):
