@@ -208,6 +208,45 @@ def test_batch_ragged_slots(cuda):
         assert tolerance_report(od[b], wants[b]) <= ATOL[dtype], b
 
 
+@pytest.mark.parametrize("hq,hkv,page_size,dtype", [(8, 2, 16, torch.float16), (4, 4, 16, torch.bfloat16),
+                                                    (8, 8, 5, torch.float16), (16, 2, 8, torch.bfloat16)])
+def test_batch_ragged_page_lists_with_logits(cuda, hq, hkv, page_size, dtype):
+    """Selection-layer mode for a batch: every sequence's page table in order through indptr, its
+    own last page and last-page length, logits and log-sum-exp per sequence and head."""
+    from oracle import tidal_oracle as orc
+
+    d = 128
+    lens = [37, 1000, page_size, 333, 1]
+    b = len(lens)
+    cases = [PagedCase(n, hkv, d, page_size, dtype, seed=60 + i, spare=2) for i, n in enumerate(lens)]
+    offs = np.cumsum([0] + [c.max_pages for c in cases])
+    pool = torch.cat([c.pool for c in cases]).to(cuda)
+    q = randn((b, hq, d), 5, dtype)
+    idx = torch.cat([c.page_table[:-1] + int(offs[i]) for i, c in enumerate(cases)]).to(torch.int32)[None]
+    counts = [c.n_pages - 1 for c in cases]
+    indptr = torch.tensor([0] + list(np.cumsum(counts)), dtype=torch.int32, device=cuda)
+    ll = torch.tensor([c.last_page_len for c in cases], dtype=torch.int32, device=cuda)
+    li = torch.tensor([int(c.page_table[-1]) + int(offs[i]) for i, c in enumerate(cases)],
+                      dtype=torch.int32, device=cuda)
+    stride = max(c.n_pages for c in cases) * page_size + 3
+    scores = torch.full((b * hq, stride), float("nan"), dtype=torch.float32, device=cuda)
+    lse = torch.empty((b, hq), dtype=torch.float32, device=cuda)
+    w = _wrapper(0, hq, hkv, d, page_size, dtype)
+    qd = q.to(dtype).to(cuda)
+    od = torch.empty_like(qd)
+    w.forward(qd, od, pool, idx.to(cuda).contiguous(), indptr, ll, li, scores, lse=lse,
+              n_list=max(counts))
+    torch.cuda.synchronize()
+    for i, c in enumerate(cases):
+        logits = orc.attn_logits(q[i], c.k)
+        want = orc.softmax_pv(logits, c.v)
+        assert tolerance_report(od[i], want) <= ATOL[dtype], i
+        got = scores[i * hq: (i + 1) * hq].cpu()
+        assert (got[:, : c.n] - logits).abs().max() <= 2e-4 * max(1.0, logits.abs().max().item()), i
+        assert torch.isnan(got[:, c.n:]).all(), i
+        assert (lse[i].cpu() - torch.logsumexp(logits, -1)).abs().max() <= 1e-3, i
+
+
 @pytest.mark.parametrize("knobs", [dict(waves_per_block=8, fused_merge=1),
                                    dict(waves_per_block=16, fused_merge=1),
                                    dict(waves_per_block=8, fused_merge=0),
