@@ -70,7 +70,9 @@ typedef struct {
  *
  * idx is a 2-D int32 array with `idx_rows` rows of `idx_row_stride` elements.  Sequence b uses
  * columns [indptr[b], indptr[b+1]) of every row (indptr lives on the device; if indptr is NULL
- * the call is for one sequence that uses columns [0, n_list_host)).  Row r belongs to query
+ * the call is for one sequence that uses columns [0, n_list_host)).  With count_arr (device,
+ * [batch]) sequence b uses count_arr[b] columns starting at indptr[b] instead: the rows of a
+ * padded table, one fixed-width segment per sequence, which can grow in place.  Row r belongs to query
  * head r (idx_rows == num_qo_heads), to KV head r (idx_rows == num_kv_heads) or to everybody
  * (idx_rows == 1).
  *
@@ -90,6 +92,7 @@ typedef struct {
   const int32_t* last_page_idx_arr; /* device [batch] or NULL */
   int32_t last_page_len;
   int32_t last_page_idx;
+  const int32_t* count_arr; /* device [batch] or NULL; needs indptr */
 } td_index_list;
 
 /*

@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     raw = ctypes.CDLL(_lib.LIB_PATH)
     for n in names:
         assert hasattr(raw, n), n
-    assert _lib.lib.td_version() == 1
+    assert _lib.lib.td_version() == 2
     assert isinstance(_lib.last_error(), str)
 
 
@@ -184,3 +184,39 @@ def test_controller_budget_arithmetic(scope):
         InferenceController(2, 8, 64, 16, 100, 1000, torch.float16, dev, select_mode="nope")
     with pytest.raises(ValueError):
         InferenceController(2, 8, 64, 16, 100, 1000, torch.float16, dev, num_kv_heads=3)
+
+
+def test_batch_controller_bookkeeping():
+    """Page-table segments, per-step metadata and page accounting of the batched controller
+    (host arithmetic only: no kernel runs)."""
+    from tidaldecode_amd.utils import BatchInferenceController
+
+    dev = torch.device("cpu")
+    c = BatchInferenceController(2, 8, 64, 4, 16, 40, 3, torch.float16, dev, num_kv_heads=2,
+                                 select_mode="group_sum", page_order_seed=1)
+    assert c.pages_per_seq == 10 and c.pool.capacity == 30 and c.index_rows == 2
+    assert c.topk_dindices_buffer.shape == (2, 3 * 16) and c.qk_product.shape == (24, 40)
+    c.add_sequences([5, 9])
+    assert c.batch == 2 and c.pool.num_free_blocks == 30 - 2 - 3
+    assert c.page_table[0, :2].tolist() == c._pages[0] and c.page_table[1, :3].tolist() == c._pages[1]
+    assert len(set(c._pages[0] + c._pages[1])) == 5
+    for _ in range(4):                       # 5 -> 9 tokens (third page), 9 -> 13 (fourth page)
+        c.begin_step()
+    assert c.seq_lens == [9, 13] and [len(p) for p in c._pages] == [3, 4]
+    meta = c._meta[:, :2].tolist()
+    assert meta[0] == [2, 3]                                 # pages before the last one
+    assert meta[1] == [1, 1]                                 # fill of the last page
+    assert meta[2] == [c._pages[0][-1], c._pages[1][-1]]     # last page id
+    assert meta[3] == [c._pages[0][-1] * 4, c._pages[1][-1] * 4]   # slot of the new token
+    assert meta[4] == [8, 12] and meta[5] == [9, 13]         # position, selected = min(budget, n)
+    assert c.positions.tolist() == [8, 12] and c.selected.tolist() == [9, 13]
+    for _ in range(10):
+        c.begin_step()
+    assert c.selected.tolist() == [16, 16]                   # the budget caps the lists
+    with pytest.raises(RuntimeError, match="max_batch"):
+        c.add_sequences([4, 4])
+    with pytest.raises(RuntimeError, match="max_seq_len"):   # a failed call keeps nothing
+        c.add_sequences([41])
+    assert c.batch == 2 and c.pool.num_free_blocks == 30 - 5 - 6
+    c.release()
+    assert c.batch == 0 and c.pool.num_free_blocks == 30

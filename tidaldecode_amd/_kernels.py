@@ -426,12 +426,14 @@ class BatchDecodeWithPagedKVCachePyTorchWrapper:
                 qk_product: Optional[torch.Tensor], rope_scale: float = 1.0,
                 rope_theta: float = 1e4, *, index_kind: str = "pages",
                 lse: Optional[torch.Tensor] = None, n_list: Optional[int] = None,
-                fresh=None) -> None:
+                fresh=None, counts: Optional[torch.Tensor] = None) -> None:
         """q, o ``[B, H_q, D]``; ``paged_kv_indices`` ``[rows, budget]`` int32 with rows in
         {H_q, H_kv, 1}; sequence b uses columns ``indptr[b]:indptr[b+1]`` of every row and then
         the first ``last_page_len`` entries of page ``last_page_idx`` (ints, or int32 device
         tensors ``[B]``).  ``index_kind="slots"`` reads the entries as token slots.
         ``n_list`` bounds the per-sequence column count (default: all columns).
+        ``counts`` (int32 device ``[B]``): sequence b uses ``counts[b]`` columns from
+        ``indptr[b]`` on — segments of a padded table instead of a packed one.
         rope_scale / rope_theta are accepted for signature parity; RoPE is applied before the
         cache is written (RotaryMode::kNone in the reference, approx_attn.cu:52,139).
         ``fresh=(k, v, cos, sin, dst_slot)`` fuses the decode step: q, k ``[B, H, D]`` are then
@@ -473,6 +475,11 @@ class BatchDecodeWithPagedKVCachePyTorchWrapper:
             if paged_kv_indptr.numel() != batch + 1:
                 raise RuntimeError("paged_kv_indptr must hold batch + 1 entries")
             lst.indptr = paged_kv_indptr.data_ptr()
+        if counts is not None:
+            _check_i32(counts, "counts")
+            if paged_kv_indptr is None or counts.numel() != batch:
+                raise RuntimeError("counts needs paged_kv_indptr and one entry per sequence")
+            lst.count_arr = counts.data_ptr()
         lst.n_list_host = budget if n_list is None else min(int(n_list), budget)
         max_last = 0
         if isinstance(paged_kv_last_page_len, torch.Tensor):

@@ -46,6 +46,7 @@ class IndexList(Structure):
         ("last_page_idx_arr", c_void_p),
         ("last_page_len", c_int32),
         ("last_page_idx", c_int32),
+        ("count_arr", c_void_p),
     ]
 
 

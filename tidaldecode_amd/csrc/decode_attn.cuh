@@ -49,6 +49,7 @@ struct DecodeParams {
   int32_t idx_row_stride;  // 0 for a shared row
   int32_t idx_per_kv;      // 1: rows are per KV head while QPG == 1
   const int32_t* indptr;
+  const int32_t* count_arr;  // per-sequence entry counts of a padded table (else indptr differences)
   int32_t n_list_host;
   const int32_t* last_len_arr;
   const int32_t* last_idx_arr;
@@ -198,7 +199,7 @@ __device__ __forceinline__ int seq_items(const DecodeParams& p, int b, SeqList& 
   list_beg = 0;
   if (p.indptr) {
     list_beg = p.indptr[b];
-    s.n_list = p.indptr[b + 1] - list_beg;
+    s.n_list = p.count_arr ? p.count_arr[b] : p.indptr[b + 1] - list_beg;
   } else {
     s.n_list = p.n_list_host;
   }

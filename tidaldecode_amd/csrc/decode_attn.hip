@@ -127,6 +127,8 @@ static int build_params(const td_paged_kv* kv, const td_index_list* list, const 
   TD_REQUIRE(list->kind == TD_IDX_PAGES || list->kind == TD_IDX_SLOTS, "td_decode_attn: kind %d",
              list->kind);
   TD_REQUIRE(list->n_list_host >= 0, "td_decode_attn: n_list_host %d", list->n_list_host);
+  TD_REQUIRE(list->count_arr == nullptr || list->indptr != nullptr,
+             "td_decode_attn: count_arr needs indptr (the first column of every sequence)");
   TD_REQUIRE(list->idx != nullptr || list->n_list_host == 0,
              "td_decode_attn: idx is NULL but n_list_host is %d", list->n_list_host);
   TD_REQUIRE(list->idx_rows == 1 || list->idx_row_stride >= list->n_list_host,
@@ -222,6 +224,7 @@ static int build_params(const td_paged_kv* kv, const td_index_list* list, const 
   p.page_mode = list->kind == TD_IDX_PAGES ? 1 : 0;
   p.max_page = (uint32_t)(kv->max_pages - 1);
   p.indptr = list->indptr;
+  p.count_arr = list->count_arr;
   p.n_list_host = list->n_list_host;
   p.last_len_arr = list->last_page_len_arr;
   p.last_idx_arr = list->last_page_idx_arr;

@@ -10,6 +10,7 @@ from typing import Optional
 import torch
 
 from .. import _kernels
+from .batch_controller import BatchInferenceController
 from .controller import InferenceController
 from .paged import BatchDecodeWithPagedKVCacheWrapper, KvCache, KvPool, TensorLayout
 
@@ -18,6 +19,7 @@ __all__ = [
     "KvCache",
     "KvPool",
     "InferenceController",
+    "BatchInferenceController",
     "BatchDecodeWithPagedKVCacheWrapper",
     "append_kv",
     "prefill_forward",

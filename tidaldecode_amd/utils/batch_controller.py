@@ -1,0 +1,260 @@
+"""Bookkeeping of several sequences that decode in lock step over one shared page pool.
+
+The reference's controller serves one sequence (tidal/utils/controller.py:8-193, its kv cache
+asserts a single page table, tidal/utils/kv_cache.py:70-137); its kernels already take a batch
+(``indptr``, kernels/include/decode/decode_attn.cuh:432-470).  This class is the batched
+counterpart of ``InferenceController`` for that kernel surface:
+
+* one pool per layer shared by all sequences, one fixed-width page-table segment per sequence in a
+  device tensor ``[max_batch, pages_per_seq]`` that grows in place;
+* the per-sequence metadata of a decode step (pages before the last one, fill of the last page,
+  its id, the slot and the position of the new token, the number of selected tokens) is one
+  ``[6, max_batch]`` int32 device tensor refreshed by a single small copy per step — never the
+  page tables themselves;
+* selection state for the whole batch: logits ``[B * H_q, max tokens]`` (``-inf`` where a sequence
+  has no token, so that one top-k call serves ragged lengths), the log-sum-exp per head and the
+  persisted token lists ``[rows, B * budget]`` with one fixed-width segment per sequence.
+
+Every attention call is ONE launch for the whole batch.  The per-step copy makes this controller
+an eager-mode one (a captured graph would replay one step's metadata); token lists are valid for
+the decode step they were selected in.
+"""
+from typing import List, Optional, Sequence
+
+import torch
+
+from .. import _kernels
+from .paged import BatchDecodeWithPagedKVCacheWrapper, KvPool, TensorLayout
+
+_SELECT_MODES = ("per_head", "group_sum", "head_sum")
+# rows of the per-step metadata tensor
+_PAGES_BEFORE_LAST, _LAST_LEN, _LAST_IDX, _DST_SLOT, _POSITION, _SELECTED = range(6)
+
+
+class BatchInferenceController:
+    def __init__(self, num_layers: int, num_heads: int, head_dim: int, page_size: int,
+                 token_budget: int, max_seq_len: int, max_batch: int, dtype, device, *,
+                 num_kv_heads: Optional[int] = None, select_mode: str = "per_head",
+                 kv_layout: str = "NHD", page_order_seed=None):
+        if select_mode not in _SELECT_MODES:
+            raise KeyError(f"Invalid select_mode {select_mode}")
+        num_kv_heads = num_heads if num_kv_heads is None else num_kv_heads
+        if num_heads % num_kv_heads != 0:
+            raise ValueError("num_heads must be a multiple of num_kv_heads")
+        if max_batch < 1 or max_seq_len < 1:
+            raise ValueError("max_batch and max_seq_len must be positive")
+        self.layout = TensorLayout.parse(kv_layout)
+        self.device, self.dtype = device, dtype
+        self.num_heads, self.num_kv_heads, self.head_dim = num_heads, num_kv_heads, head_dim
+        self.page_size, self.max_seq_len, self.max_batch = page_size, max_seq_len, max_batch
+        self.select_mode = select_mode
+        self.pages_per_seq = -(-max_seq_len // page_size)
+        self.pool = KvPool(num_layers, num_kv_heads, head_dim, max_batch * self.pages_per_seq,
+                           page_size, dtype, device, self.layout, page_order_seed)
+
+        i32 = dict(dtype=torch.int32, device=device)
+        self.page_table = torch.zeros((max_batch, self.pages_per_seq), **i32)
+        self._pages: List[List[int]] = []
+        self.seq_lens: List[int] = []
+        self._meta = torch.zeros((6, max_batch), **i32)
+        # staging for the per-step copy: a small ring of pinned rows, so that the copy is
+        # asynchronous and a buffer is only rewritten after its copy has completed
+        self._on_gpu = torch.device(device).type == "cuda"
+        self._stage = [torch.zeros((6, max_batch), dtype=torch.int32, pin_memory=self._on_gpu)
+                       for _ in range(4)]
+        self._stage_done = [None] * len(self._stage)
+        self._stage_next = 0
+        self._table_starts = torch.arange(max_batch + 1, **i32) * self.pages_per_seq
+
+        self.score_cols = self.pages_per_seq * page_size
+        self.budget = min(int(token_budget), self.score_cols)
+        self.index_rows = {"per_head": num_heads, "group_sum": num_kv_heads, "head_sum": 1}[select_mode]
+        self.qk_product = torch.full((max_batch * num_heads, self.score_cols), float("-inf"),
+                                     dtype=torch.float32, device=device)
+        self.lse = torch.zeros((max_batch, num_heads), dtype=torch.float32, device=device)
+        self.score_sum = None
+        if select_mode != "per_head":
+            self.score_sum = torch.zeros((max_batch * self.index_rows, self.score_cols),
+                                         dtype=torch.float32, device=device)
+        # lists: row r of sequence b lives in columns [b * budget, b * budget + selected[b])
+        self.topk_dindices_buffer = torch.zeros((self.index_rows, max_batch * self.budget), **i32)
+        self._positions = torch.zeros((max_batch * self.index_rows, self.budget), **i32)
+        self._list_starts = torch.arange(max_batch + 1, **i32) * self.budget
+        self.topk_buf = torch.zeros(_kernels.topk_workspace_bytes(max_batch * self.index_rows),
+                                    dtype=torch.uint8, device=device)
+        self._handle = BatchDecodeWithPagedKVCacheWrapper(kv_layout=kv_layout)
+        self._handle.begin_forward(None, num_heads, num_kv_heads, head_dim, page_size, dtype)
+        layer_bytes = self.pool.buf[0].numel() * self.pool.buf.element_size()
+        self.fused_step_ok = (page_size & (page_size - 1)) == 0 and layer_bytes < (1 << 32)
+
+    # ---- sequences ----------------------------------------------------------------------------
+    @property
+    def batch(self) -> int:
+        return len(self.seq_lens)
+
+    def buf_layer(self, layer_idx: int) -> torch.Tensor:
+        return self.pool.buf[layer_idx % self.pool.num_layers]
+
+    def _reserve(self, b: int, n_tokens: int) -> None:
+        have = len(self._pages[b])
+        total = self.seq_lens[b] + n_tokens
+        if total > self.max_seq_len:
+            raise RuntimeError(f"sequence {b} would hold {total} tokens, max_seq_len is {self.max_seq_len}")
+        grow = -(-total // self.page_size) - have
+        if grow > 0:
+            fresh = self.pool.take(grow)
+            self.page_table[b, have: have + grow] = torch.tensor(fresh, dtype=torch.int32)
+            self._pages[b] += fresh
+        self.seq_lens[b] = total
+
+    def add_sequences(self, lengths: Sequence[int]) -> None:
+        """Open one sequence per entry with room for that many prompt tokens."""
+        if self.batch + len(lengths) > self.max_batch:
+            raise RuntimeError(f"{self.batch + len(lengths)} sequences, max_batch is {self.max_batch}")
+        if any(n < 1 for n in lengths):
+            raise ValueError("a sequence starts with at least one token")
+        opened = self.batch
+        try:
+            for n in lengths:
+                self._pages.append([])
+                self.seq_lens.append(0)
+                self._reserve(self.batch - 1, int(n))
+        except Exception:
+            for pages in self._pages[opened:]:   # leave the controller as it was
+                self.pool.give_back(pages)
+            del self._pages[opened:], self.seq_lens[opened:]
+            raise
+        self._refresh()
+
+    def release(self) -> None:
+        """Close every sequence and return its pages."""
+        for pages in self._pages:
+            self.pool.give_back(pages)
+        self._pages, self.seq_lens = [], []
+        self.qk_product.fill_(float("-inf"))
+
+    def _refresh(self) -> None:
+        """Per-sequence metadata of the current lengths: one host row set, one copy."""
+        P = self.page_size
+        cols = []
+        for b, n in enumerate(self.seq_lens):
+            pages = self._pages[b]
+            last_len = (n - 1) % P + 1
+            cols.append((len(pages) - 1, last_len, pages[-1], pages[-1] * P + last_len - 1, n - 1,
+                         min(self.budget, n)))
+        cols += [(0,) * 6] * (self.max_batch - len(cols))
+        i = self._stage_next
+        self._stage_next = (i + 1) % len(self._stage)
+        if self._stage_done[i] is not None:
+            self._stage_done[i].synchronize()
+        m = self._stage[i]
+        m.copy_(torch.tensor(cols, dtype=torch.int32).t())
+        self._meta.copy_(m, non_blocking=True)
+        if self._on_gpu:
+            self._stage_done[i] = torch.cuda.Event()
+            self._stage_done[i].record()
+
+    def begin_step(self) -> None:
+        """Make room for one new token in every sequence (call once per decode step)."""
+        full = [b for b, n in enumerate(self.seq_lens) if n + 1 > self.max_seq_len]
+        if full:
+            raise RuntimeError(f"sequences {full} already hold max_seq_len = {self.max_seq_len} tokens")
+        for b in range(self.batch):
+            self._reserve(b, 1)
+        self._refresh()
+
+    # views of the step's metadata, all int32 device [B]
+    def _row(self, r: int) -> torch.Tensor:
+        return self._meta[r, : self.batch]
+
+    @property
+    def positions(self) -> torch.Tensor:
+        return self._row(_POSITION)
+
+    @property
+    def dst_slots(self) -> torch.Tensor:
+        return self._row(_DST_SLOT)
+
+    @property
+    def selected(self) -> torch.Tensor:
+        return self._row(_SELECTED)
+
+    def rope_table(self, rope_scale: float = 1.0, rope_theta: float = 1e4):
+        """cos, sin ``[B, D/2]`` of the new tokens' positions (once per step, all layers)."""
+        return _kernels.rope_table(self.positions, self.head_dim, rope_scale, rope_theta)
+
+    # ---- cache writes -------------------------------------------------------------------------
+    def append_prompt(self, b: int, k: torch.Tensor, v: torch.Tensor, layer_idx: int) -> None:
+        """Write the (already rotated) prompt K/V ``[n, H_kv, D]`` of sequence b: its first n tokens."""
+        n, P = k.size(0), self.page_size
+        n_pages = -(-n // P)
+        indptr = torch.tensor([0, n_pages], dtype=torch.int32, device=self.device)
+        fn = _kernels.append_kv_cache_prefill if n > 1 else _kernels.append_kv_cache_decode
+        fn(k, v, self.buf_layer(layer_idx), self.page_table[b, :n_pages], indptr, (n - 1) % P + 1,
+           self._pages[b][n_pages - 1], None, None, None, 0, 0, int(self.layout))
+
+    def rope_append(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, layer_idx: int,
+                    rope_scale: float = 1.0, rope_theta: float = 1e4) -> None:
+        """Rotate q ``[B, H_q, D]`` in place and store the rotated k and v ``[B, H_kv, D]`` of the
+        step's new tokens (the un-fused form of ``fresh=``)."""
+        _kernels.rope_append_decode(q, k, v, self.buf_layer(layer_idx), self.positions,
+                                    self.dst_slots, int(self.layout), rope_scale, rope_theta)
+
+    # ---- attention ----------------------------------------------------------------------------
+    def _fresh(self, fresh):
+        if fresh is None:
+            return None
+        k, v, cos, sin = fresh
+        return (k, v, cos, sin, self.dst_slots)
+
+    def attend_full(self, q: torch.Tensor, layer_idx: int, output_qk_product: bool = False,
+                    fresh=None) -> torch.Tensor:
+        """Attention of every sequence's new token over its whole cache; with
+        ``output_qk_product`` the logits and log-sum-exps are kept for ``select``.
+        ``fresh=(k, v, cos, sin)`` folds RoPE and the append of the new tokens into the launch."""
+        B = self.batch
+        o = torch.empty_like(q)
+        self._handle.forward(
+            q, o, self.buf_layer(layer_idx), self.page_table.view(1, -1),
+            self._table_starts[: B + 1], self._row(_LAST_LEN), self._row(_LAST_IDX),
+            self.qk_product[: B * self.num_heads] if output_qk_product else None,
+            lse=self.lse[:B] if output_qk_product else None,
+            n_list=max(len(p) for p in self._pages) - 1, counts=self._row(_PAGES_BEFORE_LAST),
+            fresh=self._fresh(fresh))
+        return o
+
+    def select(self) -> None:
+        """Top-k of the last ``attend_full(..., output_qk_product=True)`` for every sequence:
+        physical token slots, sorted by position, in its segment of ``topk_dindices_buffer``."""
+        B, P, k = self.batch, self.page_size, self.budget
+        n = max(self.seq_lens)
+        rows = self.index_rows
+        scores = self.qk_product[: B * self.num_heads]
+        if self.select_mode != "per_head":
+            # rows of a sequence are reduced together: one call per sequence keeps its own lse
+            for b in range(B):
+                _kernels.score_reduce(scores[b * self.num_heads: (b + 1) * self.num_heads],
+                                      self.lse[b], self.num_kv_heads, n, self.select_mode,
+                                      out=self.score_sum[b * rows: (b + 1) * rows])
+            scores = self.score_sum[: B * rows]
+        k_eff = min(k, n)
+        pos = self._positions[: B * rows, :k_eff]
+        _kernels.topk_filtering(scores[:, :n], None, None, pos, self.topk_buf, k_eff)
+        # positions -> physical slots through each sequence's page table; entries past a
+        # sequence's own count are never read (positions come out sorted, the valid ones first)
+        pos = pos.view(B, rows, k_eff).long()
+        page = (pos // P).clamp_(max=self.pages_per_seq - 1)
+        table = self.page_table[:B].long().unsqueeze(1).expand(B, rows, self.pages_per_seq)
+        slots = table.gather(2, page) * P + pos % P
+        self.topk_dindices_buffer.view(rows, self.max_batch, k)[:, :B, :k_eff] = \
+            slots.permute(1, 0, 2).to(torch.int32)
+
+    def attend_sparse(self, q: torch.Tensor, layer_idx: int, fresh=None) -> torch.Tensor:
+        """Attention over the persisted token lists (``fresh`` as in ``attend_full``)."""
+        B = self.batch
+        o = torch.empty_like(q)
+        self._handle.forward(q, o, self.buf_layer(layer_idx), self.topk_dindices_buffer,
+                             self._list_starts[: B + 1], 0, 0, None, index_kind="slots",
+                             n_list=min(self.budget, max(self.seq_lens)), counts=self.selected,
+                             fresh=self._fresh(fresh))
+        return o
