@@ -240,7 +240,9 @@ int td_score_reduce(const float* logits, int64_t logits_stride, const float* lse
  * row, sorted by ascending position: out_values[r, j] (same dtype as values, may be NULL) and
  * out_idx[r, j] = payload of the selected position p:
  *     in_idx != NULL              -> in_idx[r * in_idx_stride + p]   (reference meaning)
- *     page_table != NULL          -> page_table[p / page_size] * page_size + p % page_size
+ *     page_table != NULL          -> table[p / page_size] * page_size + p % page_size, where
+ *                                    table = page_table + (r / rows_per_table) * page_table_stride
+ *                                    (rows_per_table == 0: one table for all rows)
  *     both NULL                   -> p
  * k is clamped to len.  NaNs order above +inf.  out rows have stride out_stride.
  * workspace: see td_topk_workspace_bytes (optional).
@@ -249,8 +251,9 @@ int td_score_reduce(const float* logits, int64_t logits_stride, const float* lse
  */
 int td_topk(const void* values, int32_t values_dtype, int64_t values_stride, int32_t rows,
             int32_t len, int32_t k, const int32_t* in_idx, int64_t in_idx_stride,
-            const int32_t* page_table, int32_t page_size, void* out_values, int32_t* out_idx,
-            int64_t out_stride, void* workspace, int64_t workspace_bytes, void* stream);
+            const int32_t* page_table, int64_t page_table_stride, int32_t rows_per_table,
+            int32_t page_size, void* out_values, int32_t* out_idx, int64_t out_stride,
+            void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
  * Bytes of device scratch that lets td_topk spread a row over several workgroups (rows of more

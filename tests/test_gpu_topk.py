@@ -189,6 +189,31 @@ def test_payloads(cuda):
     assert torch.equal(got, torch.gather(payload, 1, orc.stable_topk(v[:, :500], k)))
 
 
+def test_page_table_per_row_group(cuda):
+    """A batch of sequences in one call: rows of group g read page table g.  Short rows (one
+    workgroup per row) and long rows (several workgroups per row) against the oracle."""
+    from oracle import tidal_oracle as orc
+
+    g = torch.Generator().manual_seed(17)
+    for groups, per, n, k, page in ((3, 4, 3000, 100, 16), (4, 8, 20000, 2048, 16), (2, 1, 9000, 50, 5)):
+        rows = groups * per
+        v = torch.randn((rows, n), generator=g)
+        n_pages = (n + page - 1) // page
+        tables = torch.stack([torch.randperm(n_pages + 7, generator=g)[:n_pages] for _ in range(groups)]).int()
+        want_pos = orc.stable_topk(v, k)
+        want = torch.stack([tables[r // per].long()[want_pos[r] // page] * page + want_pos[r] % page
+                            for r in range(rows)])
+        for scratch in (False, True):
+            got, _ = _gpu_topk(v, k, cuda, page_table=tables, page_size=page, want_vals=False,
+                               scratch=scratch)
+            assert torch.equal(got.long(), want), (groups, per, n, scratch)
+    from tidaldecode_amd import _kernels
+    out = torch.zeros((5, 10), dtype=torch.int32, device=cuda)
+    with pytest.raises(RuntimeError, match="tables"):
+        _kernels.topk_filtering(torch.zeros((5, 100), device=cuda), None, None, out, None, 10,
+                                page_table=torch.zeros((2, 100), dtype=torch.int32, device=cuda))
+
+
 def test_topk_errors(cuda):
     from tidaldecode_amd import _kernels
 

@@ -174,7 +174,8 @@ def topk_filtering(estimated_value: torch.Tensor, estimated_indices: Optional[to
     ``estimated_value.size(1)``, kernels/include/topk/decode_select_k.cuh:53-55).
 
     Extensions: ``estimated_indices=None`` returns positions, or physical token slots when a
-    ``page_table`` ``[n_pages]`` is given; fp32 values.
+    ``page_table`` ``[n_pages]`` is given (``[groups, n_pages]``: one table per ``H / groups``
+    consecutive rows, the sequences of a batch); fp32 values.
     """
     _check_rows(estimated_value, "estimated_value")
     rows, length = estimated_value.shape
@@ -201,11 +202,18 @@ def topk_filtering(estimated_value: torch.Tensor, estimated_indices: Optional[to
         out_vals = d_out.data_ptr()
     if k > length:
         raise RuntimeError(f"page_budget {k} exceeds the row length {length}")
-    pt_ptr = None
+    pt_ptr, pt_stride, rows_per_table = None, 0, 0
     if page_table is not None:
         _check_input(page_table, "page_table")
         _check_i32(page_table, "page_table")
-        if page_table.numel() * page_size < length:
+        if page_table.dim() == 2:   # one table per group of consecutive rows (a batch of sequences)
+            groups = page_table.size(0)
+            if groups < 1 or rows % groups != 0:
+                raise RuntimeError(f"page_table has {groups} tables for {rows} rows")
+            pt_stride, rows_per_table = page_table.stride(0), rows // groups
+        elif page_table.dim() != 1:
+            raise RuntimeError("page_table must be [n_pages] or [groups, n_pages]")
+        if page_table.size(-1) * page_size < length:
             raise RuntimeError("page_table does not cover the row")
         pt_ptr = page_table.data_ptr()
     ws_ptr, ws_bytes = None, 0
@@ -216,7 +224,7 @@ def topk_filtering(estimated_value: torch.Tensor, estimated_indices: Optional[to
     check(lib.td_topk(estimated_value.data_ptr(),
                       _dtype_code(estimated_value.dtype, "Top-k filtering"),
                       estimated_value.stride(0), rows, length, k, in_ptr, in_stride, pt_ptr,
-                      int(page_size), out_vals, indices_out.data_ptr(), indices_out.stride(0),
+                      pt_stride, rows_per_table, int(page_size), out_vals, indices_out.data_ptr(), indices_out.stride(0),
                       ws_ptr, ws_bytes if ws_ptr else 0, _stream()))
 
 

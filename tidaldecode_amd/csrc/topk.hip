@@ -28,6 +28,8 @@ struct TopkParams {
   const int32_t* in_idx;
   int64_t in_idx_stride;
   const int32_t* page_table;
+  int64_t page_table_stride;  // elements between the tables of consecutive row groups
+  int32_t rows_per_table;     // rows that share one table (all rows when there is one table)
   int32_t page_size;
   int32_t page_shift;  // log2(page_size) when it is a power of two, else -1
   void* out_values;
@@ -36,10 +38,14 @@ struct TopkParams {
 };
 
 // physical slot of position i through the page table
-__device__ __forceinline__ int32_t slot_of(const TopkParams& p, int i) {
+__device__ __forceinline__ const int32_t* table_of(const TopkParams& p, int row) {
+  if (p.page_table == nullptr || p.page_table_stride == 0) return p.page_table;
+  return p.page_table + (int64_t)(row / p.rows_per_table) * p.page_table_stride;
+}
+__device__ __forceinline__ int32_t slot_of(const TopkParams& p, const int32_t* table, int i) {
   if (p.page_shift >= 0)
-    return (p.page_table[i >> p.page_shift] << p.page_shift) | (i & (p.page_size - 1));
-  return p.page_table[i / p.page_size] * p.page_size + i % p.page_size;
+    return (table[i >> p.page_shift] << p.page_shift) | (i & (p.page_size - 1));
+  return table[i / p.page_size] * p.page_size + i % p.page_size;
 }
 
 struct F32 {};
@@ -106,6 +112,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_kernel(const TopkParams p) 
   typedef KeyTraits<T> KT;
   typedef typename KT::elem_t elem_t;
   const int row = blockIdx.x;
+  const int32_t* table = table_of(p, row);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -214,7 +221,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_kernel(const TopkParams p) 
       if (p.in_idx)
         payload = p.in_idx[(int64_t)row * p.in_idx_stride + i];
       else if (p.page_table)
-        payload = slot_of(p, i);
+        payload = slot_of(p, table, i);
       else
         payload = i;
       out_idx[pos] = payload;
@@ -264,6 +271,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_reg_kernel(const TopkParams
   typedef KeyTraits<T> KT;
   typedef typename KT::elem_t elem_t;
   const int row = blockIdx.x;
+  const int32_t* table = table_of(p, row);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -376,7 +384,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_reg_kernel(const TopkParams
       if (p.in_idx)
         payload = p.in_idx[(int64_t)row * p.in_idx_stride + i];
       else if (p.page_table)
-        payload = slot_of(p, i);
+        payload = slot_of(p, table, i);
       else
         payload = i;
       out_idx[pos] = payload;
@@ -820,6 +828,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_coop_emit_kernel(const Topk
   // Payloads and values of every element are fetched right away, unconditionally (they sit in
   // L2): together with the keys they are one round trip, and no load follows a store (vector
   // loads and stores complete in order on one counter).
+  const int32_t* table = table_of(p, row);
   int32_t payload[kCoopIPT];
   elem_t val[kCoopIPT];
 #pragma unroll
@@ -829,7 +838,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_coop_emit_kernel(const Topk
     if (p.in_idx)
       payload[j] = p.in_idx[(int64_t)row * p.in_idx_stride + i];
     else if (p.page_table)
-      payload[j] = slot_of(p, i);
+      payload[j] = slot_of(p, table, i);
     else
       payload[j] = i;
     if (out_val) val[j] = vals[i];
@@ -939,7 +948,8 @@ using namespace tidal;
 
 extern "C" int td_topk(const void* values, int32_t values_dtype, int64_t values_stride,
                        int32_t rows, int32_t len, int32_t k, const int32_t* in_idx,
-                       int64_t in_idx_stride, const int32_t* page_table, int32_t page_size,
+                       int64_t in_idx_stride, const int32_t* page_table,
+                       int64_t page_table_stride, int32_t rows_per_table, int32_t page_size,
                        void* out_values, int32_t* out_idx, int64_t out_stride, void* workspace,
                        int64_t workspace_bytes, void* stream) {
   TD_REQUIRE(values && out_idx, "td_topk: NULL values or out_idx");
@@ -951,6 +961,9 @@ extern "C" int td_topk(const void* values, int32_t values_dtype, int64_t values_
   TD_REQUIRE(out_stride >= k, "td_topk: out_stride %lld < k %d", (long long)out_stride, k);
   TD_REQUIRE(!in_idx || in_idx_stride >= 0, "td_topk: in_idx_stride %lld", (long long)in_idx_stride);
   TD_REQUIRE(!page_table || page_size >= 1, "td_topk: page_size %d", page_size);
+  TD_REQUIRE(!page_table || (rows_per_table >= 0 && page_table_stride >= 0),
+             "td_topk: rows_per_table %d / page_table_stride %lld", rows_per_table,
+             (long long)page_table_stride);
   if (k == 0) return TD_OK;
   TopkParams p;
   p.values = values;
@@ -960,6 +973,8 @@ extern "C" int td_topk(const void* values, int32_t values_dtype, int64_t values_
   p.in_idx = in_idx;
   p.in_idx_stride = in_idx_stride;
   p.page_table = in_idx ? nullptr : page_table;
+  p.page_table_stride = page_table_stride;
+  p.rows_per_table = rows_per_table >= 1 ? rows_per_table : rows;
   p.page_size = page_size;
   p.page_shift = -1;
   if (page_size >= 1 && (page_size & (page_size - 1)) == 0) p.page_shift = __builtin_ctz(page_size);

@@ -78,7 +78,7 @@ class BatchInferenceController:
                                          dtype=torch.float32, device=device)
         # lists: row r of sequence b lives in columns [b * budget, b * budget + selected[b])
         self.topk_dindices_buffer = torch.zeros((self.index_rows, max_batch * self.budget), **i32)
-        self._positions = torch.zeros((max_batch * self.index_rows, self.budget), **i32)
+        self._slots = torch.zeros((max_batch * self.index_rows, self.budget), **i32)
         self._list_starts = torch.arange(max_batch + 1, **i32) * self.budget
         self.topk_buf = torch.zeros(_kernels.topk_workspace_bytes(max_batch * self.index_rows),
                                     dtype=torch.uint8, device=device)
@@ -238,16 +238,14 @@ class BatchInferenceController:
                                       out=self.score_sum[b * rows: (b + 1) * rows])
             scores = self.score_sum[: B * rows]
         k_eff = min(k, n)
-        pos = self._positions[: B * rows, :k_eff]
-        _kernels.topk_filtering(scores[:, :n], None, None, pos, self.topk_buf, k_eff)
-        # positions -> physical slots through each sequence's page table; entries past a
-        # sequence's own count are never read (positions come out sorted, the valid ones first)
-        pos = pos.view(B, rows, k_eff).long()
-        page = (pos // P).clamp_(max=self.pages_per_seq - 1)
-        table = self.page_table[:B].long().unsqueeze(1).expand(B, rows, self.pages_per_seq)
-        slots = table.gather(2, page) * P + pos % P
+        # one call: row b * rows + r is row r of sequence b and goes through that sequence's page
+        # table; entries past a sequence's own count are never read (positions come out sorted,
+        # the valid ones first)
+        out = self._slots[: B * rows, :k_eff]
+        _kernels.topk_filtering(scores[:, :n], None, None, out, self.topk_buf, k_eff,
+                                page_table=self.page_table[:B], page_size=P)
         self.topk_dindices_buffer.view(rows, self.max_batch, k)[:, :B, :k_eff] = \
-            slots.permute(1, 0, 2).to(torch.int32)
+            out.view(B, rows, k_eff).permute(1, 0, 2)
 
     def attend_sparse(self, q: torch.Tensor, layer_idx: int, fresh=None) -> torch.Tensor:
         """Attention over the persisted token lists (``fresh`` as in ``attend_full``)."""
