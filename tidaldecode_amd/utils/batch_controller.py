@@ -231,11 +231,9 @@ class BatchInferenceController:
         rows = self.index_rows
         scores = self.qk_product[: B * self.num_heads]
         if self.select_mode != "per_head":
-            # rows of a sequence are reduced together: one call per sequence keeps its own lse
-            for b in range(B):
-                _kernels.score_reduce(scores[b * self.num_heads: (b + 1) * self.num_heads],
-                                      self.lse[b], self.num_kv_heads, n, self.select_mode,
-                                      out=self.score_sum[b * rows: (b + 1) * rows])
+            # the B * H_q logit rows form B * rows groups of consecutive heads: one grouped sum
+            _kernels.score_reduce(scores, self.lse[:B].view(-1), B * rows, n, "group_sum",
+                                  out=self.score_sum[: B * rows])
             scores = self.score_sum[: B * rows]
         k_eff = min(k, n)
         # one call: row b * rows + r is row r of sequence b and goes through that sequence's page
