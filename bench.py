@@ -470,10 +470,46 @@ def batch8_leg(args):
     algo = nb * k * h * d * 2 * 2 + nb * k * h * 4 + 2 * nb * h * d * 2
     del pools
     torch.cuda.empty_cache()
-    return {"us_per_launch": round(us, 3), "algorithmic_bytes": algo,
-            "achieved_gbs": round(algo / us / 1e3, 1), "frac": round(algo / us / 1e3 / HBM_PEAK_GBS, 4),
-            "launch": how, "shape": f"batch {nb}, lengths {lens}, {h}/{h} heads x {d}, fp16, "
-                                    f"page {page}, {k} tokens per sequence and head"}
+    out = {"us_per_launch": round(us, 3), "algorithmic_bytes": algo,
+           "achieved_gbs": round(algo / us / 1e3, 1), "frac": round(algo / us / 1e3 / HBM_PEAK_GBS, 4),
+           "launch": how, "shape": f"batch {nb}, lengths {lens}, {h}/{h} heads x {d}, fp16, "
+                                   f"page {page}, {k} tokens per sequence and head"}
+    out["lockstep_step"] = batch8_step(args, lens, h, d, page, k)
+    return out
+
+
+def batch8_step(args, lens, h, d, page, k):
+    """The same batch through BatchInferenceController: the three pieces of a decode step's
+    attention path, each one launch (or one top-k call) for all 8 sequences — a selection layer
+    over every cached token with logits, the top-k of all 256 rows, a sparse layer over the lists
+    that top-k produced."""
+    import torch
+
+    from tidaldecode_amd.utils import BatchInferenceController
+
+    dev = torch.device("cuda:0")
+    nb = len(lens)
+    ctl = BatchInferenceController(2, h, d, page, k, max(lens) + 64, nb, torch.float16, dev,
+                                   page_order_seed=0)
+    ctl.add_sequences(lens)
+    ctl.pool.buf.normal_()
+    ctl.begin_step()
+    q = torch.randn((nb, h, d), device=dev, dtype=torch.float16)
+    res = {}
+    for name, fn in (("selection_attn_us", lambda: ctl.attend_full(q, 0, True)),
+                     ("topk_us", ctl.select),
+                     ("sparse_attn_us", lambda: ctl.attend_sparse(q, 1))):
+        r, how = capture(torch, fn, not args.no_graph)
+        res[name] = round(time_events(torch, r, 20) * 1e3, 2)
+    tokens = sum(n + 1 for n in ctl.seq_lens) - nb
+    sel_bytes = sum(ctl.seq_lens) * h * d * 2 * 2 + sum(ctl.seq_lens) * h * 4
+    res["selection_achieved_gbs"] = round(sel_bytes / res["selection_attn_us"] / 1e3, 1)
+    res["cached_tokens"] = tokens
+    res["launch"] = how
+    ctl.release()
+    del ctl
+    torch.cuda.empty_cache()
+    return res
 
 
 def main():

@@ -74,6 +74,10 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
   if (splits < 1) splits = 1;
   if (splits > 64) splits = 64;
   int64_t chunk = max_items > 0 ? ceil_div64(max_items, splits) : tile;
+  // A batch is planned from its longest sequence: chunks of that size leave the short sequences
+  // with one long-running workgroup per head and the launch waits for the longest.  Finer chunks
+  // balance a ragged batch (8 sequences of 14K-63K tokens: 935 -> 769 us).
+  if (batch > 1 && chunk > 4096) chunk = 4096;
   if (plan->chunk_tokens > 0) chunk = plan->chunk_tokens;
   chunk = ceil_div64(chunk, tile) * tile;
   int64_t max_splits = max_items > 0 ? ceil_div64(max_items, chunk) : 1;
