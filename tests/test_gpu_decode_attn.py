@@ -163,7 +163,17 @@ def test_full_attention_with_scores(cuda, dtype, hq, hkv, n):
     torch.cuda.synchronize()
     assert tolerance_report(od[0], want) <= ATOL[dtype]
     got_logits = scores[:, :n].cpu()
-    assert (got_logits - logits).abs().max() <= 2e-4 * max(1.0, logits.abs().max().item())
+    bound = 2e-4 * max(1.0, logits.abs().max().item())
+    err = (got_logits - logits).abs()
+    if err.max() > bound:   # say where, and whether a second launch gives the same value
+        h, i = divmod(int(err.argmax()), n)
+        scores2 = torch.full_like(scores, float("nan"))
+        w.forward(qd, od, case.pool.to(cuda), table.to(cuda), None, case.last_page_len,
+                  int(case.page_table[-1]), scores2, lse=lse)
+        torch.cuda.synchronize()
+        raise AssertionError(f"logit of head {h}, token {i}: {got_logits[h, i].item()!r}, oracle "
+                             f"{logits[h, i].item()!r}, second launch {scores2[h, i].item()!r}; "
+                             f"{int((err > bound).sum())} entries beyond {bound:.2e}")
     assert torch.isnan(scores[:, n:]).all()  # nothing written past the sequence
     assert (lse[0].cpu() - torch.logsumexp(logits, -1)).abs().max() <= 1e-3
 
