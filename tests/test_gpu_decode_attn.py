@@ -111,7 +111,10 @@ def test_c_restatement_of_reference_checker(cuda, dtype, layout):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("hq,hkv,rows", [(32, 32, 32), (32, 32, 1), (32, 8, 32), (32, 8, 8),
-                                         (32, 8, 1), (16, 8, 8), (64, 8, 8), (40, 40, 40)])
+                                         (32, 8, 1), (16, 8, 8), (64, 8, 8), (40, 40, 40),
+                                         # group sizes without a shared-row kernel (3, 5, 7, 16)
+                                         (24, 8, 8), (24, 8, 24), (20, 4, 4), (28, 4, 1),
+                                         (28, 4, 4), (32, 2, 2)])
 def test_token_slot_lists(cuda, dtype, hq, hkv, rows):
     """Token-granular lists (slots) with page size 16: per query head, per KV head, shared."""
     from oracle import tidal_oracle as orc
@@ -135,7 +138,7 @@ def test_token_slot_lists(cuda, dtype, hq, hkv, rows):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("hq,hkv", [(32, 32), (32, 8)])
+@pytest.mark.parametrize("hq,hkv", [(32, 32), (32, 8), (28, 4)])
 @pytest.mark.parametrize("n", [1, 15, 16, 17, 1000, 4099, 33000])
 def test_full_attention_with_scores(cuda, dtype, hq, hkv, n):
     """Selection-layer mode: the whole page table in order (shared row), logits and lse out.
