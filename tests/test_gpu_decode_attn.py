@@ -427,6 +427,48 @@ def test_random_configurations(cuda, seed):
     assert (lse[0].cpu() - torch.logsumexp(logits, -1)).abs().max() <= 1e-3
 
 
+@pytest.mark.parametrize("fused_merge", [1, 0])
+@pytest.mark.parametrize("hq,hkv", [(6, 2), (12, 4), (10, 2), (12, 2), (28, 4), (7, 1)])
+def test_padded_query_groups(cuda, hq, hkv, fused_merge):
+    """Groups of 3, 5, 6 and 7 query heads per KV head run on the 4- and 8-head shared-row kernels
+    with padding heads: outputs, logits and log-sum-exps of the real heads must be those of the
+    oracle, nothing may be written for the padding, on one split and on many, with the in-kernel
+    and the second-kernel merge."""
+    from oracle import tidal_oracle as orc
+
+    d, page_size, dtype = 128, 16, torch.bfloat16
+    for n, k in ((40, 33), (5000, 1500)):
+        case = PagedCase(n, hkv, d, page_size, dtype, seed=hq * n)
+        q = randn((hq, d), hq + n, dtype)
+        w = _wrapper(0, hq, hkv, d, page_size, dtype, fused_merge=fused_merge)
+        qd = q.to(dtype).to(cuda).unsqueeze(0)
+        pool = case.pool.to(cuda)
+        g = torch.Generator().manual_seed(n)
+        for rows in (hkv, 1):
+            pos = torch.stack([torch.randperm(n, generator=g)[:k] for _ in range(rows)])
+            want = orc.sparse_layer_gather(q, case.k, case.v, pos)
+            od = torch.full((1, hq + 2, d), 9.0, dtype=dtype, device=cuda)  # two guard rows behind o
+            w.forward(qd, od[:, :hq], pool, case.slots_of(pos).to(torch.int32).to(cuda), None, 0, 0, None,
+                      index_kind="slots")
+            torch.cuda.synchronize()
+            assert tolerance_report(od[0, :hq], want) <= ATOL[dtype], (n, rows)
+            assert (od[0, hq:] == 9.0).all()
+        logits = orc.attn_logits(q, case.k)
+        stride = case.n_pages * page_size
+        scores = torch.full((hq + 2, stride), float("nan"), dtype=torch.float32, device=cuda)
+        lse = torch.full((1, hq + 2), float("nan"), dtype=torch.float32, device=cuda)
+        od = torch.empty_like(qd)
+        table = case.page_table[:-1].to(torch.int32).unsqueeze(0).to(cuda)
+        w.forward(qd, od, pool, table, None, case.last_page_len, int(case.page_table[-1]),
+                  scores[:hq], lse=lse[:, :hq])
+        torch.cuda.synchronize()
+        assert tolerance_report(od[0], orc.softmax_pv(logits, case.v)) <= ATOL[dtype], n
+        assert (scores[:hq, :n].cpu() - logits).abs().max() <= 2e-4 * max(1.0, logits.abs().max().item())
+        assert torch.isnan(scores[hq:]).all() and torch.isnan(scores[:hq, n:]).all()
+        assert (lse[0, :hq].cpu() - torch.logsumexp(logits, -1)).abs().max() <= 1e-3
+        assert torch.isnan(lse[0, hq:]).all()
+
+
 @pytest.mark.parametrize("hq,hkv,d", [(4, 4, 128), (8, 2, 128), (4, 2, 128), (8, 1, 128), (2, 2, 64),
                                       (2, 2, 256)])
 def test_logits_of_long_wave_runs(cuda, hq, hkv, d):

@@ -17,7 +17,10 @@ def _ulp_close(a, b, dtype):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("hq,hkv,rows,mode", [(32, 32, 32, "slots"), (32, 32, 1, "pages"),
                                               (32, 8, 8, "slots"), (32, 8, 32, "slots"),
-                                              (32, 8, 1, "pages"), (8, 8, 8, "slots")])
+                                              (32, 8, 1, "pages"), (8, 8, 8, "slots"),
+                                              # groups of 3 and 7 run padded on the 4- and 8-head kernels
+                                              (24, 8, 8, "slots"), (28, 4, 1, "pages"),
+                                              (28, 4, 4, "slots")])
 def test_fused_equals_separate(cuda, dtype, hq, hkv, rows, mode):
     from tidaldecode_amd import _kernels
 

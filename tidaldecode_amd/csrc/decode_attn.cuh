@@ -43,7 +43,9 @@ struct DecodeParams {
   int32_t page_mode;   // 1: list entries are pages, 0: token slots
   int32_t num_qo_heads;
   int32_t n_hrows;   // head rows: num_qo_heads (QPG == 1) or num_kv_heads (QPG > 1)
-  int32_t q_per_kv;  // query heads per KV head (used when QPG == 1)
+  int32_t q_per_kv;  // query heads per KV head
+  int32_t vheads;    // head slots of the split workspace: n_hrows * QPG (QPG may be padded: a group
+                     // of 3 runs as 4, 5-7 as 8; the padding heads have q = 0 and are never stored)
   // index list
   const int32_t* idx;
   int32_t idx_row_stride;  // 0 for a shared row
@@ -117,7 +119,8 @@ __device__ __forceinline__ void load_coherent(const float* src, float& a, float&
 // lse).  Runs in one workgroup of NT threads: NT / (QPG * D / 2) "slots" of threads each own a
 // float2 column and a subset of the splits; slots are combined through LDS.
 template <typename T, int D, int QPG, int NT>
-__device__ __forceinline__ void merge_splits(const DecodeParams& p, int b, int qh0, int n_splits) {
+__device__ __forceinline__ void merge_splits(const DecodeParams& p, int b, int qh0, int rq0, int gsz,
+                                             int n_splits) {
   constexpr int COLS = QPG * D / 2;
   constexpr int SLOTS = NT / COLS;
   constexpr int PRE = SLOTS >= 8 ? 4 : (SLOTS >= 4 ? 8 : 16);  // partial loads in flight per thread
@@ -127,7 +130,7 @@ __device__ __forceinline__ void merge_splits(const DecodeParams& p, int b, int q
   const int tid = threadIdx.x;
   const int c = tid % COLS, slot = tid / COLS;
   const int j = c / (D / 2), d2 = c % (D / 2);
-  const int64_t part0 = ((int64_t)b * p.num_qo_heads + qh0 + j) * p.max_splits;
+  const int64_t part0 = ((int64_t)b * p.vheads + qh0 + j) * p.max_splits;
 
   // (m, l) of every split and head: one pair per thread; the load is unconditional (clamped
   // thread index) so that it is in flight together with the partial loads below
@@ -136,7 +139,7 @@ __device__ __forceinline__ void merge_splits(const DecodeParams& p, int b, int q
   {
     const int tc = has_ml ? tid : 0;
     const int jj = tc / n_splits, ss = tc % n_splits;
-    load_coherent(p.ws_ml + (((int64_t)b * p.num_qo_heads + qh0 + jj) * p.max_splits + ss) * 2,
+    load_coherent(p.ws_ml + (((int64_t)b * p.vheads + qh0 + jj) * p.max_splits + ss) * 2,
                   ml_m, ml_l);
   }
   // Loads are unconditional (index clamped, contribution zeroed) so that a batch of PRE of them
@@ -176,7 +179,7 @@ __device__ __forceinline__ void merge_splits(const DecodeParams& p, int b, int q
     mg_part[slot][c][1] = rb;
   }
   __syncthreads();
-  if (tid < COLS) {
+  if (tid < COLS && j < gsz) {
     float L = 0.f;
     for (int sidx = 0; sidx < n_splits; ++sidx)
       L = fmaf(mg_l[j][sidx], fast_exp2(mg_m[j][sidx] - M), L);
@@ -187,7 +190,7 @@ __device__ __forceinline__ void merge_splits(const DecodeParams& p, int b, int q
       ob += mg_part[sl][c][1];
     }
     const float inv = L > 0.f ? 1.f / L : 0.f;
-    const int qh = qh0 + j;
+    const int qh = rq0 + j;
     reinterpret_cast<uint32_t*>(p.o)[((int64_t)b * p.num_qo_heads + qh) * (D / 2) + d2] =
         pack2<T>(oa * inv, ob * inv);
     if (p.lse && d2 == 0)
@@ -228,7 +231,9 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
   const int split = blockIdx.y;
   const int b = blockIdx.z;
   const int kv_head = (QPG > 1) ? hrow : hrow / p.q_per_kv;
-  const int qh0 = hrow * QPG;  // first query head of this head row
+  const int qh0 = hrow * QPG;  // first head slot of this head row in the split workspace
+  const int gsz = QPG > 1 ? p.q_per_kv : 1;          // query heads that really exist in the row
+  const int rq0 = QPG > 1 ? hrow * p.q_per_kv : hrow;  // first query head of this head row
 
   SeqList s;
   int list_beg;
@@ -246,14 +251,15 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
   uint32_t qp[QPG][4];
   {
     const u32x4* qptr =
-        reinterpret_cast<const u32x4*>(p.q) + ((int64_t)b * p.num_qo_heads + qh0) * LPR + li;
+        reinterpret_cast<const u32x4*>(p.q) + ((int64_t)b * p.num_qo_heads + rq0) * LPR + li;
 #pragma unroll
     for (int j = 0; j < QPG; ++j) {
-      const u32x4 v = qptr[j * LPR];
-      qp[j][0] = v.x;
-      qp[j][1] = v.y;
-      qp[j][2] = v.z;
-      qp[j][3] = v.w;
+      const u32x4 v = qptr[(j < gsz ? j : gsz - 1) * LPR];  // unconditional load, clamped row
+      const bool real = j < gsz;                            // padding heads score with q = 0
+      qp[j][0] = real ? v.x : 0u;
+      qp[j][1] = real ? v.y : 0u;
+      qp[j][2] = real ? v.z : 0u;
+      qp[j][3] = real ? v.w : 0u;
     }
   }
 
@@ -278,7 +284,7 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
     rsn[0] = sgn * s0.x; rsn[1] = sgn * s0.y; rsn[2] = sgn * s0.z; rsn[3] = sgn * s0.w;
     rsn[4] = sgn * s1.x; rsn[5] = sgn * s1.y; rsn[6] = sgn * s1.z; rsn[7] = sgn * s1.w;
     const int64_t fresh_off =
-        ((int64_t)b * (p.num_qo_heads / (QPG > 1 ? QPG : p.q_per_kv)) + kv_head) * LPR + li;
+        ((int64_t)b * (p.num_qo_heads / p.q_per_kv) + kv_head) * LPR + li;
     const u32x4 kn = reinterpret_cast<const u32x4*>(p.fresh_k)[fresh_off];
     const u32x4 vn = reinterpret_cast<const u32x4*>(p.fresh_v)[fresh_off];
     knew[0] = kn.x; knew[1] = kn.y; knew[2] = kn.z; knew[3] = kn.w;
@@ -453,9 +459,9 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
         const int i = emit_first + n * emit_step + ltok;
 #pragma unroll
         for (int j = 0; j < QPG; ++j) {
-          if (n < emit_n && i < c1) {
+          if (n < emit_n && i < c1 && j < gsz) {
             const float nat = emit_buf[((wave * EMIT_TILES + n) * QPG + j) * TILE + ltok];
-            const int64_t at = ((int64_t)b * p.num_qo_heads + qh0 + j) * p.score_stride + i;
+            const int64_t at = ((int64_t)b * p.num_qo_heads + rq0 + j) * p.score_stride + i;
             if (p.scores_f32)
               reinterpret_cast<float*>(p.scores)[at] = nat;
             else
@@ -727,8 +733,9 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
 #pragma unroll
         for (int d = 0; d < 8; ++d) r[d] = fmaf(sm_o[j][w][d][lane], f, r[d]);
       }
-      const int qh = qh0 + j;
+      const int qh = rq0 + j;
       if (n_splits == 1) {
+        if (j >= gsz) continue;  // a padding head: nothing to write
         const float inv = L > 0.f ? 1.f / L : 0.f;
         u32x4 out;
         out.x = pack2<T>(r[0] * inv, r[1] * inv);
@@ -739,7 +746,7 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
         if (p.lse && lane == 0)
           p.lse[(int64_t)b * p.num_qo_heads + qh] = L > 0.f ? (M + fast_log2(L)) * kLn2 : -INFINITY;
       } else {
-        const int64_t part = ((int64_t)b * p.num_qo_heads + qh) * p.max_splits + split;
+        const int64_t part = ((int64_t)b * p.vheads + qh0 + j) * p.max_splits + split;
         float* dst = p.ws_o + part * D + lane * 8;
         store_coherent(dst + 0, r[0], r[1]);
         store_coherent(dst + 2, r[2], r[3]);
@@ -760,7 +767,7 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
     sm_ticket = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
   if (sm_ticket != n_splits - 1) return;
-  merge_splits<T, D, QPG, NW * 64>(p, b, qh0, n_splits);
+  merge_splits<T, D, QPG, NW * 64>(p, b, qh0, rq0, gsz, n_splits);
   if (tid == 0) __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
@@ -773,7 +780,8 @@ __global__ __launch_bounds__(NT) void merge_partials_kernel(const DecodeParams p
   int list_beg;
   const int n_splits = seq_items(p, b, s, list_beg);
   if (n_splits <= 1) return;  // the attention kernel already wrote the final result
-  merge_splits<T, D, QPG, NT>(p, b, hrow * QPG, n_splits);
+  merge_splits<T, D, QPG, NT>(p, b, hrow * QPG, QPG > 1 ? hrow * p.q_per_kv : hrow,
+                              QPG > 1 ? p.q_per_kv : 1, n_splits);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -796,8 +804,11 @@ static bool shape_supported(int head_dim, int qpg, int nw, int rows = 4) {
 // query head walks the list on its own (same result, the KV rows are read once per query head).
 static int qpg_for(int num_qo_heads, int num_kv_heads, int idx_rows, int head_dim) {
   const int group = num_qo_heads / num_kv_heads;
-  if (group > 1 && idx_rows != num_qo_heads && shape_supported(head_dim, group, 8)) return group;
-  return 1;
+  if (group <= 1 || group > 8 || idx_rows == num_qo_heads) return 1;
+  // groups of 3 run on the 4-head kernel, 5 to 7 on the 8-head kernel: the padding heads cost
+  // arithmetic, not memory traffic, which is what bounds these kernels
+  const int padded = group <= 2 ? 2 : (group <= 4 ? 4 : 8);
+  return shape_supported(head_dim, padded, 8) ? padded : 1;
 }
 
 template <typename T, int D, int QPG, int NW, int U, bool PAGE_MODE, bool EMIT>

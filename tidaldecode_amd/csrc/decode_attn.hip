@@ -50,7 +50,7 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
              (long long)max_items);
 
   const int qpg = qpg_for(num_qo_heads, num_kv_heads, idx_rows, head_dim);
-  const int n_hrows = num_qo_heads / qpg;
+  const int n_hrows = qpg > 1 ? num_kv_heads : num_qo_heads;
 
   int nw = plan->waves_per_block;
   if (nw == 0) nw = 8;
@@ -96,7 +96,7 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
   TD_REQUIRE((int64_t)batch * n_hrows * 4 <= kTicketBytes,
              "td_decode_make_plan: batch %d x %d head rows exceeds the %lld ticket counters", batch,
              n_hrows, (long long)(kTicketBytes / 4));
-  const int64_t n_part = (int64_t)batch * num_qo_heads * max_splits;
+  const int64_t n_part = (int64_t)batch * n_hrows * qpg * max_splits;  // head slots incl. padding
   plan->workspace_bytes = kTicketBytes + align256(n_part * head_dim * 4) + align256(n_part * 2 * 4);
   return TD_OK;
 }
@@ -162,11 +162,11 @@ static int build_params(const td_paged_kv* kv, const td_index_list* list, const 
   }
 
   const int qpg = qpg_for(num_qo_heads, Hkv, list->idx_rows, D);
-  const int n_hrows = num_qo_heads / qpg;
+  const int n_hrows = qpg > 1 ? Hkv : num_qo_heads;
   qpg_out = qpg;
   n_hrows_out = n_hrows;
 
-  const int64_t n_part = (int64_t)batch * num_qo_heads * plan->max_splits;
+  const int64_t n_part = (int64_t)batch * n_hrows * qpg * plan->max_splits;
   const int64_t off_o = kTicketBytes;
   const int64_t off_ml = off_o + align256(n_part * D * 4);
   const int64_t need = off_ml + align256(n_part * 2 * 4);
@@ -221,6 +221,7 @@ static int build_params(const td_paged_kv* kv, const td_index_list* list, const 
   }
   p.num_qo_heads = num_qo_heads;
   p.n_hrows = n_hrows;
+  p.vheads = n_hrows * qpg;
   p.q_per_kv = num_qo_heads / Hkv;
   p.idx = list->idx;
   p.idx_row_stride = list->idx_rows == 1 ? 0 : list->idx_row_stride;
