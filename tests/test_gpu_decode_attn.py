@@ -428,10 +428,11 @@ def test_random_configurations(cuda, seed):
 
 
 @pytest.mark.parametrize("fused_merge", [1, 0])
-@pytest.mark.parametrize("hq,hkv", [(6, 2), (12, 4), (10, 2), (12, 2), (28, 4), (7, 1)])
+@pytest.mark.parametrize("hq,hkv", [(6, 2), (12, 4), (10, 2), (12, 2), (28, 4), (7, 1),
+                                    (32, 2), (24, 2), (32, 1), (18, 2)])
 def test_padded_query_groups(cuda, hq, hkv, fused_merge):
     """Groups of 3, 5, 6 and 7 query heads per KV head run on the 4- and 8-head shared-row kernels
-    with padding heads: outputs, logits and log-sum-exps of the real heads must be those of the
+    with padding heads, larger groups (16, 12, 32, 9) as several head rows of 8: outputs, logits and log-sum-exps of the real heads must be those of the
     oracle, nothing may be written for the padding, on one split and on many, with the in-kernel
     and the second-kernel merge."""
     from oracle import tidal_oracle as orc

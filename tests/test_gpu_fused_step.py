@@ -20,7 +20,9 @@ def _ulp_close(a, b, dtype):
                                               (32, 8, 1, "pages"), (8, 8, 8, "slots"),
                                               # groups of 3 and 7 run padded on the 4- and 8-head kernels
                                               (24, 8, 8, "slots"), (28, 4, 1, "pages"),
-                                              (28, 4, 4, "slots")])
+                                              (28, 4, 4, "slots"),
+                                              # 12 heads per KV head: two head rows (8 + 4) per KV head
+                                              (24, 2, 2, "slots"), (24, 2, 1, "pages")])
 def test_fused_equals_separate(cuda, dtype, hq, hkv, rows, mode):
     from tidaldecode_amd import _kernels
 

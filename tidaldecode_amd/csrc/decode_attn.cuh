@@ -46,6 +46,8 @@ struct DecodeParams {
   int32_t q_per_kv;  // query heads per KV head
   int32_t vheads;    // head slots of the split workspace: n_hrows * QPG (QPG may be padded: a group
                      // of 3 runs as 4, 5-7 as 8; the padding heads have q = 0 and are never stored)
+  int32_t subs;      // head rows per KV head on the shared-row kernels: groups above 8 are cut
+                     // into rows of 8 query heads (the last one padded)
   // index list
   const int32_t* idx;
   int32_t idx_row_stride;  // 0 for a shared row
@@ -198,6 +200,24 @@ __device__ __forceinline__ void merge_splits(const DecodeParams& p, int b, int q
   }
 }
 
+// Which query heads a head row of a shared-row kernel (QPG > 1) stands for: its KV head, its first
+// query head and how many of its QPG head slots are real.
+template <int QPG>
+__device__ __forceinline__ void head_row_geom(const DecodeParams& p, int hrow, int& kv_head, int& rq0,
+                                              int& gsz) {
+  if constexpr (QPG > 1) {
+    kv_head = hrow / p.subs;
+    const int sub = hrow - kv_head * p.subs;
+    rq0 = kv_head * p.q_per_kv + sub * QPG;
+    const int left = p.q_per_kv - sub * QPG;
+    gsz = left < QPG ? left : QPG;
+  } else {
+    kv_head = hrow / p.q_per_kv;
+    rq0 = hrow;
+    gsz = 1;
+  }
+}
+
 __device__ __forceinline__ int seq_items(const DecodeParams& p, int b, SeqList& s, int& list_beg) {
   list_beg = 0;
   if (p.indptr) {
@@ -230,16 +250,15 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
   const int hrow = blockIdx.x;
   const int split = blockIdx.y;
   const int b = blockIdx.z;
-  const int kv_head = (QPG > 1) ? hrow : hrow / p.q_per_kv;
   const int qh0 = hrow * QPG;  // first head slot of this head row in the split workspace
-  const int gsz = QPG > 1 ? p.q_per_kv : 1;          // query heads that really exist in the row
-  const int rq0 = QPG > 1 ? hrow * p.q_per_kv : hrow;  // first query head of this head row
+  int kv_head, rq0, gsz;       // KV head, first query head, query heads that really exist in the row
+  head_row_geom<QPG>(p, hrow, kv_head, rq0, gsz);
 
   SeqList s;
   int list_beg;
   const int n_splits = seq_items(p, b, s, list_beg);
   if (split >= n_splits) return;  // uniform for the whole workgroup
-  const int idx_row = (QPG == 1 && p.idx_per_kv) ? kv_head : hrow;
+  const int idx_row = (QPG > 1 || p.idx_per_kv) ? kv_head : hrow;
   s.row = p.idx + (int64_t)idx_row * p.idx_row_stride + list_beg;
 
   // The splits of a head row interleave: split s takes the workgroup-wide tiles s, s + n_splits,
@@ -318,7 +337,7 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
 #pragma unroll
       for (int j = 0; j < QPG; ++j) rotate(qp[j]);
       rotate(knew);
-      const bool writer_row = QPG > 1 || (hrow % p.q_per_kv) == 0;
+      const bool writer_row = rq0 == kv_head * p.q_per_kv;  // the KV head's first head row
       if (split == 0 && wave == 0 && g == 0 && writer_row) {
         const uint32_t page_c = new_page > p.max_page ? p.max_page : new_page;
         char* dst = reinterpret_cast<char*>(const_cast<void*>(p.kv)) + page_c * p.page_stride_b +
@@ -780,8 +799,9 @@ __global__ __launch_bounds__(NT) void merge_partials_kernel(const DecodeParams p
   int list_beg;
   const int n_splits = seq_items(p, b, s, list_beg);
   if (n_splits <= 1) return;  // the attention kernel already wrote the final result
-  merge_splits<T, D, QPG, NT>(p, b, hrow * QPG, QPG > 1 ? hrow * p.q_per_kv : hrow,
-                              QPG > 1 ? p.q_per_kv : 1, n_splits);
+  int kv_head, rq0, gsz;
+  head_row_geom<QPG>(p, hrow, kv_head, rq0, gsz);
+  merge_splits<T, D, QPG, NT>(p, b, hrow * QPG, rq0, gsz, n_splits);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -804,9 +824,10 @@ static bool shape_supported(int head_dim, int qpg, int nw, int rows = 4) {
 // query head walks the list on its own (same result, the KV rows are read once per query head).
 static int qpg_for(int num_qo_heads, int num_kv_heads, int idx_rows, int head_dim) {
   const int group = num_qo_heads / num_kv_heads;
-  if (group <= 1 || group > 8 || idx_rows == num_qo_heads) return 1;
-  // groups of 3 run on the 4-head kernel, 5 to 7 on the 8-head kernel: the padding heads cost
-  // arithmetic, not memory traffic, which is what bounds these kernels
+  if (group <= 1 || idx_rows == num_qo_heads) return 1;
+  // groups of 3 run on the 4-head kernel, 5 to 7 on the 8-head kernel, larger ones as several head
+  // rows of 8: the padding heads cost arithmetic, not memory traffic, which is what bounds these
+  // kernels
   const int padded = group <= 2 ? 2 : (group <= 4 ? 4 : 8);
   return shape_supported(head_dim, padded, 8) ? padded : 1;
 }

@@ -50,7 +50,8 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
              (long long)max_items);
 
   const int qpg = qpg_for(num_qo_heads, num_kv_heads, idx_rows, head_dim);
-  const int n_hrows = qpg > 1 ? num_kv_heads : num_qo_heads;
+  const int subs = qpg > 1 ? (num_qo_heads / num_kv_heads + qpg - 1) / qpg : 1;
+  const int n_hrows = qpg > 1 ? num_kv_heads * subs : num_qo_heads;
 
   int nw = plan->waves_per_block;
   if (nw == 0) nw = 8;
@@ -162,7 +163,8 @@ static int build_params(const td_paged_kv* kv, const td_index_list* list, const 
   }
 
   const int qpg = qpg_for(num_qo_heads, Hkv, list->idx_rows, D);
-  const int n_hrows = qpg > 1 ? Hkv : num_qo_heads;
+  const int subs = qpg > 1 ? (num_qo_heads / Hkv + qpg - 1) / qpg : 1;
+  const int n_hrows = qpg > 1 ? Hkv * subs : num_qo_heads;
   qpg_out = qpg;
   n_hrows_out = n_hrows;
 
@@ -222,6 +224,7 @@ static int build_params(const td_paged_kv* kv, const td_index_list* list, const 
   p.num_qo_heads = num_qo_heads;
   p.n_hrows = n_hrows;
   p.vheads = n_hrows * qpg;
+  p.subs = subs;
   p.q_per_kv = num_qo_heads / Hkv;
   p.idx = list->idx;
   p.idx_row_stride = list->idx_rows == 1 ? 0 : list->idx_row_stride;
