@@ -13,6 +13,8 @@
 //
 // With grouped-query attention and an index list shared by the query heads of a KV head
 // (QPG > 1) each lane group loads the KV row once and scores it against QPG query heads.
+// QPG is 2, 4 or 8; other group sizes are padded up (3 -> 4, 5..7 -> 8) or cut into head rows of
+// 8 (groups above 8), the padding heads scoring with q = 0 and never being written.
 //
 // Semantics follow kernels/include/decode/decode_attn.cuh:432-658 of the reference
 // (BatchDecodeWithPagedKVCacheKernel) including the forced last page
@@ -42,7 +44,7 @@ struct DecodeParams {
   uint32_t max_page;   // max_pages - 1
   int32_t page_mode;   // 1: list entries are pages, 0: token slots
   int32_t num_qo_heads;
-  int32_t n_hrows;   // head rows: num_qo_heads (QPG == 1) or num_kv_heads (QPG > 1)
+  int32_t n_hrows;   // head rows: num_qo_heads (QPG == 1) or num_kv_heads * subs (QPG > 1)
   int32_t q_per_kv;  // query heads per KV head
   int32_t vheads;    // head slots of the split workspace: n_hrows * QPG (QPG may be padded: a group
                      // of 3 runs as 4, 5-7 as 8; the padding heads have q = 0 and are never stored)
