@@ -245,6 +245,10 @@ int td_score_reduce(const float* logits, int64_t logits_stride, const float* lse
  *                                    (rows_per_table == 0: one table for all rows)
  *     both NULL                   -> p
  * k is clamped to len.  NaNs order above +inf.  out rows have stride out_stride.
+ * len_arr (device, one entry per group of rows_per_table rows, or NULL): row r takes only its
+ * first len_arr[r / rows_per_table] elements (clamped to 1..len) and selects min(k, that many);
+ * the rest of its output row is left untouched.  Lengths that live on the device let a batch of
+ * sequences of different lengths, or a captured graph whose sequence grows, use one call.
  * workspace: see td_topk_workspace_bytes (optional).
  * Replaces topk_filtering (bsk_ops.h:34-39, tidal/ops/csrc/topk.cu:7-44) and decode_select_k
  * (kernels/include/topk/decode_select_k.cuh:25-62; RAFT radix_topk_one_block_kernel).
@@ -252,7 +256,7 @@ int td_score_reduce(const float* logits, int64_t logits_stride, const float* lse
 int td_topk(const void* values, int32_t values_dtype, int64_t values_stride, int32_t rows,
             int32_t len, int32_t k, const int32_t* in_idx, int64_t in_idx_stride,
             const int32_t* page_table, int64_t page_table_stride, int32_t rows_per_table,
-            int32_t page_size, void* out_values, int32_t* out_idx, int64_t out_stride,
+            const int32_t* len_arr, int32_t page_size, void* out_values, int32_t* out_idx, int64_t out_stride,
             void* workspace, int64_t workspace_bytes, void* stream);
 
 /*

@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     raw = ctypes.CDLL(_lib.LIB_PATH)
     for n in names:
         assert hasattr(raw, n), n
-    assert _lib.lib.td_version() == 3
+    assert _lib.lib.td_version() == 4
     assert isinstance(_lib.last_error(), str)
 
 
@@ -85,7 +85,7 @@ def test_argument_checks_fire_before_any_launch():
     assert lib.td_decode_attn(None, None, None, None, None, 1, 32, 0.1, None, 0, 0, None, None, None,
                               0, None) == _lib.TD_ERR_INVALID_ARG
     assert lib.td_rope_table(None, 1, 128, 1.0, 1e4, None, None, None) == _lib.TD_ERR_INVALID_ARG
-    assert lib.td_topk(None, 2, 0, 1, 1, 1, None, 0, None, 0, 0, 1, None, None, 1, None, 0, None) \
+    assert lib.td_topk(None, 2, 0, 1, 1, 1, None, 0, None, 0, 0, None, 1, None, None, 1, None, 0, None) \
         == _lib.TD_ERR_INVALID_ARG
     assert lib.td_rope_in_place(None, None, 1, 1, 1, 128, 0, 1.0, 1e4, 0, None) \
         == _lib.TD_ERR_INVALID_ARG

@@ -214,6 +214,44 @@ def test_page_table_per_row_group(cuda):
                                 page_table=torch.zeros((2, 100), dtype=torch.int32, device=cuda))
 
 
+def test_lengths_per_row_group(cuda):
+    """Device-side lengths: rows of group g rank only their first lengths[g] columns (what lies
+    behind is larger than everything and must not be chosen) and select min(k, lengths[g]);
+    the rest of a short row's output stays as it was."""
+    from oracle import tidal_oracle as orc
+    from tidaldecode_amd import _kernels
+
+    g = torch.Generator().manual_seed(23)
+    for per, n, k, lens, page in ((4, 3000, 100, [3000, 57, 1, 100, 2999], 16),
+                                  (8, 40000, 2048, [40000, 9000, 17, 8193, 30000], 16),
+                                  (1, 70000, 500, [70000, 12, 65537], 4)):
+        groups = len(lens)
+        rows = groups * per
+        v = torch.randn((rows, n), generator=g)
+        for gi, ln in enumerate(lens):
+            v[gi * per: (gi + 1) * per, ln:] = 1e9
+        n_pages = (n + page - 1) // page
+        tables = torch.stack([torch.randperm(n_pages + 3, generator=g)[:n_pages] for _ in range(groups)]).int()
+        lengths = torch.tensor(lens, dtype=torch.int32, device=cuda)
+        for scratch in (False, True):
+            out = torch.full((rows, k), -1, dtype=torch.int32, device=cuda)
+            _kernels.topk_filtering(v.to(cuda), None, None, out, _shared_scratch(cuda, rows) if scratch else None,
+                                    k, page_table=tables.to(cuda), page_size=page, lengths=lengths)
+            torch.cuda.synchronize()
+            out = out.cpu().long()
+            for r in range(rows):
+                ln = lens[r // per]
+                kr = min(k, ln)
+                pos = orc.stable_topk(v[r: r + 1, :ln], kr)[0]
+                want = tables[r // per].long()[pos // page] * page + pos % page
+                assert torch.equal(out[r, :kr], want), (n, r, scratch)
+                assert (out[r, kr:] == -1).all(), (n, r, scratch)
+    with pytest.raises(RuntimeError, match="lengths"):
+        _kernels.topk_filtering(torch.zeros((5, 100), device=cuda), None, None,
+                                torch.zeros((5, 10), dtype=torch.int32, device=cuda), None, 10,
+                                lengths=torch.ones(2, dtype=torch.int32, device=cuda))
+
+
 def test_topk_errors(cuda):
     from tidaldecode_amd import _kernels
 

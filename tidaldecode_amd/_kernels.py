@@ -160,7 +160,8 @@ def gemv(weight: torch.Tensor, x: torch.Tensor, *, norm_weight: Optional[torch.T
 def topk_filtering(estimated_value: torch.Tensor, estimated_indices: Optional[torch.Tensor],
                    d_out: Optional[torch.Tensor], indices_out: torch.Tensor,
                    buf: Optional[torch.Tensor], page_budget: int, *,
-                   page_table: Optional[torch.Tensor] = None, page_size: int = 1) -> None:
+                   page_table: Optional[torch.Tensor] = None, page_size: int = 1,
+                   lengths: Optional[torch.Tensor] = None) -> None:
     """bsk_ops.h:34-39 / topk.cu:7-44.  Row-wise top-``page_budget`` of ``estimated_value``
     ``[H, len]``; ``indices_out[h, j]`` is ``estimated_indices[h, p]`` of the selected position
     ``p``.  ``buf`` is scratch, as in the reference (there: RAFT's): a zero-initialised uint8 /
@@ -175,7 +176,9 @@ def topk_filtering(estimated_value: torch.Tensor, estimated_indices: Optional[to
 
     Extensions: ``estimated_indices=None`` returns positions, or physical token slots when a
     ``page_table`` ``[n_pages]`` is given (``[groups, n_pages]``: one table per ``H / groups``
-    consecutive rows, the sequences of a batch); fp32 values.
+    consecutive rows, the sequences of a batch); fp32 values.  ``lengths`` (int32 device
+    ``[groups]``): rows of group g use only their first ``lengths[g]`` columns and select
+    ``min(page_budget, lengths[g])`` of them, leaving the rest of their output row untouched.
     """
     _check_rows(estimated_value, "estimated_value")
     rows, length = estimated_value.shape
@@ -216,6 +219,15 @@ def topk_filtering(estimated_value: torch.Tensor, estimated_indices: Optional[to
         if page_table.size(-1) * page_size < length:
             raise RuntimeError("page_table does not cover the row")
         pt_ptr = page_table.data_ptr()
+    len_ptr = None
+    if lengths is not None:
+        _check_input(lengths, "lengths")
+        _check_i32(lengths, "lengths")
+        groups = lengths.numel()
+        if groups < 1 or rows % groups != 0 or (rows_per_table and rows_per_table != rows // groups):
+            raise RuntimeError(f"lengths has {groups} entries for {rows} rows")
+        rows_per_table = rows // groups
+        len_ptr = lengths.data_ptr()
     ws_ptr, ws_bytes = None, 0
     if buf is not None and buf.is_cuda and buf.is_contiguous():
         ws_bytes = buf.numel() * buf.element_size()
@@ -224,7 +236,7 @@ def topk_filtering(estimated_value: torch.Tensor, estimated_indices: Optional[to
     check(lib.td_topk(estimated_value.data_ptr(),
                       _dtype_code(estimated_value.dtype, "Top-k filtering"),
                       estimated_value.stride(0), rows, length, k, in_ptr, in_stride, pt_ptr,
-                      pt_stride, rows_per_table, int(page_size), out_vals, indices_out.data_ptr(), indices_out.stride(0),
+                      pt_stride, rows_per_table, len_ptr, int(page_size), out_vals, indices_out.data_ptr(), indices_out.stride(0),
                       ws_ptr, ws_bytes if ws_ptr else 0, _stream()))
 
 

@@ -117,7 +117,8 @@ SIGNATURES = {
     "td_topk": (
         c_int32,
         [c_void_p, c_int32, c_int64, c_int32, c_int32, c_int32, c_void_p, c_int64, c_void_p,
-         c_int64, c_int32, c_int32, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p],
+         c_int64, c_int32, c_void_p, c_int32, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
+         c_void_p],
     ),
     "td_topk_workspace_bytes": (c_int64, [c_int32]),
     "td_gather_probe": (

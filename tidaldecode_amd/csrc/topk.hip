@@ -29,7 +29,8 @@ struct TopkParams {
   int64_t in_idx_stride;
   const int32_t* page_table;
   int64_t page_table_stride;  // elements between the tables of consecutive row groups
-  int32_t rows_per_table;     // rows that share one table (all rows when there is one table)
+  int32_t rows_per_table;     // rows that share one table / one length (all rows when there is one)
+  const int32_t* len_arr;     // per row group: elements that take part (clamped to 1..len), or null
   int32_t page_size;
   int32_t page_shift;  // log2(page_size) when it is a power of two, else -1
   void* out_values;
@@ -42,6 +43,14 @@ __device__ __forceinline__ const int32_t* table_of(const TopkParams& p, int row)
   if (p.page_table == nullptr || p.page_table_stride == 0) return p.page_table;
   return p.page_table + (int64_t)(row / p.rows_per_table) * p.page_table_stride;
 }
+// elements of this row that take part, and how many of them are selected
+__device__ __forceinline__ int row_len(const TopkParams& p, int row) {
+  if (p.len_arr == nullptr) return p.len;
+  const int n = p.len_arr[row / p.rows_per_table];
+  return n < 1 ? 1 : (n > p.len ? p.len : n);
+}
+__device__ __forceinline__ int row_k(const TopkParams& p, int len) { return p.k < len ? p.k : len; }
+
 __device__ __forceinline__ int32_t slot_of(const TopkParams& p, const int32_t* table, int i) {
   if (p.page_shift >= 0)
     return (table[i >> p.page_shift] << p.page_shift) | (i & (p.page_size - 1));
@@ -116,8 +125,8 @@ __global__ __launch_bounds__(kTopkThreads) void topk_kernel(const TopkParams p) 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int len = p.len;
-  const int k = p.k;  // 1 <= k <= len (host-checked)
+  const int len = row_len(p, row);
+  const int k = row_k(p, len);  // 1 <= k <= len
   const elem_t* vals = reinterpret_cast<const elem_t*>(p.values) + (int64_t)row * p.values_stride;
 
   __shared__ uint32_t hist[kMaxBins];
@@ -275,8 +284,8 @@ __global__ __launch_bounds__(kTopkThreads) void topk_reg_kernel(const TopkParams
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int len = p.len;
-  const int k = p.k;  // 1 <= k <= len <= 1024 * IPT (host-checked)
+  const int len = row_len(p, row);
+  const int k = row_k(p, len);  // 1 <= k <= len <= 1024 * IPT (host-checked for p.len)
   const elem_t* vals = reinterpret_cast<const elem_t*>(p.values) + (int64_t)row * p.values_stride;
 
   __shared__ uint32_t hist[kMaxBins];
@@ -519,7 +528,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_coop_hist_kernel(const Topk
   int slice, row;
   if (!coop_decode(n_slices, rows, slice, row)) return;
   const int tid = threadIdx.x;
-  const int len = p.len;
+  const int len = row_len(p, row);
   const void* vals = reinterpret_cast<const char*>(p.values) +
                      (int64_t)row * p.values_stride * sizeof(typename ElemOf<T>::type);
   uint32_t* rs = scratch + (int64_t)row * kCoopRowWords;
@@ -546,7 +555,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_coop_select_kernel(const To
   int slice, row;
   if (!coop_decode(n_slices, rows, slice, row)) return;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int len = p.len;
+  const int len = row_len(p, row);
   const void* vals = reinterpret_cast<const char*>(p.values) +
                      (int64_t)row * p.values_stride * sizeof(typename ElemOf<T>::type);
   uint32_t* rs = scratch + (int64_t)row * kCoopRowWords;
@@ -572,7 +581,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_coop_select_kernel(const To
   if (tid < kCoopMaxSlices) slice_gt[tid] = slice_eq[tid] = 0;
   if (tid == 0) n_cand_sh = n_above_sh = 0;
   __syncthreads();
-  uint32_t prefix = 0, mask = 0, krem = (uint32_t)p.k;
+  uint32_t prefix = 0, mask = 0, krem = (uint32_t)row_k(p, len);
   {
     const int my_bin = tid * 2;
     const uint32_t local = hist[my_bin] + hist[my_bin + 1];
@@ -806,7 +815,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_coop_emit_kernel(const Topk
   int slice, row;
   if (!coop_decode(n_slices, rows, slice, row)) return;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int len = p.len;
+  const int len = row_len(p, row);
   const elem_t* vals = reinterpret_cast<const elem_t*>(p.values) + (int64_t)row * p.values_stride;
   const uint32_t* rs = scratch + (int64_t)row * kCoopRowWords;
   const uint32_t thr = rs[2049], r = rs[2050];
@@ -877,7 +886,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_coop_emit_kernel(const Topk
     const bool sel = gt || (eq && eq_rank < r);
     const uint64_t sel_mask = __ballot(sel);
     const uint32_t pos = run_out[j * kTopkWaves + wave] + lanes_below(sel_mask);
-    if (sel && pos < (uint32_t)p.k) {
+    if (sel && pos < (uint32_t)row_k(p, len)) {
       out_idx[pos] = payload[j];
       if (out_val) out_val[pos] = val[j];
     }
@@ -949,8 +958,8 @@ using namespace tidal;
 extern "C" int td_topk(const void* values, int32_t values_dtype, int64_t values_stride,
                        int32_t rows, int32_t len, int32_t k, const int32_t* in_idx,
                        int64_t in_idx_stride, const int32_t* page_table,
-                       int64_t page_table_stride, int32_t rows_per_table, int32_t page_size,
-                       void* out_values, int32_t* out_idx, int64_t out_stride, void* workspace,
+                       int64_t page_table_stride, int32_t rows_per_table,
+                       const int32_t* len_arr, int32_t page_size, void* out_values, int32_t* out_idx, int64_t out_stride, void* workspace,
                        int64_t workspace_bytes, void* stream) {
   TD_REQUIRE(values && out_idx, "td_topk: NULL values or out_idx");
   TD_REQUIRE(rows >= 1, "td_topk: rows %d < 1", rows);
@@ -961,7 +970,7 @@ extern "C" int td_topk(const void* values, int32_t values_dtype, int64_t values_
   TD_REQUIRE(out_stride >= k, "td_topk: out_stride %lld < k %d", (long long)out_stride, k);
   TD_REQUIRE(!in_idx || in_idx_stride >= 0, "td_topk: in_idx_stride %lld", (long long)in_idx_stride);
   TD_REQUIRE(!page_table || page_size >= 1, "td_topk: page_size %d", page_size);
-  TD_REQUIRE(!page_table || (rows_per_table >= 0 && page_table_stride >= 0),
+  TD_REQUIRE((!page_table && !len_arr) || (rows_per_table >= 0 && page_table_stride >= 0),
              "td_topk: rows_per_table %d / page_table_stride %lld", rows_per_table,
              (long long)page_table_stride);
   if (k == 0) return TD_OK;
@@ -975,6 +984,7 @@ extern "C" int td_topk(const void* values, int32_t values_dtype, int64_t values_
   p.page_table = in_idx ? nullptr : page_table;
   p.page_table_stride = page_table_stride;
   p.rows_per_table = rows_per_table >= 1 ? rows_per_table : rows;
+  p.len_arr = len_arr;
   p.page_size = page_size;
   p.page_shift = -1;
   if (page_size >= 1 && (page_size & (page_size - 1)) == 0) p.page_shift = __builtin_ctz(page_size);

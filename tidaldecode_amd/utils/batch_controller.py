@@ -8,8 +8,8 @@ counterpart of ``InferenceController`` for that kernel surface:
 * one pool per layer shared by all sequences, one fixed-width page-table segment per sequence in a
   device tensor ``[max_batch, pages_per_seq]`` that grows in place;
 * the per-sequence metadata of a decode step (pages before the last one, fill of the last page,
-  its id, the slot and the position of the new token, the number of selected tokens) is one
-  ``[6, max_batch]`` int32 device tensor refreshed by a single small copy per step — never the
+  its id, the slot and the position of the new token, the number of selected tokens, the length) is one
+  ``[7, max_batch]`` int32 device tensor refreshed by a single small copy per step — never the
   page tables themselves;
 * selection state for the whole batch: logits ``[B * H_q, max tokens]`` (``-inf`` where a sequence
   has no token, so that one top-k call serves ragged lengths), the log-sum-exp per head and the
@@ -28,7 +28,8 @@ from .paged import BatchDecodeWithPagedKVCacheWrapper, KvPool, TensorLayout
 
 _SELECT_MODES = ("per_head", "group_sum", "head_sum")
 # rows of the per-step metadata tensor
-_PAGES_BEFORE_LAST, _LAST_LEN, _LAST_IDX, _DST_SLOT, _POSITION, _SELECTED = range(6)
+_PAGES_BEFORE_LAST, _LAST_LEN, _LAST_IDX, _DST_SLOT, _POSITION, _SELECTED, _SEQ_LEN = range(7)
+_META_ROWS = 7
 
 
 class BatchInferenceController:
@@ -56,11 +57,11 @@ class BatchInferenceController:
         self.page_table = torch.zeros((max_batch, self.pages_per_seq), **i32)
         self._pages: List[List[int]] = []
         self.seq_lens: List[int] = []
-        self._meta = torch.zeros((6, max_batch), **i32)
+        self._meta = torch.zeros((_META_ROWS, max_batch), **i32)
         # staging for the per-step copy: a small ring of pinned rows, so that the copy is
         # asynchronous and a buffer is only rewritten after its copy has completed
         self._on_gpu = torch.device(device).type == "cuda"
-        self._stage = [torch.zeros((6, max_batch), dtype=torch.int32, pin_memory=self._on_gpu)
+        self._stage = [torch.zeros((_META_ROWS, max_batch), dtype=torch.int32, pin_memory=self._on_gpu)
                        for _ in range(4)]
         self._stage_done = [None] * len(self._stage)
         self._stage_next = 0
@@ -141,8 +142,8 @@ class BatchInferenceController:
             pages = self._pages[b]
             last_len = (n - 1) % P + 1
             cols.append((len(pages) - 1, last_len, pages[-1], pages[-1] * P + last_len - 1, n - 1,
-                         min(self.budget, n)))
-        cols += [(0,) * 6] * (self.max_batch - len(cols))
+                         min(self.budget, n), n))
+        cols += [(0,) * _META_ROWS] * (self.max_batch - len(cols))
         i = self._stage_next
         self._stage_next = (i + 1) % len(self._stage)
         if self._stage_done[i] is not None:
@@ -236,12 +237,12 @@ class BatchInferenceController:
                                   out=self.score_sum[: B * rows])
             scores = self.score_sum[: B * rows]
         k_eff = min(k, n)
-        # one call: row b * rows + r is row r of sequence b and goes through that sequence's page
-        # table; entries past a sequence's own count are never read (positions come out sorted,
-        # the valid ones first)
+        # one call: row b * rows + r is row r of sequence b, ranks that sequence's tokens only
+        # (its length is read on the device) and goes through that sequence's page table
         out = self._slots[: B * rows, :k_eff]
         _kernels.topk_filtering(scores[:, :n], None, None, out, self.topk_buf, k_eff,
-                                page_table=self.page_table[:B], page_size=P)
+                                page_table=self.page_table[:B], page_size=P,
+                                lengths=self._row(_SEQ_LEN))
         self.topk_dindices_buffer.view(rows, self.max_batch, k)[:, :B, :k_eff] = \
             out.view(B, rows, k_eff).permute(1, 0, 2)
 
