@@ -359,6 +359,13 @@ def e2e_leg(args):
                                   "prefill_tokens_per_s": round(ctx / (t1 - t0), 1),
                                   "greedy_steps": n_gen,
                                   "greedy_ms_per_token": round((time.perf_counter() - t1) / n_gen * 1e3, 4)}
+            # the same prompt again, decoded by replaying ONE captured step whose sequence state
+            # lives on the device (no host work between tokens)
+            model.tidal_clear()
+            toks = model.generate_graph(ids, n_gen, use_graph=not args.no_graph)
+            row["real_prompt"]["greedy_graph_replay_ms_per_token"] = round(
+                model.iController.decode_latency[-1] * 1e3, 4)
+            row["real_prompt"]["greedy_graph_replay_tokens"] = int(toks.numel())
         out[str(ctx)] = row
     del model
     torch.cuda.empty_cache()

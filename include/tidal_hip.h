@@ -224,6 +224,36 @@ int td_rope_table(const int32_t* positions, int32_t batch, int32_t head_dim, flo
                   float rope_theta, float* cos, float* sin, void* stream);
 
 /*
+ * Device-resident state of one decoding sequence: everything the launches of a decode step need to
+ * know about the sequence, as int32 words that td_step_advance keeps current, so that a decode
+ * step captured in a HIP graph stays valid while the sequence grows (td_index_list.count_arr,
+ * last_page_len_arr, last_page_idx_arr, td_fresh_token.dst_slot, td_rope_table's positions and
+ * td_topk's len_arr all point into it).  No counterpart in the reference, whose controller
+ * rebuilds and re-uploads this on the host every step (tidal/utils/controller.py:89-147).
+ */
+enum {
+  TD_STEP_SEQ_LEN = 0,           /* tokens in the cache, the one being decoded included */
+  TD_STEP_PAGES_BEFORE_LAST = 1, /* full pages before the page being filled */
+  TD_STEP_LAST_PAGE_LEN = 2,     /* entries in use in the page being filled, 1..page_size */
+  TD_STEP_LAST_PAGE_IDX = 3,     /* its physical page id */
+  TD_STEP_DST_SLOT = 4,          /* physical slot of the token being decoded */
+  TD_STEP_POSITION = 5,          /* its position, seq_len - 1 */
+  TD_STEP_N_SELECTED = 6,        /* min(budget, seq_len): entries of the persisted token lists */
+  TD_STEP_COUNT = 7,             /* steps taken */
+  TD_STEP_WORDS = 8
+};
+
+/*
+ * Advance the state by one token (one tiny launch, graph-safe): seq_len += 1 and the other words
+ * follow from page_table [n_pages] (the pages of the sequence in order; the caller has reserved
+ * pages for every token it will decode).  If token / tokens_out are given, the token id the step
+ * consumes (*token) is first recorded at tokens_out[steps taken] (ignored beyond tokens_cap).
+ */
+int td_step_advance(int32_t* state, const int32_t* page_table, int32_t n_pages, int32_t page_size,
+                    int32_t budget, const int64_t* token, int64_t* tokens_out, int32_t tokens_cap,
+                    void* stream);
+
+/*
  * Cross-head reduction of selection-layer scores: out[r, i] = sum over the query heads h of
  * row r of exp(logits[h, i] - lse[h]) (i < n), fp32.  rows = 1 (TD_REDUCE_HEAD_SUM) or
  * num_kv_heads (TD_REDUCE_GROUP_SUM).  logits is float [num_qo_heads, logits_stride].

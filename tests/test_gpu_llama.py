@@ -157,3 +157,58 @@ def test_layer_schedule_and_full_mode(cuda):
     assert _close(model.decode_step(tok), _reference_logits(model, torch.cat([ids, tok])))
     dt, how = model.timed_decode(steps=3, warmup=1)
     assert dt > 0 and how in ("hipGraph", "eager")
+
+
+@pytest.mark.parametrize("select_mode,top_k", [("per_head", 4096), ("head_sum", 4096), ("per_head", 12),
+                                               ("group_sum", 24)])
+def test_generation_by_replaying_one_captured_step(cuda, select_mode, top_k):
+    """generate_graph: the step state lives on the device and one captured step is replayed per
+    token.  Every replay must give what the same step gives when launched eagerly (bit for bit:
+    same kernels, same plans), and the logits must be those of the host-driven decode_step fed
+    with the same tokens (another split plan: bf16 tolerance; with a small budget a near-tie in
+    the selection may pick another token, so that comparison is looser)."""
+    from tidaldecode_amd import _lib
+    from tidaldecode_amd.llama import TidalLlama
+
+    n_prompt, n_new = 70, 40   # crosses two page boundaries
+    model = TidalLlama(_small(select_mode=select_mode, top_k=top_k), cuda, seed=4, init_std=0.05)
+    model.tidal_init(page_size=16, max_seq_len=256, page_order_seed=5)
+    ids = torch.randint(0, 1000, (n_prompt,), device=cuda, generator=torch.Generator(device=cuda).manual_seed(9))
+    tokens, kept = model.generate_graph(ids, n_new, keep_logits=True)
+    assert model.iController.kv_cache.seqlen == n_prompt + n_new
+    model.tidal_clear()
+    tokens_e, kept_e = model.generate_graph(ids, n_new, keep_logits=True, use_graph=False)
+    assert torch.equal(tokens, tokens_e) and torch.equal(kept, kept_e)
+    assert torch.equal(tokens[1:], kept[:-1].argmax(-1))       # greedy: each row chose the next token
+    model.tidal_clear()
+    # host-driven steps with the same tokens
+    logits = model.prefill(ids)
+    assert int(logits.argmax()) == int(tokens[0])
+    rel = 2e-2 if top_k >= 4096 else 1e-1
+    for i in range(n_new):
+        logits = model.decode_step(tokens[i: i + 1])
+        assert _close(kept[i], logits.float(), rel=rel), i
+    model.tidal_clear()
+    assert model._dev is None
+
+
+def test_step_state_words(cuda):
+    from tidaldecode_amd import _kernels, _lib
+
+    table = torch.tensor([7, 3, 9, 1], dtype=torch.int32, device=cuda)
+    state = torch.zeros(_lib.TD_STEP_WORDS, dtype=torch.int32, device=cuda)
+    state[_lib.TD_STEP_SEQ_LEN] = 6
+    token = torch.tensor([41], dtype=torch.int64, device=cuda)
+    out = torch.full((5,), -1, dtype=torch.int64, device=cuda)
+    want = []
+    for step in range(7):   # lengths 7 .. 13 with pages of 4
+        token.fill_(100 + step)
+        _kernels.step_advance(state, table, 4, 10, token, out)
+        n = 7 + step
+        pos = n - 1
+        page = [7, 3, 9, 1][pos // 4]
+        want = [n, pos // 4, pos % 4 + 1, page, page * 4 + pos % 4, pos, min(10, n), step + 1]
+        assert state.tolist() == want, step
+    assert out.tolist() == [100, 101, 102, 103, 104]          # recording stops at the capacity
+    with pytest.raises(RuntimeError):
+        _kernels.step_advance(state, table, 4, 10, token, None)

@@ -345,6 +345,33 @@ def rope_append_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, kv_dat
                                     float(rope_theta), _stream()))
 
 
+def step_advance(state: torch.Tensor, page_table: torch.Tensor, page_size: int, budget: int,
+                 token: Optional[torch.Tensor] = None,
+                 tokens_out: Optional[torch.Tensor] = None) -> None:
+    """Extension: the sequence described by ``state`` (int32 device ``[TD_STEP_WORDS]``, see
+    ``_lib.TD_STEP_*``) grows by one token; its words are recomputed on the device from the
+    sequence's ``page_table`` (int32 ``[n_pages]``, pages reserved ahead).  ``token`` (int64
+    ``[1]``) is recorded at ``tokens_out[steps taken]`` first.  Safe inside a captured graph."""
+    _check_input(state, "state")
+    _check_input(page_table, "page_table")
+    _check_i32(state, "state")
+    _check_i32(page_table, "page_table")
+    if state.numel() < _lib.TD_STEP_WORDS:
+        raise RuntimeError(f"state must hold {_lib.TD_STEP_WORDS} int32 words")
+    tok_ptr = out_ptr = None
+    cap = 0
+    if token is not None or tokens_out is not None:
+        if token is None or tokens_out is None:
+            raise RuntimeError("token and tokens_out go together")
+        _check_input(token, "token")
+        _check_input(tokens_out, "tokens_out")
+        if token.dtype != torch.int64 or tokens_out.dtype != torch.int64 or token.numel() < 1:
+            raise RuntimeError("token and tokens_out must be int64")
+        tok_ptr, out_ptr, cap = token.data_ptr(), tokens_out.data_ptr(), tokens_out.numel()
+    check(lib.td_step_advance(state.data_ptr(), page_table.data_ptr(), page_table.numel(),
+                              int(page_size), int(budget), tok_ptr, out_ptr, cap, _stream()))
+
+
 def rope_table(positions: torch.Tensor, head_dim: int, rope_scale: float = 1.0,
                rope_theta: float = 1e4, cos: Optional[torch.Tensor] = None,
                sin: Optional[torch.Tensor] = None):

@@ -16,6 +16,9 @@ TD_F16, TD_BF16, TD_F32 = 0, 1, 2
 TD_NHD, TD_HND = 0, 1
 TD_IDX_PAGES, TD_IDX_SLOTS = 0, 1
 TD_REDUCE_HEAD_SUM, TD_REDUCE_GROUP_SUM = 0, 1
+# words of the device-resident step state (td_step_advance)
+(TD_STEP_SEQ_LEN, TD_STEP_PAGES_BEFORE_LAST, TD_STEP_LAST_PAGE_LEN, TD_STEP_LAST_PAGE_IDX,
+ TD_STEP_DST_SLOT, TD_STEP_POSITION, TD_STEP_N_SELECTED, TD_STEP_COUNT, TD_STEP_WORDS) = range(9)
 
 
 class PagedKV(Structure):
@@ -104,6 +107,10 @@ SIGNATURES = {
         [POINTER(PagedKV), POINTER(IndexList), POINTER(DecodePlan), c_void_p, c_void_p, c_int32,
          c_int32, c_float, c_void_p, c_int32, c_int64, c_void_p, POINTER(FreshToken), c_void_p,
          c_int64, c_void_p],
+    ),
+    "td_step_advance": (
+        c_int32,
+        [c_void_p, c_void_p, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_int32, c_void_p],
     ),
     "td_rope_table": (
         c_int32,

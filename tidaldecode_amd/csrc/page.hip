@@ -469,6 +469,45 @@ extern "C" int td_rope_table(const int32_t* positions, int32_t batch, int32_t he
   return TD_OK;
 }
 
+// One thread: the sequence grows by one token; everything a decode step's launches read about the
+// sequence is recomputed from the new length and the page table.
+__global__ void step_advance_kernel(int32_t* state, const int32_t* page_table, int32_t n_pages,
+                                    int32_t page_size, int32_t budget, const int64_t* token,
+                                    int64_t* tokens_out, int32_t tokens_cap) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  const int32_t step = state[TD_STEP_COUNT];
+  if (token && tokens_out && step < tokens_cap) tokens_out[step] = *token;
+  const int32_t n = state[TD_STEP_SEQ_LEN] + 1;
+  const int32_t pos = n - 1;
+  int32_t pi = pos / page_size;
+  pi = pi < n_pages ? pi : n_pages - 1;  // a length beyond the table cannot index past it
+  const int32_t entry = pos - (pos / page_size) * page_size;
+  const int32_t page = page_table[pi];
+  state[TD_STEP_SEQ_LEN] = n;
+  state[TD_STEP_PAGES_BEFORE_LAST] = pi;
+  state[TD_STEP_LAST_PAGE_LEN] = entry + 1;
+  state[TD_STEP_LAST_PAGE_IDX] = page;
+  state[TD_STEP_DST_SLOT] = page * page_size + entry;
+  state[TD_STEP_POSITION] = pos;
+  state[TD_STEP_N_SELECTED] = n < budget ? n : budget;
+  state[TD_STEP_COUNT] = step + 1;
+}
+
+extern "C" int td_step_advance(int32_t* state, const int32_t* page_table, int32_t n_pages,
+                               int32_t page_size, int32_t budget, const int64_t* token,
+                               int64_t* tokens_out, int32_t tokens_cap, void* stream) {
+  TD_REQUIRE(state && page_table, "td_step_advance: NULL argument");
+  TD_REQUIRE(n_pages >= 1 && page_size >= 1 && budget >= 0,
+             "td_step_advance: %d pages of %d, budget %d", n_pages, page_size, budget);
+  TD_REQUIRE((token == nullptr) == (tokens_out == nullptr) && tokens_cap >= 0,
+             "td_step_advance: token and tokens_out go together");
+  hipLaunchKernelGGL(step_advance_kernel, dim3(1), dim3(64), 0,
+                     reinterpret_cast<hipStream_t>(stream), state, page_table, n_pages, page_size,
+                     budget, token, tokens_out, tokens_cap);
+  TD_HIP_CHECK(hipGetLastError());
+  return TD_OK;
+}
+
 extern "C" int td_estimate_score(const td_paged_kv* meta, const int32_t* meta_indices,
                                  int32_t n_meta_pages, int32_t meta_last_page_len, const void* q,
                                  int32_t num_qo_heads, void* o, int64_t o_stride, void* stream) {

@@ -18,7 +18,7 @@ from typing import Optional, Tuple
 
 import torch
 
-from . import _kernels
+from . import _kernels, _lib
 from . import utils as tidal_utils
 from .utils import InferenceController
 
@@ -94,6 +94,9 @@ class TidalLlama:
         # batch-1 decode: one launch per projection with the norm / gate / residual folded in
         # (False: torch GEMMs and separate element-wise kernels, as the reference's driver)
         self.use_gemv = True
+        # set by generate_graph: the sequence's step state lives on the device and every launch of
+        # a decode step reads it there, so one captured step serves every token
+        self._dev = None
 
     # ----- cache lifecycle (tidal/models/llama.py:616-656) -----------------------------------
     def tidal_init(self, page_size: int, max_seq_len: int, token_budget: Optional[int] = None,
@@ -178,8 +181,53 @@ class TidalLlama:
         _kernels.rope_table(self._positions, self.config.head_dim, self.config.rope_scale,
                             self.config.rope_theta, self._cos, self._sin)
 
+    def _attention_dev(self, idx, q, k, v):
+        """_attention with every per-step quantity (list lengths, last page, slot and position of
+        the new token) read from the device-resident step state instead of host integers."""
+        c, ctrl, dev = self.config, self.iController, self._dev
+        st = dev["state"]
+
+        def word(i):
+            return st[i: i + 1]
+
+        fresh = None
+        if self.fuse_decode_step and ctrl.fused_step_ok:
+            fresh = (k, v, self._cos, self._sin, word(_lib.TD_STEP_DST_SLOT))
+        else:
+            _kernels.rope_append_decode(q, k, v, ctrl.kv_cache.buf_layer(idx),
+                                        word(_lib.TD_STEP_POSITION), word(_lib.TD_STEP_DST_SLOT),
+                                        ctrl.layout, c.rope_scale, c.rope_theta)
+        kind = c.layer_kind(idx)
+        o = torch.empty_like(q)
+        buf = ctrl.kv_cache.buf_layer(idx)
+        if kind == "sparse":
+            ctrl._decode_handler.forward(q, o, buf, dev["lists"], dev["list_indptr"], 0, 0, None,
+                                         index_kind="slots", n_list=dev["k"],
+                                         counts=word(_lib.TD_STEP_N_SELECTED), fresh=fresh)
+            return o
+        select = kind == "select"
+        ctrl._decode_handler.forward(q, o, buf, dev["table"].unsqueeze(0), dev["table_indptr"],
+                                     word(_lib.TD_STEP_LAST_PAGE_LEN),
+                                     word(_lib.TD_STEP_LAST_PAGE_IDX),
+                                     ctrl.qk_product if select else None,
+                                     lse=ctrl.lse if select else None,
+                                     n_list=dev["table"].numel() - 1,
+                                     counts=word(_lib.TD_STEP_PAGES_BEFORE_LAST), fresh=fresh)
+        if select:
+            scores, n = ctrl.qk_product, dev["final_len"]
+            if ctrl.select_mode != "per_head":   # columns past the current length are never ranked
+                _kernels.score_reduce(ctrl.qk_product, ctrl.lse.view(-1), ctrl.num_kv_heads, n,
+                                      ctrl.select_mode, out=ctrl.score_sum)
+                scores = ctrl.score_sum
+            _kernels.topk_filtering(scores[:, :n], None, None, dev["lists"], ctrl.topk_buf,
+                                    dev["k"], page_table=dev["table"], page_size=ctrl.page_size,
+                                    lengths=word(_lib.TD_STEP_SEQ_LEN))
+        return o
+
     def _attention(self, idx, q, k, v):
         """attention of one decode step for layer idx; q [1, H, D], k/v [1, H_kv, D] un-rotated"""
+        if self._dev is not None:
+            return self._attention_dev(idx, q, k, v)
         c, ctrl = self.config, self.iController
         fresh = None
         if self.fuse_decode_step and ctrl.fused_step_ok:
@@ -248,6 +296,73 @@ class TidalLlama:
             out.append(tok)
             logits = self.decode_step(tok)
         return torch.cat(out)
+
+    @torch.no_grad()
+    def generate_graph(self, input_ids: torch.Tensor, max_new_tokens: int,
+                       keep_logits: bool = False, use_graph: bool = True):
+        """Greedy decoding in which ONE captured decode step is replayed for every token: the
+        sequence's step state (length, last page, slot and position of the new token, list
+        length) lives on the device and is advanced by a one-thread launch inside the step, the
+        next token id never leaves the device, and pages for all tokens to come are reserved up
+        front.  No host work, copy or synchronisation between tokens.  Returns the token ids
+        (and, with ``keep_logits``, the logits that chose them: row i chose token i + 1)."""
+        c = self.config
+        logits = self.prefill(input_ids)
+        ctrl = self.iController
+        prompt_len = ctrl.kv_cache.seqlen
+        ctrl.prepare_metadata(max_new_tokens)   # pages for every token to come
+        ctrl.begin_forward(1)
+        final_len = ctrl.kv_cache.seqlen
+        table = ctrl.kv_cache.indices_device      # covers all of them already
+        k = min(int(ctrl._token_budget), final_len, ctrl.topk_dindices_buffer_full.size(1))
+        i32 = dict(dtype=torch.int32, device=self.device)
+        state = torch.zeros(_lib.TD_STEP_WORDS, **i32)
+        state[_lib.TD_STEP_SEQ_LEN] = prompt_len
+        self._dev = dict(state=state, table=table, final_len=final_len, k=k,
+                         lists=ctrl.topk_dindices_buffer_full[:, :k],
+                         list_indptr=torch.tensor([0, k], **i32),
+                         table_indptr=torch.tensor([0, table.numel()], **i32))
+        token = logits.argmax().view(1)
+        tokens = torch.zeros(max_new_tokens, dtype=torch.int64, device=self.device)
+        kept = torch.zeros((max_new_tokens, c.vocab_size), dtype=torch.float32,
+                           device=self.device) if keep_logits else None
+
+        def step():
+            _kernels.step_advance(state, table, ctrl.page_size, k, token, tokens)
+            _kernels.rope_table(state[_lib.TD_STEP_POSITION: _lib.TD_STEP_POSITION + 1], c.head_dim,
+                                c.rope_scale, c.rope_theta, self._cos, self._sin)
+            out = self.decode_layers(self.embed.index_select(0, token)).view(-1)
+            if kept is not None:
+                row = (state[_lib.TD_STEP_COUNT: _lib.TD_STEP_COUNT + 1] - 1).long()
+                kept.index_copy_(0, row, out.float().view(1, -1))
+            token.copy_(out.argmax().view(1))
+
+        try:
+            run = step
+            if use_graph:
+                # warm-up on a side stream (plans, scratch), then undo its one step on the device
+                s = torch.cuda.Stream()
+                s.wait_stream(torch.cuda.current_stream())
+                saved = (state.clone(), token.clone())
+                with torch.cuda.stream(s):
+                    step()
+                torch.cuda.current_stream().wait_stream(s)
+                torch.cuda.synchronize()
+                state.copy_(saved[0])
+                token.copy_(saved[1])
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    step()
+                run = g.replay
+            t0 = time.perf_counter()
+            for _ in range(max_new_tokens):
+                run()
+            torch.cuda.synchronize()
+            ctrl.decode_latency.append((time.perf_counter() - t0) / max(1, max_new_tokens))
+        finally:
+            self._dev = None
+            ctrl.end_forward()
+        return (tokens, kept) if keep_logits else tokens
 
     @torch.no_grad()
     def timed_decode(self, steps: int, warmup: int = 3, use_graph: bool = True) -> Tuple[float, str]:
