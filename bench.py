@@ -26,7 +26,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # HBM bytes one sparse-layer launch of the default workload moves, from rocprofv3 FETCH_SIZE /
 # WRITE_SIZE scaled by a plain 256 MiB copy (profiles/decode_attn_sparse_llama2-7b_ctx32k_top2048.md)
-TRAFFIC_DEFAULT_WORKLOAD = 35279657
+TRAFFIC_DEFAULT_WORKLOAD = 35291948
 
 
 def parse():
