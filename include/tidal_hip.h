@@ -254,6 +254,14 @@ int td_step_advance(int32_t* state, const int32_t* page_table, int32_t n_pages, 
                     void* stream);
 
 /*
+ * out[0] = index of the largest of the n values of x (dtype: td_dtype; NaN counts as largest, ties
+ * go to the lower index).  The greedy choice of the next token without leaving the device: a plain
+ * one-workgroup launch with no scratch, so that it can sit in a captured decode step.  No
+ * counterpart in the reference (its driver takes torch.argmax on the host side of each step).
+ */
+int td_argmax(const void* x, int32_t dtype, int32_t n, int64_t* out, void* stream);
+
+/*
  * Cross-head reduction of selection-layer scores: out[r, i] = sum over the query heads h of
  * row r of exp(logits[h, i] - lse[h]) (i < n), fp32.  rows = 1 (TD_REDUCE_HEAD_SUM) or
  * num_kv_heads (TD_REDUCE_GROUP_SUM).  logits is float [num_qo_heads, logits_stride].

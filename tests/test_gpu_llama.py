@@ -192,6 +192,53 @@ def test_generation_by_replaying_one_captured_step(cuda, select_mode, top_k):
     assert model._dev is None
 
 
+def test_replays_with_eager_work_in_between_and_a_large_vocabulary(cuda):
+    """A 32000-entry vocabulary (the size the token choice runs at in the benchmark) and, between
+    the replays, synchronisations and eager launches of the program's own: every replay must
+    still give what the eagerly launched step gives."""
+    from tidaldecode_amd.llama import TidalLlama
+
+    model = TidalLlama(_small(vocab_size=32000, top_k=16, num_layers=3, correction_layer=2), cuda,
+                       seed=6, init_std=0.05)
+    model.tidal_init(page_size=16, max_seq_len=128, page_order_seed=2)
+    ids = torch.randint(0, 32000, (50,), device=cuda, generator=torch.Generator(device=cuda).manual_seed(3))
+    junk = torch.randn(1 << 16, device=cuda)
+
+    def between():
+        torch.cuda.synchronize()
+        junk.mul_(1.0001).sum().item()      # eager work, a multi-block reduction and a host sync
+
+    tokens, kept = model.generate_graph(ids, 24, keep_logits=True, between_steps=between)
+    model.tidal_clear()
+    tokens_e, kept_e = model.generate_graph(ids, 24, keep_logits=True, use_graph=False)
+    assert torch.equal(tokens, tokens_e) and torch.equal(kept, kept_e)
+    assert torch.equal(tokens[1:], kept[:-1].argmax(-1))
+
+
+def test_argmax_kernel(cuda):
+    from tidaldecode_amd import _kernels
+
+    g = torch.Generator().manual_seed(1)
+    out = torch.zeros(1, dtype=torch.int64, device=cuda)
+    for dtype in (torch.float32, torch.float16, torch.bfloat16):
+        for n in (1, 63, 1000, 32000, 128256):
+            x = torch.randn(n, generator=g).to(dtype)
+            _kernels.argmax(x.to(cuda), out)
+            assert int(out) == int(x.float().argmax()), (dtype, n)   # CPU argmax: first maximum
+        x = torch.zeros(5000, dtype=dtype)
+        x[[77, 4000, 1234]] = 3.0                                     # ties: the lowest index
+        _kernels.argmax(x.to(cuda), out)
+        assert int(out) == 77
+        x[2222] = float("nan")                                        # NaN ranks highest
+        _kernels.argmax(x.to(cuda), out)
+        assert int(out) == 2222
+        x[10] = float("inf")                                          # ... on a par with +inf
+        _kernels.argmax(x.to(cuda), out)
+        assert int(out) == 10
+    with pytest.raises(RuntimeError):
+        _kernels.argmax(torch.zeros(4, device=cuda), torch.zeros(1, dtype=torch.int32, device=cuda))
+
+
 def test_step_state_words(cuda):
     from tidaldecode_amd import _kernels, _lib
 

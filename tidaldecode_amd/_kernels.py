@@ -345,6 +345,17 @@ def rope_append_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, kv_dat
                                     float(rope_theta), _stream()))
 
 
+def argmax(x: torch.Tensor, out: torch.Tensor) -> None:
+    """Extension: ``out[0]`` (int64, device) = index of the largest element of the 1-D ``x``
+    (NaN ranks highest, ties to the lower index).  One launch without scratch: graph-safe."""
+    _check_input(x, "x")
+    _check_input(out, "out")
+    if out.dtype != torch.int64 or out.numel() < 1:
+        raise RuntimeError("out must be an int64 tensor")
+    check(lib.td_argmax(x.data_ptr(), _dtype_code(x.dtype, "argmax"), x.numel(), out.data_ptr(),
+                        _stream()))
+
+
 def step_advance(state: torch.Tensor, page_table: torch.Tensor, page_size: int, budget: int,
                  token: Optional[torch.Tensor] = None,
                  tokens_out: Optional[torch.Tensor] = None) -> None:

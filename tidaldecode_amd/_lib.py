@@ -108,6 +108,7 @@ SIGNATURES = {
          c_int32, c_float, c_void_p, c_int32, c_int64, c_void_p, POINTER(FreshToken), c_void_p,
          c_int64, c_void_p],
     ),
+    "td_argmax": (c_int32, [c_void_p, c_int32, c_int32, c_void_p, c_void_p]),
     "td_step_advance": (
         c_int32,
         [c_void_p, c_void_p, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_int32, c_void_p],

@@ -469,6 +469,56 @@ extern "C" int td_rope_table(const int32_t* positions, int32_t batch, int32_t he
   return TD_OK;
 }
 
+// Index of the largest of n values (NaN counts as largest, ties go to the lower index): the
+// greedy choice of the next token, kept on the device.  One workgroup; DT: 0 f16, 1 bf16, 2 f32.
+template <int DT>
+__global__ __launch_bounds__(1024) void argmax_kernel(const void* x, int32_t n, int64_t* out) {
+  __shared__ float sv[16];
+  __shared__ int32_t si[16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float best = -INFINITY;
+  int32_t at = 0x7fffffff;
+  for (int i = tid; i < n; i += 1024) {
+    float v;
+    if constexpr (DT == 0)
+      v = to_float<F16>(reinterpret_cast<const uint16_t*>(x)[i]);
+    else if constexpr (DT == 1)
+      v = to_float<BF16>(reinterpret_cast<const uint16_t*>(x)[i]);
+    else
+      v = reinterpret_cast<const float*>(x)[i];
+    v = (v != v) ? INFINITY : v;  // NaN ranks with +inf; the lower index wins among equals
+    if (v > best || (v == best && i < at)) { best = v; at = i; }
+  }
+  for (int off = 32; off >= 1; off >>= 1) {
+    const float ov = __shfl_xor(best, off, 64);
+    const int32_t oi = __shfl_xor(at, off, 64);
+    if (ov > best || (ov == best && oi < at)) { best = ov; at = oi; }
+  }
+  if (lane == 0) { sv[wave] = best; si[wave] = at; }
+  __syncthreads();
+  if (tid == 0) {
+    for (int w = 1; w < 16; ++w)
+      if (sv[w] > best || (sv[w] == best && si[w] < at)) { best = sv[w]; at = si[w]; }
+    out[0] = at == 0x7fffffff ? 0 : at;
+  }
+}
+
+extern "C" int td_argmax(const void* x, int32_t dtype, int32_t n, int64_t* out, void* stream) {
+  TD_REQUIRE(x && out, "td_argmax: NULL argument");
+  TD_REQUIRE(n >= 1, "td_argmax: n %d < 1", n);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (dtype == TD_F16)
+    hipLaunchKernelGGL(argmax_kernel<0>, dim3(1), dim3(1024), 0, st, x, n, out);
+  else if (dtype == TD_BF16)
+    hipLaunchKernelGGL(argmax_kernel<1>, dim3(1), dim3(1024), 0, st, x, n, out);
+  else if (dtype == TD_F32)
+    hipLaunchKernelGGL(argmax_kernel<2>, dim3(1), dim3(1024), 0, st, x, n, out);
+  else
+    return fail(TD_ERR_UNSUPPORTED, "td_argmax failed to dispatch with dtype %d", dtype);
+  TD_HIP_CHECK(hipGetLastError());
+  return TD_OK;
+}
+
 // One thread: the sequence grows by one token; everything a decode step's launches read about the
 // sequence is recomputed from the new length and the page table.
 __global__ void step_advance_kernel(int32_t* state, const int32_t* page_table, int32_t n_pages,

@@ -299,13 +299,14 @@ class TidalLlama:
 
     @torch.no_grad()
     def generate_graph(self, input_ids: torch.Tensor, max_new_tokens: int,
-                       keep_logits: bool = False, use_graph: bool = True):
+                       keep_logits: bool = False, use_graph: bool = True, between_steps=None):
         """Greedy decoding in which ONE captured decode step is replayed for every token: the
         sequence's step state (length, last page, slot and position of the new token, list
         length) lives on the device and is advanced by a one-thread launch inside the step, the
         next token id never leaves the device, and pages for all tokens to come are reserved up
         front.  No host work, copy or synchronisation between tokens.  Returns the token ids
-        (and, with ``keep_logits``, the logits that chose them: row i chose token i + 1)."""
+        (and, with ``keep_logits``, the logits that chose them: row i chose token i + 1).
+        ``between_steps`` (a callable, for tests) runs on the host after every step."""
         c = self.config
         logits = self.prefill(input_ids)
         ctrl = self.iController
@@ -335,7 +336,7 @@ class TidalLlama:
             if kept is not None:
                 row = (state[_lib.TD_STEP_COUNT: _lib.TD_STEP_COUNT + 1] - 1).long()
                 kept.index_copy_(0, row, out.float().view(1, -1))
-            token.copy_(out.argmax().view(1))
+            _kernels.argmax(out, token)
 
         try:
             run = step
@@ -357,6 +358,8 @@ class TidalLlama:
             t0 = time.perf_counter()
             for _ in range(max_new_tokens):
                 run()
+                if between_steps is not None:
+                    between_steps()
             torch.cuda.synchronize()
             ctrl.decode_latency.append((time.perf_counter() - t0) / max(1, max_new_tokens))
         finally:
