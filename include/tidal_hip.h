@@ -254,6 +254,14 @@ int td_step_advance(int32_t* state, const int32_t* page_table, int32_t n_pages, 
                     void* stream);
 
 /*
+ * td_step_advance for a batch decoding in lock step: word w of sequence b is state[w * stride + b]
+ * (so every word is a contiguous [batch] array, the form the *_arr arguments take), sequence b's
+ * pages are row b of page_table [batch, table_stride].
+ */
+int td_step_advance_batch(int32_t* state, int32_t stride, int32_t batch, const int32_t* page_table,
+                          int32_t table_stride, int32_t page_size, int32_t budget, void* stream);
+
+/*
  * out[0] = index of the largest of the n values of x (dtype: td_dtype; NaN counts as largest, ties
  * go to the lower index).  The greedy choice of the next token without leaving the device: a plain
  * one-workgroup launch with no scratch, so that it can sit in a captured decode step.  No

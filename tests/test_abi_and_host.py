@@ -203,20 +203,30 @@ def test_batch_controller_bookkeeping():
     for _ in range(4):                       # 5 -> 9 tokens (third page), 9 -> 13 (fourth page)
         c.begin_step()
     assert c.seq_lens == [9, 13] and [len(p) for p in c._pages] == [3, 4]
+    from tidaldecode_amd import _lib
     meta = c._meta[:, :2].tolist()
-    assert meta[0] == [2, 3]                                 # pages before the last one
-    assert meta[1] == [1, 1]                                 # fill of the last page
-    assert meta[2] == [c._pages[0][-1], c._pages[1][-1]]     # last page id
-    assert meta[3] == [c._pages[0][-1] * 4, c._pages[1][-1] * 4]   # slot of the new token
-    assert meta[4] == [8, 12] and meta[5] == [9, 13]         # position, selected = min(budget, n)
+    assert meta[_lib.TD_STEP_SEQ_LEN] == [9, 13] and meta[_lib.TD_STEP_COUNT] == [4, 4]
+    assert meta[_lib.TD_STEP_PAGES_BEFORE_LAST] == [2, 3]
+    assert meta[_lib.TD_STEP_LAST_PAGE_LEN] == [1, 1]
+    assert meta[_lib.TD_STEP_LAST_PAGE_IDX] == [c._pages[0][-1], c._pages[1][-1]]
+    assert meta[_lib.TD_STEP_DST_SLOT] == [c._pages[0][-1] * 4, c._pages[1][-1] * 4]
+    assert meta[_lib.TD_STEP_POSITION] == [8, 12]
+    assert meta[_lib.TD_STEP_N_SELECTED] == [9, 13]          # min(budget, n)
     assert c.positions.tolist() == [8, 12] and c.selected.tolist() == [9, 13]
     for _ in range(10):
         c.begin_step()
     assert c.selected.tolist() == [16, 16]                   # the budget caps the lists
+    c.reserve_ahead(9)                       # pages beyond the one being filled change nothing
+    assert c.seq_lens == [19, 23] and [len(p) for p in c._pages] == [7, 8]
+    before = c._meta.clone()
+    c._refresh()
+    assert torch.equal(c._meta, before)
+    with pytest.raises(RuntimeError, match="max_seq_len"):
+        c.reserve_ahead(30)
     with pytest.raises(RuntimeError, match="max_batch"):
         c.add_sequences([4, 4])
     with pytest.raises(RuntimeError, match="max_seq_len"):   # a failed call keeps nothing
         c.add_sequences([41])
-    assert c.batch == 2 and c.pool.num_free_blocks == 30 - 5 - 6
+    assert c.batch == 2 and c.pool.num_free_blocks == 30 - 7 - 8
     c.release()
     assert c.batch == 0 and c.pool.num_free_blocks == 30

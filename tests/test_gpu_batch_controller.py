@@ -23,7 +23,11 @@ def _rot(x, positions, dtype, theta):
                                                     (8, 2, "per_head", torch.float16, 8),
                                                     (4, 4, "head_sum", torch.float16, 16),
                                                     (16, 4, "head_sum", torch.bfloat16, 4)])
-def test_lockstep_decode_of_a_ragged_batch(cuda, hq, hkv, mode, dtype, page):
+@pytest.mark.parametrize("stepping", ["host", "captured"])
+def test_lockstep_decode_of_a_ragged_batch(cuda, hq, hkv, mode, dtype, page, stepping):
+    """stepping = "captured": pages are reserved ahead, the whole step (metadata advance on the
+    device, RoPE table, the three layers, top-k) is captured once and replayed per token, with
+    eager copies of the step's inputs and synchronisations between the replays."""
     from oracle import tidal_oracle as orc
     from tidaldecode_amd.utils import BatchInferenceController
 
@@ -41,24 +45,73 @@ def test_lockstep_decode_of_a_ragged_batch(cuda, hq, hkv, mode, dtype, page):
         for b in range(B):
             ctl.append_prompt(b, hist_k[l][b].to(dtype).to(cuda), hist_v[l][b].to(dtype).to(cuda), l)
     rows = ctl.index_rows
+
+    def inputs(step):
+        return [tuple(randn(shape, 1000 * step + 10 * l + i, dtype)
+                      for i, shape in enumerate(((B, hq, d), (B, hkv, d), (B, hkv, d))))
+                for l in range(layers)]
+
+    def run_layers(dev_in):
+        """the device work of one step after the metadata is current; returns the three outputs"""
+        cos, sin = ctl.rope_table(1.0, theta)
+        outs = []
+        for l, (qd, kd, vd) in enumerate(dev_in):
+            if l == 0:
+                outs.append(ctl.attend_full(qd, l, True, fresh=(kd, vd, cos, sin)))
+                ctl.select()
+            elif l == 1:   # the un-fused form: RoPE + append, then attention
+                ctl.rope_append(qd, kd, vd, l, 1.0, theta)
+                outs.append(ctl.attend_sparse(qd, l))
+            else:
+                outs.append(ctl.attend_sparse(qd, l, fresh=(kd, vd, cos, sin)))
+        return outs
+
+    graph = static_in = static_out = None
+    if stepping == "captured":
+        ctl.reserve_ahead(steps)
+        static_in = [tuple(t.to(dtype).to(cuda) for t in qkv) for qkv in inputs(0)]
+
+        def body():
+            ctl.advance_on_device()
+            return run_layers(static_in)
+
+        saved = ctl._meta.clone()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            body()                       # warm-up: plans, scratch, kernel loading
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        ctl._meta.copy_(saved)           # undo the warm-up's step on the device
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static_out = body()
+
     for step in range(steps):
-        ctl.begin_step()
+        host_in = inputs(step)
+        if stepping == "captured":
+            for dst, src in zip(static_in, host_in):
+                for t_dst, t_src in zip(dst, src):
+                    t_dst.copy_(t_src.to(dtype))
+            ctl.note_step()
+            graph.replay()
+            torch.cuda.synchronize()
+            outs = static_out
+        else:
+            ctl.begin_step()
+            outs = run_layers([tuple(t.to(dtype).to(cuda) for t in qkv) for qkv in host_in])
+            torch.cuda.synchronize()
         positions = [n - 1 for n in ctl.seq_lens]
         assert ctl.positions.tolist() == positions
-        cos, sin = ctl.rope_table(1.0, theta)
         chosen = None
         for l in range(layers):
-            seed = 1000 * step + 10 * l
-            q, k, v = randn((B, hq, d), seed, dtype), randn((B, hkv, d), seed + 1, dtype), randn((B, hkv, d), seed + 2, dtype)
+            q, k, v = host_in[l]
             q_rot, k_rot = _rot(q, positions, dtype, theta), _rot(k, positions, dtype, theta)
             for b in range(B):
                 hist_k[l][b] = torch.cat([hist_k[l][b], k_rot[b: b + 1]])
                 hist_v[l][b] = torch.cat([hist_v[l][b], v[b: b + 1]])
-            qd, kd, vd = (t.to(dtype).to(cuda) for t in (q, k, v))
+            o = outs[l]
             if l == 0:
-                o = ctl.attend_full(qd, l, True, fresh=(kd, vd, cos, sin))
-                ctl.select()
-                torch.cuda.synchronize()
                 chosen = []
                 for b in range(B):
                     n = ctl.seq_lens[b]
@@ -78,12 +131,6 @@ def test_lockstep_decode_of_a_ragged_batch(cuda, hq, hkv, mode, dtype, page):
                     assert torch.equal(got_slots, want_slots), (step, b)
                     chosen.append(pos)
             else:
-                if l == 1:   # the un-fused form: RoPE + append, then attention
-                    ctl.rope_append(qd, kd, vd, l, 1.0, theta)
-                    o = ctl.attend_sparse(qd, l)
-                else:
-                    o = ctl.attend_sparse(qd, l, fresh=(kd, vd, cos, sin))
-                torch.cuda.synchronize()
                 for b in range(B):
                     want = orc.sparse_layer_gather(q_rot[b], hist_k[l][b], hist_v[l][b], chosen[b])
                     assert tolerance_report(o[b], want) <= ATOL[dtype], (step, l, b)

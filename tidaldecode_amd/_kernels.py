@@ -383,6 +383,24 @@ def step_advance(state: torch.Tensor, page_table: torch.Tensor, page_size: int, 
                               int(page_size), int(budget), tok_ptr, out_ptr, cap, _stream()))
 
 
+def step_advance_batch(state: torch.Tensor, batch: int, page_table: torch.Tensor, page_size: int,
+                       budget: int) -> None:
+    """Extension: ``step_advance`` for ``batch`` sequences in lock step.  ``state`` is int32
+    ``[TD_STEP_WORDS, stride]`` (word w of sequence b at ``state[w, b]``), ``page_table`` int32
+    ``[>= batch, pages_per_seq]`` with the pages of sequence b in row b."""
+    _check_input(state, "state")
+    _check_input(page_table, "page_table")
+    _check_i32(state, "state")
+    _check_i32(page_table, "page_table")
+    _check_dim(2, state, "state")
+    _check_dim(2, page_table, "page_table")
+    if state.size(0) < _lib.TD_STEP_WORDS or page_table.size(0) < batch:
+        raise RuntimeError("state must be [TD_STEP_WORDS, stride], page_table [batch, pages]")
+    check(lib.td_step_advance_batch(state.data_ptr(), state.size(1), int(batch),
+                                    page_table.data_ptr(), page_table.size(1), int(page_size),
+                                    int(budget), _stream()))
+
+
 def rope_table(positions: torch.Tensor, head_dim: int, rope_scale: float = 1.0,
                rope_theta: float = 1e4, cos: Optional[torch.Tensor] = None,
                sin: Optional[torch.Tensor] = None):

@@ -109,6 +109,8 @@ SIGNATURES = {
          c_int64, c_void_p],
     ),
     "td_argmax": (c_int32, [c_void_p, c_int32, c_int32, c_void_p, c_void_p]),
+    "td_step_advance_batch": (
+        c_int32, [c_void_p, c_int32, c_int32, c_void_p, c_int32, c_int32, c_int32, c_void_p]),
     "td_step_advance": (
         c_int32,
         [c_void_p, c_void_p, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_int32, c_void_p],

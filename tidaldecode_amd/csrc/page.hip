@@ -543,6 +543,45 @@ __global__ void step_advance_kernel(int32_t* state, const int32_t* page_table, i
   state[TD_STEP_COUNT] = step + 1;
 }
 
+// The same for a batch: word w of sequence b is state[w * stride + b], sequence b's pages are row
+// b of page_table.  One thread per sequence.
+__global__ void step_advance_batch_kernel(int32_t* state, int32_t stride, int32_t batch,
+                                          const int32_t* page_table, int32_t table_stride,
+                                          int32_t page_size, int32_t budget) {
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b >= batch) return;
+  int32_t* st = state + b;
+  const int32_t n = st[TD_STEP_SEQ_LEN * stride] + 1;
+  const int32_t pos = n - 1;
+  int32_t pi = pos / page_size;
+  pi = pi < table_stride ? pi : table_stride - 1;
+  const int32_t entry = pos - (pos / page_size) * page_size;
+  const int32_t page = page_table[(int64_t)b * table_stride + pi];
+  st[TD_STEP_SEQ_LEN * stride] = n;
+  st[TD_STEP_PAGES_BEFORE_LAST * stride] = pi;
+  st[TD_STEP_LAST_PAGE_LEN * stride] = entry + 1;
+  st[TD_STEP_LAST_PAGE_IDX * stride] = page;
+  st[TD_STEP_DST_SLOT * stride] = page * page_size + entry;
+  st[TD_STEP_POSITION * stride] = pos;
+  st[TD_STEP_N_SELECTED * stride] = n < budget ? n : budget;
+  st[TD_STEP_COUNT * stride] += 1;
+}
+
+extern "C" int td_step_advance_batch(int32_t* state, int32_t stride, int32_t batch,
+                                     const int32_t* page_table, int32_t table_stride,
+                                     int32_t page_size, int32_t budget, void* stream) {
+  TD_REQUIRE(state && page_table, "td_step_advance_batch: NULL argument");
+  TD_REQUIRE(batch >= 1 && stride >= batch, "td_step_advance_batch: batch %d, stride %d", batch, stride);
+  TD_REQUIRE(table_stride >= 1 && page_size >= 1 && budget >= 0,
+             "td_step_advance_batch: %d pages of %d per sequence, budget %d", table_stride, page_size,
+             budget);
+  hipLaunchKernelGGL(step_advance_batch_kernel, dim3((batch + 63) / 64), dim3(64), 0,
+                     reinterpret_cast<hipStream_t>(stream), state, stride, batch, page_table,
+                     table_stride, page_size, budget);
+  TD_HIP_CHECK(hipGetLastError());
+  return TD_OK;
+}
+
 extern "C" int td_step_advance(int32_t* state, const int32_t* page_table, int32_t n_pages,
                                int32_t page_size, int32_t budget, const int64_t* token,
                                int64_t* tokens_out, int32_t tokens_cap, void* stream) {

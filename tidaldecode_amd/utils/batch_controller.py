@@ -9,27 +9,32 @@ counterpart of ``InferenceController`` for that kernel surface:
   device tensor ``[max_batch, pages_per_seq]`` that grows in place;
 * the per-sequence metadata of a decode step (pages before the last one, fill of the last page,
   its id, the slot and the position of the new token, the number of selected tokens, the length) is one
-  ``[7, max_batch]`` int32 device tensor refreshed by a single small copy per step — never the
-  page tables themselves;
+  ``[8, max_batch]`` int32 device tensor (the words of ``td_step_advance``), refreshed by a single
+  small copy per step (``begin_step``) or, with pages reserved ahead (``reserve_ahead``), advanced
+  on the device by a one-launch ``begin_step_on_device`` — never the page tables themselves;
 * selection state for the whole batch: logits ``[B * H_q, max tokens]`` (``-inf`` where a sequence
   has no token, so that one top-k call serves ragged lengths), the log-sum-exp per head and the
   persisted token lists ``[rows, B * budget]`` with one fixed-width segment per sequence.
 
-Every attention call is ONE launch for the whole batch.  The per-step copy makes this controller
-an eager-mode one (a captured graph would replay one step's metadata); token lists are valid for
-the decode step they were selected in.
+Every attention call is ONE launch for the whole batch.  After ``reserve_ahead`` every host-side
+argument of a step's calls is an upper bound that holds for the reserved tokens and everything
+else is read on the device, so ``begin_step_on_device`` + the attention calls can be captured in a
+graph and replayed per token.  Token lists are valid for the decode step they were selected in.
 """
 from typing import List, Optional, Sequence
 
 import torch
 
-from .. import _kernels
+from .. import _kernels, _lib
 from .paged import BatchDecodeWithPagedKVCacheWrapper, KvPool, TensorLayout
 
 _SELECT_MODES = ("per_head", "group_sum", "head_sum")
-# rows of the per-step metadata tensor
-_PAGES_BEFORE_LAST, _LAST_LEN, _LAST_IDX, _DST_SLOT, _POSITION, _SELECTED, _SEQ_LEN = range(7)
-_META_ROWS = 7
+# rows of the per-step metadata tensor: the words of the device-resident step state
+_SEQ_LEN, _PAGES_BEFORE_LAST, _LAST_LEN = (_lib.TD_STEP_SEQ_LEN, _lib.TD_STEP_PAGES_BEFORE_LAST,
+                                           _lib.TD_STEP_LAST_PAGE_LEN)
+_LAST_IDX, _DST_SLOT, _POSITION = (_lib.TD_STEP_LAST_PAGE_IDX, _lib.TD_STEP_DST_SLOT,
+                                   _lib.TD_STEP_POSITION)
+_SELECTED, _STEPS, _META_ROWS = _lib.TD_STEP_N_SELECTED, _lib.TD_STEP_COUNT, _lib.TD_STEP_WORDS
 
 
 class BatchInferenceController:
@@ -57,6 +62,7 @@ class BatchInferenceController:
         self.page_table = torch.zeros((max_batch, self.pages_per_seq), **i32)
         self._pages: List[List[int]] = []
         self.seq_lens: List[int] = []
+        self._cap: List[int] = []   # tokens each sequence has pages for (>= its length)
         self._meta = torch.zeros((_META_ROWS, max_batch), **i32)
         # staging for the per-step copy: a small ring of pinned rows, so that the copy is
         # asynchronous and a buffer is only rewritten after its copy has completed
@@ -65,6 +71,7 @@ class BatchInferenceController:
                        for _ in range(4)]
         self._stage_done = [None] * len(self._stage)
         self._stage_next = 0
+        self._steps = 0
         self._table_starts = torch.arange(max_batch + 1, **i32) * self.pages_per_seq
 
         self.score_cols = self.pages_per_seq * page_size
@@ -96,17 +103,30 @@ class BatchInferenceController:
     def buf_layer(self, layer_idx: int) -> torch.Tensor:
         return self.pool.buf[layer_idx % self.pool.num_layers]
 
-    def _reserve(self, b: int, n_tokens: int) -> None:
-        have = len(self._pages[b])
-        total = self.seq_lens[b] + n_tokens
+    def _ensure_pages(self, b: int, total: int) -> None:
+        """pages for `total` tokens of sequence b"""
         if total > self.max_seq_len:
             raise RuntimeError(f"sequence {b} would hold {total} tokens, max_seq_len is {self.max_seq_len}")
+        have = len(self._pages[b])
         grow = -(-total // self.page_size) - have
         if grow > 0:
             fresh = self.pool.take(grow)
             self.page_table[b, have: have + grow] = torch.tensor(fresh, dtype=torch.int32)
             self._pages[b] += fresh
-        self.seq_lens[b] = total
+        self._cap[b] = max(self._cap[b], total)
+
+    def _reserve(self, b: int, n_tokens: int) -> None:
+        self._ensure_pages(b, self.seq_lens[b] + n_tokens)
+        self.seq_lens[b] += n_tokens
+
+    def reserve_ahead(self, n_tokens: int) -> None:
+        """Pages for the next ``n_tokens`` decode steps of every sequence, so that those steps
+        need nothing from the host (``begin_step_on_device``)."""
+        over = [b for b, n in enumerate(self.seq_lens) if n + int(n_tokens) > self.max_seq_len]
+        if over:
+            raise RuntimeError(f"sequences {over} would exceed max_seq_len = {self.max_seq_len}")
+        for b in range(self.batch):
+            self._ensure_pages(b, self.seq_lens[b] + int(n_tokens))
 
     def add_sequences(self, lengths: Sequence[int]) -> None:
         """Open one sequence per entry with room for that many prompt tokens."""
@@ -119,11 +139,12 @@ class BatchInferenceController:
             for n in lengths:
                 self._pages.append([])
                 self.seq_lens.append(0)
+                self._cap.append(0)
                 self._reserve(self.batch - 1, int(n))
         except Exception:
             for pages in self._pages[opened:]:   # leave the controller as it was
                 self.pool.give_back(pages)
-            del self._pages[opened:], self.seq_lens[opened:]
+            del self._pages[opened:], self.seq_lens[opened:], self._cap[opened:]
             raise
         self._refresh()
 
@@ -131,7 +152,7 @@ class BatchInferenceController:
         """Close every sequence and return its pages."""
         for pages in self._pages:
             self.pool.give_back(pages)
-        self._pages, self.seq_lens = [], []
+        self._pages, self.seq_lens, self._cap = [], [], []
         self.qk_product.fill_(float("-inf"))
 
     def _refresh(self) -> None:
@@ -139,10 +160,13 @@ class BatchInferenceController:
         P = self.page_size
         cols = []
         for b, n in enumerate(self.seq_lens):
-            pages = self._pages[b]
-            last_len = (n - 1) % P + 1
-            cols.append((len(pages) - 1, last_len, pages[-1], pages[-1] * P + last_len - 1, n - 1,
-                         min(self.budget, n), n))
+            before, entry = divmod(n - 1, P)
+            page = self._pages[b][before]   # pages may be reserved beyond the one being filled
+            row = [0] * _META_ROWS
+            row[_SEQ_LEN], row[_PAGES_BEFORE_LAST], row[_LAST_LEN] = n, before, entry + 1
+            row[_LAST_IDX], row[_DST_SLOT], row[_POSITION] = page, page * P + entry, n - 1
+            row[_SELECTED], row[_STEPS] = min(self.budget, n), self._steps
+            cols.append(tuple(row))
         cols += [(0,) * _META_ROWS] * (self.max_batch - len(cols))
         i = self._stage_next
         self._stage_next = (i + 1) % len(self._stage)
@@ -162,7 +186,30 @@ class BatchInferenceController:
             raise RuntimeError(f"sequences {full} already hold max_seq_len = {self.max_seq_len} tokens")
         for b in range(self.batch):
             self._reserve(b, 1)
+        self._steps += 1
         self._refresh()
+
+    def advance_on_device(self) -> None:
+        """The device half of ``begin_step_on_device``: one launch recomputes every sequence's
+        metadata for one more token from the page tables.  This is the call to capture."""
+        _kernels.step_advance_batch(self._meta, self.batch, self.page_table, self.page_size,
+                                    self.budget)
+
+    def note_step(self) -> None:
+        """The host half: the mirrors of the lengths move on by one token (call it before every
+        replay of a captured step).  The pages must have been reserved (``reserve_ahead``)."""
+        short = [b for b, n in enumerate(self.seq_lens) if n + 1 > self._cap[b]]
+        if short:
+            raise RuntimeError(f"sequences {short} have no page reserved for another token; call "
+                               "reserve_ahead first")
+        for b in range(self.batch):
+            self.seq_lens[b] += 1
+        self._steps += 1
+
+    def begin_step_on_device(self) -> None:
+        """``begin_step`` without host data: nothing is copied, one launch advances the metadata."""
+        self.note_step()
+        self.advance_on_device()
 
     # views of the step's metadata, all int32 device [B]
     def _row(self, r: int) -> torch.Tensor:
@@ -220,7 +267,7 @@ class BatchInferenceController:
             self._table_starts[: B + 1], self._row(_LAST_LEN), self._row(_LAST_IDX),
             self.qk_product[: B * self.num_heads] if output_qk_product else None,
             lse=self.lse[:B] if output_qk_product else None,
-            n_list=max(len(p) for p in self._pages) - 1, counts=self._row(_PAGES_BEFORE_LAST),
+            n_list=-(-max(self._cap) // self.page_size) - 1, counts=self._row(_PAGES_BEFORE_LAST),
             fresh=self._fresh(fresh))
         return o
 
@@ -228,7 +275,7 @@ class BatchInferenceController:
         """Top-k of the last ``attend_full(..., output_qk_product=True)`` for every sequence:
         physical token slots, sorted by position, in its segment of ``topk_dindices_buffer``."""
         B, P, k = self.batch, self.page_size, self.budget
-        n = max(self.seq_lens)
+        n = max(self._cap)   # an upper bound; every sequence's own length is read on the device
         rows = self.index_rows
         scores = self.qk_product[: B * self.num_heads]
         if self.select_mode != "per_head":
@@ -252,6 +299,6 @@ class BatchInferenceController:
         o = torch.empty_like(q)
         self._handle.forward(q, o, self.buf_layer(layer_idx), self.topk_dindices_buffer,
                              self._list_starts[: B + 1], 0, 0, None, index_kind="slots",
-                             n_list=min(self.budget, max(self.seq_lens)), counts=self.selected,
+                             n_list=min(self.budget, max(self._cap)), counts=self.selected,
                              fresh=self._fresh(fresh))
         return o
