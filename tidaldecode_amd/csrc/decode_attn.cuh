@@ -553,9 +553,22 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
 #pragma unroll
       for (int u = 0; u < U; ++u)
         pr[u] = (base + u * TPI + g < c1) ? fast_exp2(sv[u] - m_new) : 0.f;
-      // the probabilities enter the matrix product rounded to the KV type (zero-mean rounding of
-      // weights in [0, 1]); the denominator, which also gives the log-sum-exp, stays in fp32
+      // The probabilities enter the matrix product in the KV type; the denominator, which also
+      // gives the log-sum-exp, stays in fp32.  bf16 keeps 8 bits of a weight: against an exact
+      // denominator that is an error of 2^-9 |v| in o, which with few selected tokens and |v| of
+      // 3-4 reached the bf16 tolerance together with the rounding of o itself.  bf16 weights are
+      // therefore split into a rounded part and the (rounded) remainder, two products instead of
+      // one: 16 good bits, and the matrix pipeline has the room.  fp16 weights (11 bits) go in once.
       const uint32_t p01 = pack2<T>(pr[0], pr[1]), p23 = pack2<T>(pr[2], pr[3]);
+      constexpr bool kSplitP = std::is_same<T, BF16>::value;
+      uint32_t e01 = 0, e23 = 0;
+      if constexpr (kSplitP) {
+        float r0, r1, r2, r3;
+        unpack2<T>(p01, r0, r1);
+        unpack2<T>(p23, r2, r3);
+        e01 = pack2<T>(pr[0] - r0, pr[1] - r1);
+        e23 = pack2<T>(pr[2] - r2, pr[3] - r3);
+      }
       lh = fmaf(lh, alpha, (pr[0] + pr[1]) + (pr[2] + pr[3]));
       // rescale the accumulators: row 4g + i belongs to head (4g + i) % QPG; the factors are
       // wave-uniform per head (lane x < QPG holds head x), so they travel through SGPRs
@@ -593,6 +606,10 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
         const uint32_t hi1 = __builtin_amdgcn_perm(vw[3][c], vw[2][c], 0x07060302u);
         accm[2 * c] = mfma_16x16x16<T>(p01, p23, lo0, lo1, accm[2 * c]);
         accm[2 * c + 1] = mfma_16x16x16<T>(p01, p23, hi0, hi1, accm[2 * c + 1]);
+        if constexpr (kSplitP) {
+          accm[2 * c] = mfma_16x16x16<T>(e01, e23, lo0, lo1, accm[2 * c]);
+          accm[2 * c + 1] = mfma_16x16x16<T>(e01, e23, hi0, hi1, accm[2 * c + 1]);
+        }
       }
       return;
     }
