@@ -554,13 +554,13 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
       for (int u = 0; u < U; ++u)
         pr[u] = (base + u * TPI + g < c1) ? fast_exp2(sv[u] - m_new) : 0.f;
       // The probabilities enter the matrix product in the KV type; the denominator, which also
-      // gives the log-sum-exp, stays in fp32.  bf16 keeps 8 bits of a weight: against an exact
-      // denominator that is an error of 2^-9 |v| in o, which with few selected tokens and |v| of
-      // 3-4 reached the bf16 tolerance together with the rounding of o itself.  bf16 weights are
-      // therefore split into a rounded part and the (rounded) remainder, two products instead of
-      // one: 16 good bits, and the matrix pipeline has the room.  fp16 weights (11 bits) go in once.
+      // gives the log-sum-exp, stays in fp32.  bf16 keeps 8 bits of a weight (fp16 11): against an
+      // exact denominator that is an error of 2^-9 |v| (2^-12 |v|) in o, which with few selected
+      // tokens and |v| of 3-4 reached the tolerance together with the rounding of o itself.  The
+      // weights are therefore split into a rounded part and the (rounded) remainder, two products
+      // instead of one: twice the bits, and the matrix pipeline has the room.
       const uint32_t p01 = pack2<T>(pr[0], pr[1]), p23 = pack2<T>(pr[2], pr[3]);
-      constexpr bool kSplitP = std::is_same<T, BF16>::value;
+      constexpr bool kSplitP = true;
       uint32_t e01 = 0, e23 = 0;
       if constexpr (kSplitP) {
         float r0, r1, r2, r3;
