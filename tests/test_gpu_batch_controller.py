@@ -25,15 +25,26 @@ def _rot(x, positions, dtype, theta):
                                                     (16, 4, "head_sum", torch.bfloat16, 4)])
 @pytest.mark.parametrize("stepping", ["host", "captured"])
 def test_lockstep_decode_of_a_ragged_batch(cuda, hq, hkv, mode, dtype, page, stepping):
+    _lockstep(cuda, hq, hkv, mode, dtype, page, stepping, [5, 130, 47, 64], 48, 20)
+
+
+@pytest.mark.parametrize("stepping", ["host", "captured"])
+@pytest.mark.parametrize("lens,budget,steps", [([1, 16, 17, 200, 31], 8, 18),     # from one token on
+                                               ([200], 1000, 5),                   # budget above the length
+                                               ([3, 3, 3, 3, 3, 3, 3, 90], 33, 35)])
+def test_lockstep_decode_other_shapes(cuda, lens, budget, steps, stepping):
+    _lockstep(cuda, 12, 4, "group_sum", torch.bfloat16, 8, stepping, lens, budget, steps)
+    _lockstep(cuda, 4, 4, "per_head", torch.float16, 16, stepping, lens, budget, steps)
+
+
+def _lockstep(cuda, hq, hkv, mode, dtype, page, stepping, lens, budget, steps):
     """stepping = "captured": pages are reserved ahead, the whole step (metadata advance on the
     device, RoPE table, the three layers, top-k) is captured once and replayed per token, with
     eager copies of the step's inputs and synchronisations between the replays."""
     from oracle import tidal_oracle as orc
     from tidaldecode_amd.utils import BatchInferenceController
 
-    d, layers, budget, theta = 128, 3, 48, 1e4
-    lens = [5, 130, 47, 64]
-    steps = 20
+    d, layers, theta = 128, 3, 1e4
     B = len(lens)
     ctl = BatchInferenceController(layers, hq, d, page, budget, 256, B + 1, dtype, cuda,
                                    num_kv_heads=hkv, select_mode=mode, page_order_seed=3)
