@@ -192,6 +192,31 @@ def test_generation_by_replaying_one_captured_step(cuda, select_mode, top_k):
     assert model._dev is None
 
 
+@pytest.mark.parametrize("heads,kv,hd,page,mode,gemv", [(8, 2, 128, 5, "group_sum", True),    # un-fused step
+                                                         (6, 2, 128, 16, "head_sum", False),  # padded group
+                                                         (2, 1, 256, 1, "per_head", True)])
+def test_replayed_generation_on_other_shapes(cuda, heads, kv, hd, page, mode, gemv):
+    """Page sizes without a fused step (RoPE + append as their own launch, positions and slots
+    read from the device state), shared-row and padded query groups, head_dim 256."""
+    from tidaldecode_amd.llama import TidalLlama
+
+    cfg = _small(num_heads=heads, num_kv_heads=kv, head_dim=hd, select_mode=mode, top_k=10)
+    model = TidalLlama(cfg, cuda, seed=4, init_std=0.05)
+    model.use_gemv = gemv
+    model.tidal_init(page_size=page, max_seq_len=160, page_order_seed=5)
+    ids = torch.randint(0, 1000, (50,), device=cuda, generator=torch.Generator(device=cuda).manual_seed(9))
+    tokens, kept = model.generate_graph(ids, 30, keep_logits=True)
+    model.tidal_clear()
+    tokens_e, kept_e = model.generate_graph(ids, 30, keep_logits=True, use_graph=False)
+    assert torch.equal(tokens, tokens_e) and torch.equal(kept, kept_e)
+    model.tidal_clear()
+    logits = model.prefill(ids)
+    assert int(logits.argmax()) == int(tokens[0])
+    for i in range(30):
+        logits = model.decode_step(tokens[i: i + 1])
+        assert _close(kept[i], logits.float(), rel=1.5e-1), i
+
+
 def test_replays_with_eager_work_in_between_and_a_large_vocabulary(cuda):
     """A 32000-entry vocabulary (the size the token choice runs at in the benchmark) and, between
     the replays, synchronisations and eager launches of the program's own: every replay must
