@@ -103,3 +103,50 @@ def test_list_of_every_token_equals_full_attention(cuda):
     want = orc.softmax_pv(orc.attn_logits(q, case.k), case.v)
     assert tolerance_report(o_full[0], want) <= ATOL[dtype]
     assert tolerance_report(o_all[0], want) <= ATOL[dtype]
+
+
+def test_ragged_batch_of_eight_at_full_size(cuda):
+    """cfg3: 8 sequences of randint(8192, 65537) tokens (seed 0), fp16, 32 heads x 128, page 16,
+    1024 tokens selected per sequence and head — one launch for the batch per piece (selection layer
+    with logits, top-k of all 256 rows, sparse layer) through BatchInferenceController.  The pool
+    (8.6 GB) is filled on the device; the oracle checks the shortest and the longest sequence from
+    their own pages, and every sequence through properties that do not need its K/V on the host:
+    lists sorted by position, duplicate-free, inside the sequence, and equal to the oracle's
+    selection from the logits the GPU wrote."""
+    from oracle import tidal_oracle as orc
+    from tidaldecode_amd.utils import BatchInferenceController
+
+    dtype, h, d, page, k = torch.float16, 32, 128, 16, 1024
+    lens = torch.randint(8192, 65537, (8,), generator=torch.Generator().manual_seed(0)).tolist()
+    ctl = BatchInferenceController(1, h, d, page, k, max(lens) + 64, 8, dtype, cuda, page_order_seed=0)
+    ctl.add_sequences(lens)
+    ctl.pool.buf.normal_()
+    ctl.begin_step()
+    q = randn((8, h, d), 3, dtype)
+    qd = q.to(dtype).to(cuda)
+    o_full = ctl.attend_full(qd, 0, True)
+    ctl.select()
+    o_sparse = ctl.attend_sparse(qd, 0)
+    torch.cuda.synchronize()
+    order = sorted(range(8), key=lambda b: ctl.seq_lens[b])
+    for b in range(8):
+        n = ctl.seq_lens[b]
+        table = torch.tensor(ctl._pages[b])
+        logits_gpu = ctl.qk_product[b * h: (b + 1) * h, :n].cpu()
+        slots = ctl.topk_dindices_buffer[:, b * k: (b + 1) * k].cpu().long()
+        inv = torch.full((int(table.max()) + 1,), -1, dtype=torch.long)
+        inv[table] = torch.arange(table.numel())
+        pos = inv[slots // page] * page + slots % page
+        assert (inv[slots // page] >= 0).all() and (pos < n).all(), b
+        assert (pos[:, 1:] > pos[:, :-1]).all(), b                     # sorted, no duplicates
+        assert torch.equal(pos, orc.stable_topk(logits_gpu, k)), b
+        assert torch.isinf(ctl.qk_product[b * h: (b + 1) * h, n:]).all(), b
+        if b in (order[0], order[-1]):
+            pages = ctl.buf_layer(0)[table.to(cuda)]                   # [pages, 2, P, H, D]
+            kk = pages[:, 0].reshape(-1, h, d)[:n].float().cpu()
+            vv = pages[:, 1].reshape(-1, h, d)[:n].float().cpu()
+            logits = orc.attn_logits(q[b], kk)
+            assert (logits_gpu - logits).abs().max() <= 2e-4 * max(1.0, logits.abs().max().item()), b
+            assert tolerance_report(o_full[b], orc.softmax_pv(logits, vv)) <= ATOL[dtype], b
+            assert tolerance_report(o_sparse[b], orc.sparse_layer_gather(q[b], kk, vv, pos)) <= ATOL[dtype], b
+    ctl.release()
