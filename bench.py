@@ -278,6 +278,10 @@ def cpu_baseline(args, budget_s=12.0):
                   f"sparse layer at ctx {n}, top_k {k}, 32 heads x 128, fp32, torch-CPU; median; selection layer "
                   f"{statistics.median(sel_t) * 1e6:.0f} us",
         "selection_us_per_layer": round(statistics.median(sel_t) * 1e6, 1),
+        # the step of the benchmarked schedule, scaled from the two layer kinds: 2 selection
+        # layers + (layers - 2) sparse layers (the reference's CPU path does O(N) work in both)
+        "attention_path_ms_per_step_scaled": round(
+            (2 * statistics.median(sel_t) + (args.layers - 2) * statistics.median(sp_t)) * 1e3, 2),
         "configs0_selection_plus_sparse_us": round(statistics.median(c0) * 1e6, 1),
         "gather_variant_us_per_layer": round(statistics.median(ga_t) * 1e6, 1),
         "gather_variant_note": "index_select of the selected rows, then attention over them: not "
