@@ -356,7 +356,10 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
   // hsel = li % QPG; the running maximum mh of a head is kept equal in all lanes of the wave, lh
   // is the lane group's share of the denominator, and p.V runs on the matrix cores with the 16
   // tokens of a tile as the inner dimension: accm[dd][i] = o[head (4g + i) % QPG][li * 8 + dd].
-  static_assert(QPG == 1 || (U == 4 && TPI == 4), "shared-row tiles are 16 tokens: 4 rows x 4 groups");
+  // MMA: that path, for head_dim 128 (rows of 16 lanes, tiles of 16 tokens: 4 rows x 4 groups).
+  // Other head sizes score their QPG query heads per loaded KV row on the vector ALU throughout.
+  constexpr bool MMA = QPG > 1 && LPR == 16;
+  static_assert(!MMA || (U == 4 && TPI == 4), "shared-row tiles are 16 tokens: 4 rows x 4 groups");
   float mh = kNegBig, lh = 0.f;
   f32x4 accm[8];
 #pragma unroll
@@ -510,7 +513,7 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
         }
       }
     }
-    if constexpr (QPG > 1) {
+    if constexpr (MMA) {
       float sv[U], xe[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
@@ -633,10 +636,14 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
       // row li (token base + li TPI + g) and nothing moves between lanes; the logits wait in the
       // wave's LDS strip and leave in batches (see emit_flush)
       static_assert(U <= LPR, "one lane of the group per row of the tile");
-      float e = sc[0][0];
 #pragma unroll
-      for (int u = 1; u < U; ++u) e = (li == u) ? sc[0][u] : e;
-      if (li < U) emit_buf[(wave * EMIT_TILES + emit_n) * TILE + li * TPI + g] = e * kLn2;
+      for (int j = 0; j < QPG; ++j) {  // strip layout [tile][head][token]
+        float e = sc[j][0];
+#pragma unroll
+        for (int u = 1; u < U; ++u) e = (li == u) ? sc[j][u] : e;
+        if (li < U)
+          emit_buf[((wave * EMIT_TILES + emit_n) * QPG + j) * TILE + li * TPI + g] = e * kLn2;
+      }
       emit_push(base);
     }
 #pragma unroll
@@ -704,12 +711,12 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
   emit_flush();
 
   // ---- combine the TPI token slots of the wave (butterfly over lane groups) ---------------------
-  if constexpr (QPG > 1) {  // the matrix product already summed the groups; only lh is per group
+  if constexpr (MMA) {  // the matrix product already summed the groups; only lh is per group
     lh += __shfl_xor(lh, 16, 64);
     lh += __shfl_xor(lh, 32, 64);
   }
 #pragma unroll
-  for (int j = 0; j < (QPG > 1 ? 0 : QPG); ++j) {
+  for (int j = 0; j < (MMA ? 0 : QPG); ++j) {
     float mw = m[j];
 #pragma unroll
     for (int off = LPR; off < 64; off <<= 1) mw = fmaxf(mw, __shfl_xor(mw, off, 64));
@@ -732,7 +739,7 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
   __shared__ float sm_o[QPG][NW][8][LPR];
   __shared__ float sm_ml[QPG][NW][2];
   __shared__ int sm_ticket;
-  if constexpr (QPG > 1) {
+  if constexpr (MMA) {
 #pragma unroll
     for (int j = 0; j < QPG; ++j) {  // head j is row j of the accumulator tile: group j / 4, i = j % 4
       if (g == j / 4) {
@@ -829,13 +836,15 @@ __global__ __launch_bounds__(NT) void merge_partials_kernel(const DecodeParams p
 
 // Instantiated shapes (tile_rows = K/V load instructions per wave tile):
 //   one query head per head row: head_dim 64/128/256, 8 waves x {2, 4} rows or 16 waves x 4 rows;
-//   2, 4 or 8 query heads per head row (KV rows shared inside a GQA group): head_dim 128,
-//   8 waves x 4 rows.
+//   2, 4 or 8 query heads per head row (KV rows shared inside a GQA group): head_dim 64 and 128
+//   (256: 2 or 4), 8 waves x 4 rows; head_dim 128 on the matrix cores, the others on the vector ALU.
 static bool shape_supported(int head_dim, int qpg, int nw, int rows = 4) {
   if (qpg == 1)
     return (head_dim == 64 || head_dim == 128 || head_dim == 256) &&
            ((nw == 8 && (rows == 2 || rows == 4)) || (nw == 16 && rows == 4));
-  return head_dim == 128 && (qpg == 2 || qpg == 4 || qpg == 8) && nw == 8 && rows == 4;
+  if (nw != 8 || rows != 4) return false;
+  if (head_dim == 256) return qpg == 2 || qpg == 4;  // the split merge holds qpg * head_dim <= 1024
+  return (head_dim == 64 || head_dim == 128) && (qpg == 2 || qpg == 4 || qpg == 8);
 }
 
 // Query heads scored per loaded KV row.  KV rows are shared between the query heads of a GQA
@@ -845,9 +854,10 @@ static int qpg_for(int num_qo_heads, int num_kv_heads, int idx_rows, int head_di
   const int group = num_qo_heads / num_kv_heads;
   if (group <= 1 || idx_rows == num_qo_heads) return 1;
   // groups of 3 run on the 4-head kernel, 5 to 7 on the 8-head kernel, larger ones as several head
-  // rows of 8: the padding heads cost arithmetic, not memory traffic, which is what bounds these
-  // kernels
-  const int padded = group <= 2 ? 2 : (group <= 4 ? 4 : 8);
+  // rows of 8 (of 4 for head_dim 256): the padding heads cost arithmetic, not memory traffic,
+  // which is what bounds these kernels
+  int padded = group <= 2 ? 2 : (group <= 4 ? 4 : 8);
+  if (head_dim == 256 && padded > 4) padded = 4;
   return shape_supported(head_dim, padded, 8) ? padded : 1;
 }
 
@@ -903,11 +913,16 @@ static int launch_shape(const DecodeParams& p, int head_dim, int qpg, int nw, in
   TD_CASE(128, 2, 8, 4)
   TD_CASE(128, 4, 8, 4)
   TD_CASE(128, 8, 8, 4)
+  TD_CASE(64, 2, 8, 4)
+  TD_CASE(64, 4, 8, 4)
+  TD_CASE(64, 8, 8, 4)
+  TD_CASE(256, 2, 8, 4)
+  TD_CASE(256, 4, 8, 4)
 #undef TD_CASE
   return fail(TD_ERR_UNSUPPORTED,
               "BatchDecodeWithPagedKVCache failed to dispatch: head_dim %d with %d query heads per "
               "shared KV row and %d waves (supported: head_dim 64/128/256 with per-head lists; "
-              "head_dim 128 with shared lists and group size 2, 4 or 8)",
+              "shared lists with 2, 4 or 8 heads per row, 2 or 4 for head_dim 256)",
               head_dim, qpg, nw);
 }
 
