@@ -194,7 +194,9 @@ def test_generation_by_replaying_one_captured_step(cuda, select_mode, top_k):
 
 @pytest.mark.parametrize("heads,kv,hd,page,mode,gemv", [(8, 2, 128, 5, "group_sum", True),    # un-fused step
                                                          (6, 2, 128, 16, "head_sum", False),  # padded group
-                                                         (2, 1, 256, 1, "per_head", True)])
+                                                         (2, 1, 256, 1, "per_head", True),
+                                                         (8, 2, 64, 16, "group_sum", True),   # shared rows, head_dim 64
+                                                         (6, 2, 256, 16, "head_sum", True)])  # padded group, head_dim 256
 def test_replayed_generation_on_other_shapes(cuda, heads, kv, hd, page, mode, gemv):
     """Page sizes without a fused step (RoPE + append as their own launch, positions and slots
     read from the device state), shared-row and padded query groups, head_dim 256."""
