@@ -473,7 +473,7 @@ def test_padded_query_groups(cuda, hq, hkv, fused_merge):
 
 
 @pytest.mark.parametrize("hq,hkv,d", [(4, 4, 128), (8, 2, 128), (4, 2, 128), (8, 1, 128), (2, 2, 64),
-                                      (2, 2, 256)])
+                                      (2, 2, 256), (8, 2, 64), (16, 2, 64), (8, 2, 256), (6, 2, 256)])
 def test_logits_of_long_wave_runs(cuda, hq, hkv, d):
     """One split for the whole sequence: every wave walks hundreds of tiles, so the logits leave
     the per-wave staging strip several times in mid-loop (and once more, partly filled, at the
