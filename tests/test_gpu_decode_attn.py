@@ -430,16 +430,19 @@ def test_random_configurations(cuda, seed):
 
 
 @pytest.mark.parametrize("fused_merge", [1, 0])
-@pytest.mark.parametrize("hq,hkv", [(6, 2), (12, 4), (10, 2), (12, 2), (28, 4), (7, 1),
-                                    (32, 2), (24, 2), (32, 1), (18, 2)])
-def test_padded_query_groups(cuda, hq, hkv, fused_merge):
+@pytest.mark.parametrize("hq,hkv,d", [(6, 2, 128), (12, 4, 128), (10, 2, 128), (12, 2, 128), (28, 4, 128),
+                                      (7, 1, 128), (32, 2, 128), (24, 2, 128), (32, 1, 128), (18, 2, 128),
+                                      # head_dim 64 / 256: shared rows on the vector ALU
+                                      (8, 2, 64), (6, 2, 64), (32, 2, 64), (14, 2, 64),
+                                      (8, 2, 256), (6, 2, 256), (10, 2, 256), (4, 2, 256)])
+def test_padded_query_groups(cuda, hq, hkv, d, fused_merge):
     """Groups of 3, 5, 6 and 7 query heads per KV head run on the 4- and 8-head shared-row kernels
     with padding heads, larger groups (16, 12, 32, 9) as several head rows of 8: outputs, logits and log-sum-exps of the real heads must be those of the
     oracle, nothing may be written for the padding, on one split and on many, with the in-kernel
     and the second-kernel merge."""
     from oracle import tidal_oracle as orc
 
-    d, page_size, dtype = 128, 16, torch.bfloat16
+    page_size, dtype = 16, torch.bfloat16
     for n, k in ((40, 33), (5000, 1500)):
         case = PagedCase(n, hkv, d, page_size, dtype, seed=hq * n)
         q = randn((hq, d), hq + n, dtype)
