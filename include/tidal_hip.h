@@ -254,6 +254,19 @@ int td_step_advance(int32_t* state, const int32_t* page_table, int32_t n_pages, 
                     void* stream);
 
 /*
+ * Merge of attention states over disjoint token subsets: o_parts [n_parts, rows, head_dim] (dtype:
+ * td_dtype, also the type of o) are the attention outputs of the parts, lse_parts [n_parts, rows]
+ * the natural-log sums of exponentials of their logits (as td_decode_attn writes to `lse`);
+ * o [rows, head_dim] = sum_i o_i e^(lse_i - lse), lse [rows] (optional) = log sum_i e^(lse_i).  A
+ * part with lse = -inf is empty and ignored.  The stand-alone form of the split merge that
+ * td_decode_attn runs inside its launch; replaces VariableLengthMergeStates of the reference's
+ * FlashInfer dependency (call site kernels/include/decode/decode_attn.cuh:1011-1020) for callers
+ * that split a sequence themselves, e.g. across devices.
+ */
+int td_merge_states(const void* o_parts, int32_t dtype, const float* lse_parts, int32_t n_parts,
+                    int32_t rows, int32_t head_dim, void* o, float* lse, void* stream);
+
+/*
  * td_step_advance for a batch decoding in lock step: word w of sequence b is state[w * stride + b]
  * (so every word is a contiguous [batch] array, the form the *_arr arguments take), sequence b's
  * pages are row b of page_table [batch, table_stride].

@@ -505,3 +505,48 @@ def test_logits_of_long_wave_runs(cuda, hq, hkv, d):
         assert tolerance_report(od[0], want) <= ATOL[dtype], knobs
         assert (scores[:, :n].cpu() - logits).abs().max() <= 2e-4 * max(1.0, logits.abs().max().item())
         assert torch.isnan(scores[:, n:]).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n_parts", [1, 2, 7, 32])
+def test_merge_states_of_any_partition_is_the_unsplit_result(cuda, dtype, n_parts):
+    """td_merge_states: the tokens of a sequence are dealt into n_parts random subsets (one left
+    empty on purpose when there are several), each attended to on its own with its log-sum-exp;
+    merged, they must give the attention over all tokens — against the oracle, and against the
+    closed form o = sum o_i e^(lse_i - lse) evaluated on the host from the same parts."""
+    from oracle import tidal_oracle as orc
+    from tidaldecode_amd import _kernels
+
+    hq, hkv, d, page_size, n = 8, 2, 128, 16, 3000
+    case = PagedCase(n, hkv, d, page_size, dtype, seed=n_parts)
+    q = randn((hq, d), 5, dtype)
+    qd = q.to(dtype).to(cuda).unsqueeze(0)
+    pool = case.pool.to(cuda)
+    g = torch.Generator().manual_seed(n_parts)
+    owner = torch.randint(0, max(1, n_parts - 1) if n_parts > 2 else n_parts, (n,), generator=g)
+    w = _wrapper(0, hq, hkv, d, page_size, dtype)
+    o_parts = torch.full((n_parts, 1, hq, d), float("nan"), dtype=dtype, device=cuda)
+    lse_parts = torch.full((n_parts, 1, hq), float("-inf"), dtype=torch.float32, device=cuda)
+    for i in range(n_parts):
+        pos = (owner == i).nonzero().flatten()
+        if pos.numel() == 0:
+            continue                      # an empty part: lse stays -inf, o stays NaN
+        slots = case.slots_of(pos).to(torch.int32).unsqueeze(0).to(cuda)
+        w.forward(qd, o_parts[i], pool, slots, None, 0, 0, None, index_kind="slots",
+                  lse=lse_parts[i])
+    o, lse = _kernels.merge_states(o_parts, lse_parts)
+    torch.cuda.synchronize()
+    logits = orc.attn_logits(q, case.k)
+    assert tolerance_report(o[0], orc.softmax_pv(logits, case.v)) <= ATOL[dtype]
+    assert (lse[0].cpu() - torch.logsumexp(logits, -1)).abs().max() <= 1e-3
+    # closed form on the host from the same parts
+    lp, op = lse_parts.cpu()[:, 0], torch.nan_to_num(o_parts.float().cpu()[:, 0])
+    tot = torch.logsumexp(lp, 0)
+    want = (op * torch.exp(lp - tot)[..., None]).sum(0)
+    eps = {torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}[dtype]
+    assert ((o[0].float().cpu() - want).abs() <= eps * want.abs() + 1e-5).all()
+    # fp32 parts, no lse wanted
+    o32, none = _kernels.merge_states(o_parts.float(), lse_parts, want_lse=False)
+    assert none is None and ((o32[0].cpu() - want).abs() <= 1e-5 * want.abs().clamp(min=1.0)).all()
+    with pytest.raises(RuntimeError):
+        _kernels.merge_states(o_parts, lse_parts[:, :, :4].contiguous())

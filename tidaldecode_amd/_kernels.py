@@ -14,7 +14,7 @@ reference.  Differences, all additive:
   torch's default current stream).
 """
 import math
-from typing import Optional
+from typing import Optional, Tuple
 
 import torch
 
@@ -343,6 +343,27 @@ def rope_append_decode(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, kv_dat
     check(lib.td_rope_append_decode(pool, q.data_ptr(), k.data_ptr(), v.data_ptr(), b, q.size(1),
                                     positions.data_ptr(), dst_slot.data_ptr(), float(rope_scale),
                                     float(rope_theta), _stream()))
+
+
+def merge_states(o_parts: torch.Tensor, lse_parts: torch.Tensor,
+                 want_lse: bool = True) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """Extension: merge attention states computed over disjoint token subsets.  ``o_parts``
+    ``[n_parts, ..., D]`` (fp16 / bf16 / fp32) and ``lse_parts`` ``[n_parts, ...]`` float32, as
+    ``forward(..., lse=)`` produces them; returns ``(o [..., D], lse [...])``."""
+    _check_input(o_parts, "o_parts")
+    _check_input(lse_parts, "lse_parts")
+    if lse_parts.dtype != torch.float32 or o_parts.dim() < 2 or \
+            tuple(lse_parts.shape) != tuple(o_parts.shape[:-1]):
+        raise RuntimeError("lse_parts must be float32 with the shape of o_parts minus its last axis")
+    n_parts, d = o_parts.size(0), o_parts.size(-1)
+    rows = lse_parts.numel() // n_parts
+    o = torch.empty(o_parts.shape[1:], dtype=o_parts.dtype, device=o_parts.device)
+    lse = torch.empty(lse_parts.shape[1:], dtype=torch.float32, device=o_parts.device) \
+        if want_lse else None
+    check(lib.td_merge_states(o_parts.data_ptr(), _dtype_code(o_parts.dtype, "merge_states"),
+                              lse_parts.data_ptr(), n_parts, rows, d, o.data_ptr(),
+                              None if lse is None else lse.data_ptr(), _stream()))
+    return o, lse
 
 
 def argmax(x: torch.Tensor, out: torch.Tensor) -> None:

@@ -108,6 +108,10 @@ SIGNATURES = {
          c_int32, c_float, c_void_p, c_int32, c_int64, c_void_p, POINTER(FreshToken), c_void_p,
          c_int64, c_void_p],
     ),
+    "td_merge_states": (
+        c_int32,
+        [c_void_p, c_int32, c_void_p, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_void_p],
+    ),
     "td_argmax": (c_int32, [c_void_p, c_int32, c_int32, c_void_p, c_void_p]),
     "td_step_advance_batch": (
         c_int32, [c_void_p, c_int32, c_int32, c_void_p, c_int32, c_int32, c_int32, c_void_p]),

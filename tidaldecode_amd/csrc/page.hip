@@ -469,6 +469,75 @@ extern "C" int td_rope_table(const int32_t* positions, int32_t batch, int32_t he
   return TD_OK;
 }
 
+// Merge of attention states: part i of a row holds the attention output o_i over its own subset of
+// the tokens and the log-sum-exp lse_i of that subset's logits; the attention over the union is
+// o = sum_i o_i e^(lse_i - lse), lse = log sum_i e^(lse_i).  One workgroup of D/2 threads per row.
+// DT: 0 f16, 1 bf16, 2 f32 (parts and result share the type; the arithmetic is fp32).
+template <int DT>
+__global__ void merge_states_kernel(const void* o_parts, const float* lse_parts, int32_t n_parts,
+                                    int32_t rows, int32_t head_dim, void* o, float* lse) {
+  const int row = blockIdx.x;
+  const int d2 = threadIdx.x;  // pair of dimensions
+  float mx = -INFINITY;
+  for (int i = 0; i < n_parts; ++i) mx = fmaxf(mx, lse_parts[(int64_t)i * rows + row]);
+  float wsum = 0.f, a = 0.f, b = 0.f;
+  if (mx > -INFINITY) {
+    for (int i = 0; i < n_parts; ++i) {
+      const float w = __expf(lse_parts[(int64_t)i * rows + row] - mx);  // 0 for an empty part
+      const int64_t at = ((int64_t)i * rows + row) * head_dim + 2 * d2;
+      float x, y;
+      if constexpr (DT == 2) {
+        x = reinterpret_cast<const float*>(o_parts)[at];
+        y = reinterpret_cast<const float*>(o_parts)[at + 1];
+      } else if constexpr (DT == 0) {
+        unpack2<F16>(reinterpret_cast<const uint32_t*>(o_parts)[at / 2], x, y);
+      } else {
+        unpack2<BF16>(reinterpret_cast<const uint32_t*>(o_parts)[at / 2], x, y);
+      }
+      if (w > 0.f) {  // an empty part may hold anything, NaN included
+        wsum += w;
+        a = fmaf(w, x, a);
+        b = fmaf(w, y, b);
+      }
+    }
+  }
+  const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
+  const int64_t out = (int64_t)row * head_dim + 2 * d2;
+  if constexpr (DT == 2) {
+    reinterpret_cast<float*>(o)[out] = a * inv;
+    reinterpret_cast<float*>(o)[out + 1] = b * inv;
+  } else if constexpr (DT == 0) {
+    reinterpret_cast<uint32_t*>(o)[out / 2] = pack2<F16>(a * inv, b * inv);
+  } else {
+    reinterpret_cast<uint32_t*>(o)[out / 2] = pack2<BF16>(a * inv, b * inv);
+  }
+  if (lse && d2 == 0) lse[row] = wsum > 0.f ? mx + __logf(wsum) : -INFINITY;
+}
+
+extern "C" int td_merge_states(const void* o_parts, int32_t dtype, const float* lse_parts,
+                               int32_t n_parts, int32_t rows, int32_t head_dim, void* o, float* lse,
+                               void* stream) {
+  TD_REQUIRE(o_parts && lse_parts && o, "td_merge_states: NULL argument");
+  TD_REQUIRE(n_parts >= 1 && rows >= 1, "td_merge_states: %d parts, %d rows", n_parts, rows);
+  TD_REQUIRE(head_dim >= 2 && head_dim % 2 == 0 && head_dim <= 2048,
+             "td_merge_states: head_dim %d (even, at most 2048)", head_dim);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const dim3 grid(rows), block(head_dim / 2);
+  if (dtype == TD_F16)
+    hipLaunchKernelGGL(merge_states_kernel<0>, grid, block, 0, st, o_parts, lse_parts, n_parts, rows,
+                       head_dim, o, lse);
+  else if (dtype == TD_BF16)
+    hipLaunchKernelGGL(merge_states_kernel<1>, grid, block, 0, st, o_parts, lse_parts, n_parts, rows,
+                       head_dim, o, lse);
+  else if (dtype == TD_F32)
+    hipLaunchKernelGGL(merge_states_kernel<2>, grid, block, 0, st, o_parts, lse_parts, n_parts, rows,
+                       head_dim, o, lse);
+  else
+    return fail(TD_ERR_UNSUPPORTED, "td_merge_states failed to dispatch with dtype %d", dtype);
+  TD_HIP_CHECK(hipGetLastError());
+  return TD_OK;
+}
+
 // Index of the largest of n values (NaN counts as largest, ties go to the lower index): the
 // greedy choice of the next token, kept on the device.  One workgroup; DT: 0 f16, 1 bf16, 2 f32.
 template <int DT>
