@@ -45,6 +45,10 @@ def parse():
     ap.add_argument("--chunk", type=int, default=0, help="tokens per workgroup (0 = default)")
     ap.add_argument("--merge", type=int, default=-1, help="1 fused / 0 second kernel / -1 default")
     ap.add_argument("--rows", type=int, default=0, help="K/V loads per wave tile: 2 / 4 / 8 (0 = default)")
+    ap.add_argument("--sparse-waves", type=int, default=0,
+                    help="short-list kernel: waves per workgroup, 4 / 8 (0 = default, -1 = never use it)")
+    ap.add_argument("--sparse-rows", type=int, default=0,
+                    help="short-list kernel: K rows per lane, 8 / 16 (0 = default)")
     ap.add_argument("--layout", default="NHD", choices=["NHD", "HND"], help="page layout")
     ap.add_argument("--no-fuse", action="store_true",
                     help="run RoPE + append as their own launch instead of inside attention")
@@ -98,6 +102,7 @@ class Workload:
         h = c._decode_handler._wrapper
         h.waves_per_block, h.chunk_tokens, h.fused_merge = args.waves, args.chunk, args.merge
         h.tile_rows = args.rows
+        h.sparse_waves, h.sparse_rows = args.sparse_waves, args.sparse_rows
         c.kv_cache.pool.buf.normal_()      # synthetic prefilled cache, resident in HBM
         c.prepare_metadata(self.N)         # the prompt
         c.prepare_metadata(1)              # the token being decoded

@@ -108,6 +108,13 @@ typedef struct {
   int32_t waves_per_block; /* 8 or 16 */
   int32_t tile_rows;       /* K/V load instructions per wave tile: 2 or 4 */
   int32_t fused_merge;     /* 1: last workgroup merges in-kernel; 0: second kernel */
+  /* Shape of the short-list kernel that serves calls with token-slot lists, head_dim 128, one
+   * list row per query head (or one shared row without grouped queries), power-of-two pages, a
+   * pool below 4 GiB and no score output: waves per workgroup (4 or 8) x K rows per lane (8 or
+   * 16).  0 on input: the planner decides; -1 on input: never use that kernel.  On output 0
+   * means the streaming kernel (waves_per_block x tile_rows) serves every call of this plan. */
+  int32_t sparse_waves;
+  int32_t sparse_rows;
   int64_t workspace_bytes; /* device scratch the call needs (partials + tickets) */
 } td_decode_plan;
 
@@ -175,9 +182,10 @@ int td_rope_append_decode(const td_paged_kv* kv, void* q, const void* k, const v
 
 /*
  * Choose the split of a decode-attention call.  max_items is an upper bound of the tokens any
- * sequence attends to; idx_rows as in td_index_list.  chunk_tokens / waves_per_block / tile_rows (non-zero)
- * and fused_merge (non-negative) may be preset in *plan to override the heuristics; pass a
- * zero-initialised struct with fused_merge = -1 for defaults.  Host arithmetic only.
+ * sequence attends to; idx_rows as in td_index_list.  chunk_tokens / waves_per_block / tile_rows /
+ * sparse_waves / sparse_rows (non-zero) and fused_merge (non-negative) may be preset in *plan to
+ * override the heuristics; pass a zero-initialised struct with fused_merge = -1 for defaults.
+ * Host arithmetic only.
  * Replaces BatchDecodeWithPagedKVCacheWorkEstimation and PartitionPagedKVCacheComputeAuxiliaryInfo
  * (kernels/include/decode/decode_attn.cuh:815-906, :687-748), reached through
  * BatchDecodeHandler::BeginForward (decode_handler.cuh:39-121, binding approx_attn.cu:27-62).
@@ -200,10 +208,10 @@ int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t num_kv_head
  *              td_rope_append_decode + td_decode_attn (tidal/models/SearchAttention.py:131-176 runs
  *              three).  Needs a power-of-two page_size and a pool below 4 GiB
  *              (TD_ERR_UNSUPPORTED otherwise).
- *   workspace  device scratch of at least plan->workspace_bytes whose first 64 KiB (ticket
- *              counters) were zero-filled once before first use; every call leaves them zero
- *              again, so one workspace serves plans of any shape.  Calls that share a
- *              workspace must be ordered on one stream.
+ *   workspace  device scratch of at least plan->workspace_bytes whose first 1 MiB (ticket
+ *              counters, 64 bytes apart) was zero-filled once before first use; every call
+ *              leaves them zero again, so one workspace serves plans of any shape.  Calls that
+ *              share a workspace must be ordered on one stream.
  * Replaces BatchDecodeWithPagedKVCachePyTorchWrapper::Forward (bsk_ops.h:104-113,
  * tidal/ops/csrc/approx_attn.cu:68-151), BatchDecodeWithPagedKVCacheKernel
  * (kernels/include/decode/decode_attn.cuh:432-658) including its score output

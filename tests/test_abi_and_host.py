@@ -42,7 +42,8 @@ def _plan(batch, hq, hkv, d, rows, items, **preset):
     from tidaldecode_amd._lib import DecodePlan, lib
 
     p = DecodePlan(preset.get("chunk", 0), 0, preset.get("waves", 0), preset.get("rows", 0),
-                   preset.get("merge", -1), 0)
+                   preset.get("merge", -1), preset.get("sparse_waves", 0),
+                   preset.get("sparse_rows", 0), 0)
     rc = lib.td_decode_make_plan(batch, hq, hkv, d, rows, items, p)
     return rc, p
 

@@ -483,6 +483,8 @@ class BatchDecodeWithPagedKVCachePyTorchWrapper:
         self.fused_merge = -1     # -1 = library default
         self.chunk_tokens = 0     # 0 = library default
         self.tile_rows = 0        # 0 = library default
+        self.sparse_waves = 0     # short-list kernel: 0 = library default, -1 = never
+        self.sparse_rows = 0
 
     def begin_forward(self, indptr: torch.Tensor, num_qo_heads: int, num_kv_heads: int,
                       head_dim: int, page_size: int, empty_data: torch.Tensor) -> None:
@@ -505,14 +507,18 @@ class BatchDecodeWithPagedKVCachePyTorchWrapper:
         self._begun = False
         self._plans.clear()
 
-    def _plan(self, batch: int, idx_rows: int, max_items: int) -> DecodePlan:
+    def _plan(self, batch: int, idx_rows: int, max_items: int, short_list: bool = True) -> DecodePlan:
+        """``short_list``: the call has token-slot lists and no score output, the two things the
+        planner cannot see that the short-list kernel needs; other calls get a plan shaped for
+        the streaming kernel."""
+        sparse_waves = self.sparse_waves if short_list else -1
         key = (batch, idx_rows, max_items, self.waves_per_block, self.fused_merge,
-               self.chunk_tokens, self.tile_rows)
+               self.chunk_tokens, self.tile_rows, sparse_waves, self.sparse_rows)
         plan = self._plans.get(key)
         if plan is None:
             hq, hkv, d, _, _ = self._geom
             plan = DecodePlan(self.chunk_tokens, 0, self.waves_per_block, self.tile_rows,
-                              self.fused_merge, 0)
+                              self.fused_merge, sparse_waves, self.sparse_rows, 0)
             check(lib.td_decode_make_plan(batch, hq, hkv, d, idx_rows, max_items, plan))
             self._plans[key] = plan
         return plan
@@ -593,7 +599,8 @@ class BatchDecodeWithPagedKVCachePyTorchWrapper:
             lst.last_page_idx = int(paged_kv_last_page_idx)
 
         max_items = lst.n_list_host * (page if kind == TD_IDX_PAGES else 1) + max_last
-        plan = self._plan(batch, rows, max_items)
+        has_scores = qk_product is not None and qk_product.numel() > 0
+        plan = self._plan(batch, rows, max_items, kind == TD_IDX_SLOTS and not has_scores)
         if plan.workspace_bytes > 0 and (self._workspace is None or
                                          self._workspace.numel() < plan.workspace_bytes or
                                          self._workspace.device != q.device):

@@ -74,6 +74,8 @@ class DecodePlan(Structure):
         ("waves_per_block", c_int32),
         ("tile_rows", c_int32),
         ("fused_merge", c_int32),
+        ("sparse_waves", c_int32),
+        ("sparse_rows", c_int32),
         ("workspace_bytes", c_int64),
     ]
 

@@ -63,6 +63,8 @@ struct DecodeParams {
   int32_t last_idx;
   // split
   int32_t chunk_tokens;
+  int32_t chunk_shift;  // log2(chunk_tokens) or -1
+  int32_t qpk_shift;    // log2(q_per_kv) or -1
   int32_t max_splits;
   int32_t fused_merge;
   float scale_log2;  // sm_scale * log2(e)
@@ -73,7 +75,9 @@ struct DecodeParams {
   float* lse;
   float* ws_o;      // [batch * H_q * max_splits, D]
   float* ws_ml;     // [batch * H_q * max_splits, 2]
-  int32_t* ws_cnt;  // [batch * head rows] ticket counters
+  int32_t* ws_cnt;  // [batch * head rows] ticket counters, ticket_stride words apart
+  int32_t ticket_stride;
+  uint64_t* ws_st;  // [batch * H_q * max_splits, 130] stamped partials of the sparse-layer kernel
   // the token being decoded (FRESH kernels): un-rotated k, v, its rotary cos/sin and its slot
   const void* fresh_k;
   const void* fresh_v;
@@ -231,8 +235,12 @@ __device__ __forceinline__ int seq_items(const DecodeParams& p, int b, SeqList& 
   s.n_list = s.n_list < 0 ? 0 : (s.n_list > p.n_list_host ? p.n_list_host : s.n_list);
   s.last_len = p.last_len_arr ? p.last_len_arr[b] : p.last_len;
   s.last_idx = p.last_idx_arr ? p.last_idx_arr[b] : p.last_idx;
+  // device-resident lengths are not trusted: a fill beyond the page, or more splits than the
+  // grid holds, would leave tickets that no workgroup ever takes
+  s.last_len = s.last_len < 0 ? 0 : (s.last_len > p.page_size ? p.page_size : s.last_len);
   s.n_items = (p.page_mode ? s.n_list * p.page_size : s.n_list) + s.last_len;
   int n_splits = (s.n_items + p.chunk_tokens - 1) / p.chunk_tokens;
+  n_splits = n_splits > p.max_splits ? p.max_splits : n_splits;
   return n_splits < 1 ? 1 : n_splits;
 }
 
@@ -807,7 +815,7 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
   // ---- the last workgroup of this (sequence, head row) to arrive reduces the partials ----------
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // partial stores have left this CU
   __syncthreads();
-  int32_t* ticket = p.ws_cnt + (int64_t)b * gridDim.x + hrow;
+  int32_t* ticket = p.ws_cnt + ((int64_t)b * gridDim.x + hrow) * p.ticket_stride;
   if (tid == 0)
     sm_ticket = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();

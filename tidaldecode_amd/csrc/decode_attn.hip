@@ -1,6 +1,6 @@
 // Host side of the decode-attention entry points: split planning and argument checks.  The
 // kernels live in decode_attn.cuh and are instantiated in decode_attn_{f16,bf16}.hip.
-#include "decode_attn.cuh"
+#include "sparse_attn.cuh"
 
 namespace tidal {
 
@@ -23,8 +23,17 @@ static int64_t align256(int64_t x) { return (x + 255) & ~(int64_t)255; }
 
 // Workspace layout: [ticket counters, fixed size | partial o | partial (m, l)].  The counters sit
 // at a fixed place so that plans of different shapes sharing one workspace never find another
-// plan's partial results where they expect zeroed tickets.
-constexpr int64_t kTicketBytes = 65536;
+// plan's partial results where they expect zeroed tickets.  A counter has 64 bytes to itself: the
+// tickets of a launch are all taken within a microsecond, and counters that share a line queue up
+// behind one another at the memory channel (measured: 0.4 us of a 9.7 us launch).
+constexpr int kTicketStride = 16;  // int32 words between counters
+constexpr int64_t kTicketBytes = (int64_t)16384 * kTicketStride * 4;
+
+// The short-list kernel (sparse_attn.cuh) covers a list in one pass of at most 64 workgroups per
+// head; longer lists go to the streaming kernel, whose waves pipeline several tiles.
+constexpr int64_t kSparseMaxItems = 64 * 256;
+
+static bool is_pow2(int64_t x) { return x > 0 && (x & (x - 1)) == 0; }
 
 }  // namespace tidal
 
@@ -52,6 +61,58 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
   const int qpg = qpg_for(num_qo_heads, num_kv_heads, idx_rows, head_dim);
   const int subs = qpg > 1 ? (num_qo_heads / num_kv_heads + qpg - 1) / qpg : 1;
   const int n_hrows = qpg > 1 ? num_kv_heads * subs : num_qo_heads;
+
+  // ---- short lists: the sparse-layer kernel -------------------------------------------------------
+  // Chunks are a power of two (the kernel divides by shifting) and a multiple of the workgroup
+  // tile; the streaming kernel at 8 waves x 4 rows (tile 128) can run the same plan when a call
+  // turns out not to fit the short-list kernel (page lists, score output, large pools).
+  int sw = plan->sparse_waves, sr = plan->sparse_rows;
+  bool sparse = sw >= 0 && sr >= 0 && head_dim == 128 && qpg == 1 &&
+                is_pow2(num_qo_heads / num_kv_heads) && max_items > 0 && max_items <= kSparseMaxItems &&
+                (plan->chunk_tokens == 0 || is_pow2(plan->chunk_tokens));
+  if (sparse) {
+    // Chunk: the smallest power of two from 128 tokens up that leaves at most 9/8 workgroups per
+    // compute unit, but no more than 512 tokens -- the waves of this kernel do not pipeline their
+    // tiles, so large launches are better served by two workgroups per compute unit than by long
+    // loops (ragged batch of 8 x 32 heads x 1024 tokens: 29 us at 512 tokens per workgroup, 35 us
+    // at 1024).  Workgroup shape: 4 waves for 128-token chunks, 8 waves otherwise, 8 K rows per lane.
+    int64_t chunk = plan->chunk_tokens;
+    if (chunk == 0) {
+      chunk = 128;
+      while (chunk < 512 && (int64_t)n_hrows * batch * ceil_div64(max_items, chunk) > num_cus() * 9 / 8)
+        chunk <<= 1;
+    }
+    while (ceil_div64(max_items, chunk) > 64) chunk <<= 1;
+    if (sr == 0) sr = 8;
+    if (sw == 0) sw = (chunk < 256 || sr == 16) ? 4 : 8;
+    if (!sparse_shape_supported(sw, sr))
+      return fail(TD_ERR_UNSUPPORTED,
+                  "td_decode_make_plan: no short-list kernel with %d waves x %d rows (4 or 8 waves, 8 or "
+                  "16 rows)", sw, sr);
+    const int stile = sw * 4 * sr;
+    if (plan->chunk_tokens == 0 && chunk < stile) chunk = stile;  // a preset shape with a larger tile
+    if (chunk % stile != 0 || chunk % 128 != 0) {
+      sparse = false;
+    } else {
+      plan->chunk_tokens = (int32_t)chunk;
+      plan->max_splits = (int32_t)ceil_div64(max_items, chunk);
+      plan->waves_per_block = 8;
+      plan->tile_rows = 4;
+      plan->sparse_waves = sw;
+      plan->sparse_rows = sr;
+    }
+  }
+  if (sparse) {
+    if (plan->fused_merge < 0) plan->fused_merge = 1;
+    plan->fused_merge = plan->fused_merge ? 1 : 0;
+    TD_REQUIRE((int64_t)batch * n_hrows * kTicketStride * 4 <= kTicketBytes,
+               "td_decode_make_plan: batch %d x %d head rows exceeds the %lld ticket counters", batch,
+               n_hrows, (long long)(kTicketBytes / (kTicketStride * 4)));
+    const int64_t n_part = (int64_t)batch * n_hrows * plan->max_splits;
+    plan->workspace_bytes = kTicketBytes + align256(n_part * head_dim * 4) + align256(n_part * 2 * 4);
+    return TD_OK;
+  }
+  plan->sparse_waves = plan->sparse_rows = 0;
 
   int nw = plan->waves_per_block;
   if (nw == 0) nw = 8;
@@ -94,9 +155,9 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
   plan->tile_rows = rows;
   if (plan->fused_merge < 0) plan->fused_merge = 1;
   plan->fused_merge = plan->fused_merge ? 1 : 0;
-  TD_REQUIRE((int64_t)batch * n_hrows * 4 <= kTicketBytes,
+  TD_REQUIRE((int64_t)batch * n_hrows * kTicketStride * 4 <= kTicketBytes,
              "td_decode_make_plan: batch %d x %d head rows exceeds the %lld ticket counters", batch,
-             n_hrows, (long long)(kTicketBytes / 4));
+             n_hrows, (long long)(kTicketBytes / (kTicketStride * 4)));
   const int64_t n_part = (int64_t)batch * n_hrows * qpg * max_splits;  // head slots incl. padding
   plan->workspace_bytes = kTicketBytes + align256(n_part * head_dim * 4) + align256(n_part * 2 * 4);
   return TD_OK;
@@ -172,7 +233,7 @@ static int build_params(const td_paged_kv* kv, const td_index_list* list, const 
   const int64_t off_o = kTicketBytes;
   const int64_t off_ml = off_o + align256(n_part * D * 4);
   const int64_t need = off_ml + align256(n_part * 2 * 4);
-  TD_REQUIRE((int64_t)batch * n_hrows * 4 <= kTicketBytes,
+  TD_REQUIRE((int64_t)batch * n_hrows * kTicketStride * 4 <= kTicketBytes,
              "td_decode_attn: batch %d x %d head rows exceeds the ticket counters", batch, n_hrows);
   TD_REQUIRE(plan->max_splits <= 64, "td_decode_attn: plan has %d splits (limit 64)",
              plan->max_splits);
@@ -239,6 +300,11 @@ static int build_params(const td_paged_kv* kv, const td_index_list* list, const 
   p.last_len = list->last_page_len;
   p.last_idx = list->last_page_idx;
   p.chunk_tokens = plan->chunk_tokens;
+  p.chunk_shift = p.qpk_shift = -1;
+  for (int sft = 0; sft < 31; ++sft) {
+    if ((1 << sft) == plan->chunk_tokens) p.chunk_shift = sft;
+    if ((1 << sft) == p.q_per_kv) p.qpk_shift = sft;
+  }
   p.max_splits = plan->max_splits;
   p.fused_merge = plan->fused_merge;
   p.scale_log2 = sm_scale * kLog2e;
@@ -248,10 +314,24 @@ static int build_params(const td_paged_kv* kv, const td_index_list* list, const 
   p.lse = lse;
   char* ws = reinterpret_cast<char*>(workspace);
   p.ws_cnt = reinterpret_cast<int32_t*>(ws);
+  p.ticket_stride = kTicketStride;
   p.ws_o = reinterpret_cast<float*>(ws ? ws + off_o : nullptr);
   p.ws_ml = reinterpret_cast<float*>(ws ? ws + off_ml : nullptr);
 
   return TD_OK;
+}
+
+// Whether a call can run on the short-list kernel of its plan: token-slot lists, head_dim 128, one
+// query head per list walk, 32-bit lean addressing whose strides fit the 24-bit multiplier, no
+// score output, chunks that are a power-of-two multiple of the kernel's workgroup tile.
+static bool sparse_kernel_fits(const DecodeParams& p, const td_decode_plan* plan,
+                               const td_index_list* list, int qpg, int head_dim, bool emit) {
+  if (plan->sparse_waves <= 0 || !sparse_shape_supported(plan->sparse_waves, plan->sparse_rows))
+    return false;
+  const int stile = plan->sparse_waves * 4 * plan->sparse_rows;
+  return list->kind == TD_IDX_SLOTS && p.lean && !emit && qpg == 1 && head_dim == 128 &&
+         p.chunk_shift >= 0 && p.qpk_shift >= 0 && plan->chunk_tokens % stile == 0 &&
+         p.page_stride_b < (1u << 24) && p.entry_stride_b < (1u << 24);
 }
 
 extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
@@ -271,6 +351,15 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
   dim3 grid(n_hrows, plan->max_splits, batch);
   const bool merge_kernel = plan->max_splits > 1 && !plan->fused_merge;
   int rc;
+  if (sparse_kernel_fits(p, plan, list, qpg, D, scores != nullptr)) {
+    if (kv->dtype == TD_F16)
+      rc = launch_sparse_f16(p, plan->sparse_waves, plan->sparse_rows, false, merge_kernel, grid, st);
+    else
+      rc = launch_sparse_bf16(p, plan->sparse_waves, plan->sparse_rows, false, merge_kernel, grid, st);
+    if (rc != TD_OK) return rc;
+    TD_HIP_CHECK(hipGetLastError());
+    return TD_OK;
+  }
   if (kv->dtype == TD_F16)
     rc = launch_decode_f16(p, D, qpg, plan->waves_per_block, plan->tile_rows, page_mode, scores != nullptr,
                            merge_kernel, grid, st);
@@ -340,6 +429,21 @@ extern "C" int td_gather_probe(const td_paged_kv* kv, const td_index_list* list,
   const int prc = build_params(kv, list, plan, out, out, batch, num_qo_heads, 1.f, nullptr, TD_F32, 0,
                                nullptr, nullptr, out, (int64_t)1 << 40, p, qpg, n_hrows);
   if (prc != TD_OK) return prc;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (sparse_kernel_fits(p, plan, list, qpg, kv->head_dim, false) && list->last_page_len == 0 &&
+      !list->last_page_len_arr) {
+    // the short-list kernel's own loads-only form; it reads `out` as q and writes nothing
+    TD_REQUIRE(out_bytes >= (int64_t)batch * num_qo_heads * kv->head_dim * 2,
+               "td_gather_probe: out holds %lld bytes, %lld needed", (long long)out_bytes,
+               (long long)batch * num_qo_heads * kv->head_dim * 2);
+    const dim3 sgrid(n_hrows, plan->max_splits, batch);
+    const int src = kv->dtype == TD_F16
+                        ? launch_sparse_f16(p, plan->sparse_waves, plan->sparse_rows, true, false, sgrid, st)
+                        : launch_sparse_bf16(p, plan->sparse_waves, plan->sparse_rows, true, false, sgrid, st);
+    if (src != TD_OK) return src;
+    TD_HIP_CHECK(hipGetLastError());
+    return TD_OK;
+  }
   const int nw = plan->waves_per_block, rows = plan->tile_rows;
   if (!(list->kind == TD_IDX_SLOTS && p.lean && qpg == 1 && kv->head_dim == 128 &&
         ((nw == 8 && (rows == 4 || rows == 2)) || (nw == 16 && rows == 4)) &&
@@ -351,7 +455,6 @@ extern "C" int td_gather_probe(const td_paged_kv* kv, const td_index_list* list,
              "td_gather_probe: out holds %lld bytes, %lld needed", (long long)out_bytes,
              (long long)batch * n_hrows * plan->max_splits * nw * 4);
   const dim3 grid(n_hrows, plan->max_splits, batch);
-  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   uint32_t* outw = reinterpret_cast<uint32_t*>(out);
   if (nw == 16)
     hipLaunchKernelGGL((gather_probe_kernel<128, 4, 16>), grid, dim3(1024), 0, st, p, outw);

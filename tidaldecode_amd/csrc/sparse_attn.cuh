@@ -1,0 +1,541 @@
+// Sparse-layer decode attention for gfx950 (MI355X): the short-list form of decode_attn_kernel,
+// for head_dim 128, one query head per head row, token-slot lists, power-of-two pages and a pool
+// below 4 GiB.  Same arguments, same split workspace and the same results as decode_attn_kernel;
+// what differs is the shape of the work, chosen for launches that move a few tens of MiB and are
+// bound by dependent round trips and instruction issue rather than by bandwidth:
+//
+//   * a wave owns 4 U tokens (U = 8 or 16 K rows and as many V rows per lane: 64 or 128 VGPRs of
+//     loads), all of them in flight at once, K rows first so that q.k runs while V arrives;
+//   * the list entry of a token is loaded once, by the lane that owns the token; its byte offset
+//     reaches the 16 lanes of a row through DPP row broadcasts (one instruction per row);
+//   * q.k partial sums are reduce-scattered over the 16 lanes of a row, so that after U partial
+//     dot products a lane holds the complete logit of ONE token and the softmax arithmetic runs
+//     once per token instead of once per lane; the probabilities go back through row broadcasts;
+//   * the maximum is wave-uniform per tile, so the four lane groups add up without rescaling;
+//   * the workgroup's waves meet once in LDS, then wave 0 alone publishes the partial, takes the
+//     ticket and, if it is the last of its head row, merges the partials (no further barrier).
+//
+// Semantics follow kernels/include/decode/decode_attn.cuh:432-658 of the reference
+// (BatchDecodeWithPagedKVCacheKernel) including the forced last page (decode_page.cuh:320-346).
+
+#pragma once
+
+#include "decode_attn.cuh"
+
+namespace tidal {
+
+// value of lane N of this lane's 16-lane row (DPP row_newbcast)
+template <int N>
+__device__ __forceinline__ uint32_t row_bcast_u32(uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x150 + N, 0xf, 0xf, true);
+}
+template <int N>
+__device__ __forceinline__ float row_bcast_f32(float x) {
+  return __builtin_bit_cast(float, row_bcast_u32<N>(__builtin_bit_cast(uint32_t, x)));
+}
+
+// a[u] = this lane's partial sum for row u (U rows, U = 8 or 16) over its 8 of the 128 dimensions;
+// returns the sum over the 16 lanes of the row group for row (lane % U).  Each butterfly step
+// halves the rows a lane keeps and hands the other half to a partner whose lane index differs in
+// the step's bit (any partner of the opposite class does, as long as every lane's contribution is
+// counted once: xor 1, xor 2, rotate by 4, rotate by 8).
+template <int U>
+__device__ __forceinline__ float reduce_scatter_rows(float (&a)[U], int li) {
+  static_assert(U == 8 || U == 16, "rows per lane group");
+  float c1[U / 2], c2[U / 4], c3[U / 8];
+  {
+    const bool hi = li & 1;
+#pragma unroll
+    for (int i = 0; i < U / 2; ++i) {
+      const float keep = hi ? a[2 * i + 1] : a[2 * i];
+      const float send = hi ? a[2 * i] : a[2 * i + 1];
+      c1[i] = keep + dpp_move<0xB1>(send);  // quad_perm [1,0,3,2]
+    }
+  }
+  {
+    const bool hi = li & 2;
+#pragma unroll
+    for (int i = 0; i < U / 4; ++i) {
+      const float keep = hi ? c1[2 * i + 1] : c1[2 * i];
+      const float send = hi ? c1[2 * i] : c1[2 * i + 1];
+      c2[i] = keep + dpp_move<0x4E>(send);  // quad_perm [2,3,0,1]
+    }
+  }
+  {
+    const bool hi = li & 4;
+#pragma unroll
+    for (int i = 0; i < U / 8; ++i) {
+      const float keep = hi ? c2[2 * i + 1] : c2[2 * i];
+      const float send = hi ? c2[2 * i] : c2[2 * i + 1];
+      c3[i] = keep + dpp_move<0x124>(send);  // row_ror:4: the sender sits in the other quad class
+    }
+  }
+  if constexpr (U == 16) {
+    const bool hi = li & 8;
+    const float keep = hi ? c3[1] : c3[0];
+    const float send = hi ? c3[0] : c3[1];
+    return keep + dpp_move<0x128>(send);  // row_ror:8
+  } else {
+    return c3[0] + dpp_move<0x128>(c3[0]);  // lanes li and li ^ 8 hold the same row
+  }
+}
+
+// maximum / sum over the 16 lanes of a row, result in every lane
+__device__ __forceinline__ float row16_max(float x) {
+  x = fmaxf(x, dpp_move<0xB1>(x));
+  x = fmaxf(x, dpp_move<0x4E>(x));
+  x = fmaxf(x, dpp_move<0x141>(x));
+  x = fmaxf(x, dpp_move<0x140>(x));
+  return x;
+}
+
+// exchange between the halves / the odd and even 16-lane rows of a wavefront: (a, b) -> x, y with
+//   swap32: x = [a.lower | b.lower], y = [a.upper | b.upper]
+//   swap16: x = [a.row0 | b.row0 | a.row2 | b.row2], y = [a.row1 | b.row1 | a.row3 | b.row3]
+__device__ __forceinline__ void swap32(float a, float b, float& x, float& y) {
+  const u32pair r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, a),
+                                                     __builtin_bit_cast(uint32_t, b), false, false);
+  const uint32_t lo = r.x, hi = r.y;
+  x = __builtin_bit_cast(float, lo);
+  y = __builtin_bit_cast(float, hi);
+}
+__device__ __forceinline__ void swap16(float a, float b, float& x, float& y) {
+  const u32pair r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(uint32_t, a),
+                                                     __builtin_bit_cast(uint32_t, b), false, false);
+  const uint32_t lo = r.x, hi = r.y;
+  x = __builtin_bit_cast(float, lo);
+  y = __builtin_bit_cast(float, hi);
+}
+
+// Wave-uniform words of device-resident state, fetched through the scalar cache in one round trip
+// (the compiler cannot: the kernel also writes memory, so it would use a vector load and a full
+// wait for each word).  The words were written by earlier launches; a launch starts with a clean
+// scalar cache.
+__device__ __forceinline__ void scalar_load2(const int32_t* a0, const int32_t* a1, int32_t& v0,
+                                             int32_t& v1) {
+  asm volatile(
+      "s_load_dword %0, %2, 0x0\n\t"
+      "s_load_dword %1, %3, 0x0\n\t"
+      "s_waitcnt lgkmcnt(0)"
+      : "=&s"(v0), "=&s"(v1)
+      : "s"(a0), "s"(a1)
+      : "memory");
+}
+__device__ __forceinline__ void scalar_load4(const int32_t* a0, const int32_t* a1, const int32_t* a2,
+                                             const int32_t* a3, int32_t& v0, int32_t& v1, int32_t& v2,
+                                             int32_t& v3) {
+  asm volatile(
+      "s_load_dword %0, %4, 0x0\n\t"
+      "s_load_dword %1, %5, 0x0\n\t"
+      "s_load_dword %2, %6, 0x0\n\t"
+      "s_load_dword %3, %7, 0x0\n\t"
+      "s_waitcnt lgkmcnt(0)"
+      : "=&s"(v0), "=&s"(v1), "=&s"(v2), "=&s"(v3)
+      : "s"(a0), "s"(a1), "s"(a2), "s"(a3)
+      : "memory");
+}
+
+template <typename T, int NW, int U, bool FRESH, bool PROBE = false>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U == 16 ? 2 : 4))) void sparse_attn_kernel(const DecodeParams p) {
+  constexpr int D = 128;
+  constexpr int LPR = 16;       // lanes per K/V row
+  constexpr int TILE = 4 * U;   // tokens of a wave tile: lane group g holds tokens g U .. g U + U - 1
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int g = lane >> 4, li = lane & 15;
+  const int hrow = blockIdx.x, split = blockIdx.y, b = blockIdx.z;
+  // One batch of scalar loads for every kernel argument the main path uses: the compiler would
+  // otherwise fetch them where they are first needed, a dependent round trip each time.
+#define TD_TOUCH(x) asm volatile("" ::"s"(x))
+  TD_TOUCH(p.q); TD_TOUCH(p.kv); TD_TOUCH(p.v_offset); TD_TOUCH(p.idx); TD_TOUCH(p.indptr);
+  TD_TOUCH(p.count_arr); TD_TOUCH(p.last_len_arr); TD_TOUCH(p.last_idx_arr);
+  TD_TOUCH(p.idx_row_stride); TD_TOUCH(p.n_list_host); TD_TOUCH(p.qpk_shift);
+  TD_TOUCH(p.chunk_shift); TD_TOUCH(p.max_splits); TD_TOUCH(p.page_shift); TD_TOUCH(p.max_slot);
+  TD_TOUCH(p.page_stride_b); TD_TOUCH(p.entry_stride_b); TD_TOUCH(p.head_stride);
+  TD_TOUCH(p.last_len); TD_TOUCH(p.last_idx); TD_TOUCH(p.scale_log2); TD_TOUCH(p.num_qo_heads);
+  if constexpr (FRESH) {
+    TD_TOUCH(p.fresh_k); TD_TOUCH(p.fresh_v); TD_TOUCH(p.fresh_cos); TD_TOUCH(p.fresh_sin);
+    TD_TOUCH(p.fresh_slot);
+  }
+#undef TD_TOUCH
+  const int kv_head = hrow >> p.qpk_shift;  // the host sends only power-of-two group sizes here
+  const int own = g * U + (li & (U - 1));   // the token of the tile this lane owns
+
+  // ---- everything that depends on the kernel arguments only is requested at once ---------------
+  // The list entries of the first tile are read before the length of the list is known: the
+  // position is clamped to the row's capacity (n_list_host), which the host has checked against
+  // the row stride.
+  const int t0 = (split * NW + wave) * TILE;
+  const int idx_row = p.idx_per_kv ? kv_head : hrow;
+  int list_beg = 0, list_end = 0;
+  if (p.indptr) scalar_load2(p.indptr + b, p.indptr + b + 1, list_beg, list_end);
+  const int32_t* row = p.idx + (int64_t)idx_row * p.idx_row_stride + list_beg;
+  const bool has_cap = p.n_list_host > 0;
+  auto fetch_entry = [&](int t) -> int32_t {
+    int pos = t + own;
+    pos = pos < p.n_list_host ? pos : p.n_list_host - 1;
+    return has_cap ? row[pos] : 0;
+  };
+  int32_t ent = fetch_entry(t0);
+
+  uint32_t qp[4];
+  {
+    const u32x4 v = reinterpret_cast<const u32x4*>(p.q)[((int64_t)b * p.num_qo_heads + hrow) * LPR + li];
+    qp[0] = v.x; qp[1] = v.y; qp[2] = v.z; qp[3] = v.w;
+  }
+  uint32_t knew[4] = {0, 0, 0, 0}, vnew[4] = {0, 0, 0, 0};
+  // slot of the token being decoded: requested now, waited for after the K/V rows are on their way
+  // (only the comparison with the list needs it)
+  int32_t new_slot_raw = -1;
+  if constexpr (FRESH)
+    asm volatile("s_load_dword %0, %1, 0x0" : "=s"(new_slot_raw) : "s"(p.fresh_slot + b) : "memory");
+  auto new_slot_wait = [&]() -> uint32_t {
+    if constexpr (FRESH) asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(new_slot_raw)::"memory");
+    return (uint32_t)new_slot_raw;
+  };
+  float rcs[8], rsn[8];
+  if constexpr (FRESH) {
+    constexpr int HALF = LPR / 2;
+    const f32x4* cp = reinterpret_cast<const f32x4*>(p.fresh_cos + (int64_t)b * (D / 2) + (li % HALF) * 8);
+    const f32x4* sp = reinterpret_cast<const f32x4*>(p.fresh_sin + (int64_t)b * (D / 2) + (li % HALF) * 8);
+    const f32x4 c0 = cp[0], c1v = cp[1], s0 = sp[0], s1 = sp[1];
+    rcs[0] = c0.x; rcs[1] = c0.y; rcs[2] = c0.z; rcs[3] = c0.w;
+    rcs[4] = c1v.x; rcs[5] = c1v.y; rcs[6] = c1v.z; rcs[7] = c1v.w;
+    const float sgn = li < HALF ? -1.f : 1.f;  // y_lo = x_lo c - x_hi s,  y_hi = x_hi c + x_lo s
+    rsn[0] = sgn * s0.x; rsn[1] = sgn * s0.y; rsn[2] = sgn * s0.z; rsn[3] = sgn * s0.w;
+    rsn[4] = sgn * s1.x; rsn[5] = sgn * s1.y; rsn[6] = sgn * s1.z; rsn[7] = sgn * s1.w;
+    const int64_t fresh_off = ((int64_t)b * (p.num_qo_heads >> p.qpk_shift) + kv_head) * LPR + li;
+    const u32x4 kn = reinterpret_cast<const u32x4*>(p.fresh_k)[fresh_off];
+    const u32x4 vn = reinterpret_cast<const u32x4*>(p.fresh_v)[fresh_off];
+    knew[0] = kn.x; knew[1] = kn.y; knew[2] = kn.z; knew[3] = kn.w;
+    vnew[0] = vn.x; vnew[1] = vn.y; vnew[2] = vn.z; vnew[3] = vn.w;
+  }
+
+  // ---- the sequence: listed entries, forced last page, splits ------------------------------------
+  // (seq_items of decode_attn.cuh with the division by the chunk size as a shift)
+  SeqList s;
+  s.n_list = p.n_list_host;
+  s.last_len = p.last_len;
+  s.last_idx = p.last_idx;
+  if (p.count_arr || p.last_len_arr || p.last_idx_arr) {
+    // absent arrays read a dummy word (q is never NULL) and keep the host value
+    const int32_t* dummy = reinterpret_cast<const int32_t*>(p.q);
+    int32_t cnt, ll, lx, unused;
+    scalar_load4(p.count_arr ? p.count_arr + b : dummy, p.last_len_arr ? p.last_len_arr + b : dummy,
+                 p.last_idx_arr ? p.last_idx_arr + b : dummy, dummy, cnt, ll, lx, unused);
+    if (p.indptr) s.n_list = p.count_arr ? cnt : list_end - list_beg;
+    if (p.last_len_arr) s.last_len = ll;
+    if (p.last_idx_arr) s.last_idx = lx;
+  } else if (p.indptr) {
+    s.n_list = list_end - list_beg;
+  }
+  s.n_list = s.n_list < 0 ? 0 : (s.n_list > p.n_list_host ? p.n_list_host : s.n_list);
+  s.last_len = s.last_len < 0 ? 0 : (s.last_len > p.page_size ? p.page_size : s.last_len);
+  const int c1 = s.n_list + s.last_len;
+  int n_splits = (c1 + p.chunk_tokens - 1) >> p.chunk_shift;
+  n_splits = n_splits > p.max_splits ? p.max_splits : n_splits;
+  n_splits = n_splits < 1 ? 1 : n_splits;
+  if (split >= n_splits) return;  // uniform for the workgroup
+  const uint32_t last_base = (uint32_t)s.last_idx << p.page_shift;
+
+  // rotate-half RoPE of 8 elements per lane; the partner dimension (+- 64) sits 8 lanes away
+  auto rotate = [&](uint32_t(&w)[4]) {
+    float x[8], y[8];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) unpack2<T>(w[c], x[2 * c], x[2 * c + 1]);
+#pragma unroll
+    for (int d = 0; d < 8; ++d) y[d] = x[d] * rcs[d] + dpp_move<0x128>(x[d]) * rsn[d];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) w[c] = pack2<T>(y[2 * c], y[2 * c + 1]);
+  };
+
+  const char* kbase = reinterpret_cast<const char*>(p.kv);
+  const char* vbase = kbase + p.v_offset * 2;
+  const uint32_t head_byte_off = (uint32_t)(kv_head * p.head_stride + li * 8) * 2u;
+  const uint32_t entry_mask = (1u << p.page_shift) - 1u;
+
+  float m_run = kNegBig;  // wave-uniform running maximum (base-2 logits)
+  float l_lane = 0.f;     // this lane's share of the denominator
+  float acc[8];
+#pragma unroll
+  for (int d = 0; d < 8; ++d) acc[d] = 0.f;
+  // Decode-step fusion: q arrives un-rotated and is rotated in registers, once per wave.  The new
+  // token's key is rotated by the wave that writes it into the cache (one per KV head) and by
+  // every wave whose tokens include its slot.
+  bool q_rot = false, k_rot = false, wrote = false;  // wave-uniform
+  const bool writer = FRESH && split == 0 && wave == 0 && hrow == (kv_head << p.qpk_shift);
+  auto fresh_duties = [&](bool any_hit) {
+    if (!q_rot) {
+      rotate(qp);
+      q_rot = true;
+    }
+    if ((any_hit || (writer && !wrote)) && !k_rot) {
+      rotate(knew);
+      k_rot = true;
+    }
+    if (writer && !wrote) {
+      const uint32_t new_slot = new_slot_wait();  // outside the lane branch: the wait is wave-wide
+      if (g == 0) {
+        const uint32_t ns = new_slot > p.max_slot ? p.max_slot : new_slot;
+        char* dst = reinterpret_cast<char*>(const_cast<void*>(p.kv)) +
+                    (ns >> p.page_shift) * p.page_stride_b + (ns & entry_mask) * p.entry_stride_b +
+                    head_byte_off;
+        const u32x4 ko = {knew[0], knew[1], knew[2], knew[3]};
+        const u32x4 vo = {vnew[0], vnew[1], vnew[2], vnew[3]};
+        *reinterpret_cast<u32x4*>(dst) = ko;
+        *reinterpret_cast<u32x4*>(dst + p.v_offset * 2) = vo;
+      }
+      wrote = true;
+    }
+  };
+
+  const int STEP = n_splits * NW * TILE;
+  for (int t = t0; t < c1; t += STEP) {
+    if (t != t0) ent = fetch_entry(t);
+    // this lane's token: its slot, whether it exists, whether it is the token being decoded
+    const int i = t + own;
+    const bool valid = i < c1;
+    // ent was read at min(i, capacity - 1), which is i for every listed token (n_list <= capacity)
+    uint32_t slot = i < s.n_list ? (uint32_t)ent : last_base + (uint32_t)(i - s.n_list);
+    slot = slot > p.max_slot ? p.max_slot : slot;
+    uint32_t off_own = __umul24(slot >> p.page_shift, p.page_stride_b) +
+                       __umul24(slot & entry_mask, p.entry_stride_b);
+    // lanes past the end of the list repeat the first token of the tile (which exists: t < c1)
+    // with weight 0: a row that holds real data, whatever the unused list entries say
+    off_own = valid ? off_own : (uint32_t)__builtin_amdgcn_readfirstlane(off_own);
+
+    u32x4 kb[U], vb[U];
+    uint32_t offs[U];
+#define TD_ROW_OFF(N) \
+  if constexpr (N < U) offs[N] = row_bcast_u32<N>(off_own) + head_byte_off;
+    TD_ROW_OFF(0) TD_ROW_OFF(1) TD_ROW_OFF(2) TD_ROW_OFF(3) TD_ROW_OFF(4) TD_ROW_OFF(5)
+    TD_ROW_OFF(6) TD_ROW_OFF(7) TD_ROW_OFF(8) TD_ROW_OFF(9) TD_ROW_OFF(10) TD_ROW_OFF(11)
+    TD_ROW_OFF(12) TD_ROW_OFF(13) TD_ROW_OFF(14) TD_ROW_OFF(15)
+#undef TD_ROW_OFF
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      kb[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kbase + offs[u]));
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      vb[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vbase + offs[u]));
+
+    if constexpr (PROBE) {  // measurement: the loads alone, no arithmetic and no merge
+      u32x4 fold = {0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int u = 0; u < U; ++u) fold ^= kb[u] ^ vb[u];
+      uint32_t w = fold.x ^ fold.y ^ fold.z ^ fold.w;
+      if (w == 0x12345678u) reinterpret_cast<uint32_t*>(p.o)[0] = w;
+      continue;
+    }
+    bool hit = false;
+    if constexpr (FRESH) {
+      hit = slot == new_slot_wait();
+      const uint32_t hit_first = __builtin_amdgcn_readfirstlane(hit ? 1u : 0u);
+      hit = valid ? hit : (hit_first != 0);
+    }
+    if constexpr (FRESH) fresh_duties(__ballot(hit) != 0);  // behind the loads: hidden by their latency
+    // The token being decoded is used from registers wherever the list names its slot: what the
+    // pool holds there is being written by another workgroup of this launch.
+    if constexpr (FRESH) {
+      if (__ballot(hit)) {
+        const uint32_t hm = hit ? 1u : 0u;
+#define TD_ROW_FIX(N)                                                                   \
+  if constexpr (N < U) {                                                                \
+    if (row_bcast_u32<N>(hm)) {                                                         \
+      kb[N].x = knew[0]; kb[N].y = knew[1]; kb[N].z = knew[2]; kb[N].w = knew[3];       \
+      vb[N].x = vnew[0]; vb[N].y = vnew[1]; vb[N].z = vnew[2]; vb[N].w = vnew[3];       \
+    }                                                                                   \
+  }
+        TD_ROW_FIX(0) TD_ROW_FIX(1) TD_ROW_FIX(2) TD_ROW_FIX(3) TD_ROW_FIX(4) TD_ROW_FIX(5)
+        TD_ROW_FIX(6) TD_ROW_FIX(7) TD_ROW_FIX(8) TD_ROW_FIX(9) TD_ROW_FIX(10) TD_ROW_FIX(11)
+        TD_ROW_FIX(12) TD_ROW_FIX(13) TD_ROW_FIX(14) TD_ROW_FIX(15)
+#undef TD_ROW_FIX
+      }
+    }
+
+    // q.k: U partial sums per lane, reduce-scattered so that the lane ends with its own token
+    float part[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      float a = dot2<T>(qp[0], kb[u].x, 0.f);
+      a = dot2<T>(qp[1], kb[u].y, a);
+      a = dot2<T>(qp[2], kb[u].z, a);
+      part[u] = dot2<T>(qp[3], kb[u].w, a);
+    }
+    const float red = reduce_scatter_rows<U>(part, li);  // every lane takes part: no branch around it
+    const float sv = valid ? red * p.scale_log2 : kNegBig;
+    const float m_new = fmaxf(m_run, rows_max(row16_max(sv)));
+    const float alpha = fast_exp2(m_run - m_new);
+    m_run = m_new;
+    const float pr = valid ? fast_exp2(sv - m_new) : 0.f;
+    // with U == 8 the lanes li and li ^ 8 hold the same token: it counts once
+    l_lane = l_lane * alpha + ((U == 16 || li < 8) ? pr : 0.f);
+#pragma unroll
+    for (int d = 0; d < 8; ++d) acc[d] *= alpha;
+#define TD_ROW_PV(N)                                        \
+  if constexpr (N < U) {                                    \
+    const float pu = row_bcast_f32<N>(pr);                  \
+    float v0, v1, v2, v3, v4, v5, v6, v7;                   \
+    unpack2<T>(vb[N].x, v0, v1);                            \
+    unpack2<T>(vb[N].y, v2, v3);                            \
+    unpack2<T>(vb[N].z, v4, v5);                            \
+    unpack2<T>(vb[N].w, v6, v7);                            \
+    acc[0] = fmaf(pu, v0, acc[0]);                          \
+    acc[1] = fmaf(pu, v1, acc[1]);                          \
+    acc[2] = fmaf(pu, v2, acc[2]);                          \
+    acc[3] = fmaf(pu, v3, acc[3]);                          \
+    acc[4] = fmaf(pu, v4, acc[4]);                          \
+    acc[5] = fmaf(pu, v5, acc[5]);                          \
+    acc[6] = fmaf(pu, v6, acc[6]);                          \
+    acc[7] = fmaf(pu, v7, acc[7]);                          \
+  }
+    TD_ROW_PV(0) TD_ROW_PV(1) TD_ROW_PV(2) TD_ROW_PV(3) TD_ROW_PV(4) TD_ROW_PV(5) TD_ROW_PV(6)
+    TD_ROW_PV(7) TD_ROW_PV(8) TD_ROW_PV(9) TD_ROW_PV(10) TD_ROW_PV(11) TD_ROW_PV(12)
+    TD_ROW_PV(13) TD_ROW_PV(14) TD_ROW_PV(15)
+#undef TD_ROW_PV
+  }
+  if constexpr (FRESH) {
+    if (writer && !wrote) fresh_duties(false);  // a wave without tokens still owes the cache write
+  }
+
+  if constexpr (PROBE) return;
+  // ---- the four lane groups of the wave: the maximum is shared, so the sums simply add ----------
+  // reduce-scatter over the groups: lane (g, li) ends with dimensions li 8 + g 2 + {0, 1}
+  float r0, r1;
+  {
+    float x, y, h[4];
+#pragma unroll
+    for (int i2 = 0; i2 < 4; ++i2) {
+      swap32(acc[i2], acc[i2 + 4], x, y);
+      h[i2] = x + y;  // lower half: dimension i2, upper half: dimension i2 + 4
+    }
+    swap16(h[0], h[2], x, y);
+    r0 = x + y;
+    swap16(h[1], h[3], x, y);
+    r1 = x + y;
+  }
+  float l_w = rows_sum(group_sum<16>(l_lane));
+
+  // ---- the waves of the workgroup meet in LDS; wave 0 carries on alone ---------------------------
+  __shared__ __attribute__((aligned(16))) float sm_o[NW][D];
+  __shared__ float sm_ml[NW][2];
+  {
+    f32x2 v = {r0, r1};
+    *reinterpret_cast<f32x2*>(&sm_o[wave][li * 8 + g * 2]) = v;
+    if (lane == 0) {
+      sm_ml[wave][0] = m_run;
+      sm_ml[wave][1] = l_w;
+    }
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  float M = kNegBig;
+#pragma unroll
+  for (int w = 0; w < NW; ++w) M = fmaxf(M, sm_ml[w][0]);
+  float L = 0.f, o0 = 0.f, o1 = 0.f;  // this lane: dimensions 2 lane, 2 lane + 1
+#pragma unroll
+  for (int w = 0; w < NW; ++w) {
+    const float f = fast_exp2(sm_ml[w][0] - M);
+    L = fmaf(sm_ml[w][1], f, L);
+    const f32x2 v = *reinterpret_cast<const f32x2*>(&sm_o[w][2 * lane]);
+    o0 = fmaf(v.x, f, o0);
+    o1 = fmaf(v.y, f, o1);
+  }
+  uint32_t* o32 = reinterpret_cast<uint32_t*>(p.o) + ((int64_t)b * p.num_qo_heads + hrow) * (D / 2) + lane;
+  float* lse_out = p.lse ? p.lse + (int64_t)b * p.num_qo_heads + hrow : nullptr;
+  if (n_splits == 1) {
+    const float inv = L > 0.f ? 1.f / L : 0.f;
+    *o32 = pack2<T>(o0 * inv, o1 * inv);
+    if (lse_out && lane == 0) *lse_out = L > 0.f ? (M + fast_log2(L)) * kLn2 : -INFINITY;
+    return;
+  }
+  const int64_t part0 = ((int64_t)b * p.vheads + hrow) * p.max_splits;
+  store_coherent(p.ws_o + (part0 + split) * D + 2 * lane, o0, o1);
+  if (lane == 0) store_coherent(p.ws_ml + (part0 + split) * 2, M, L);
+  if (!p.fused_merge) return;
+
+  // ---- the last workgroup of this (sequence, head) to arrive reduces the partials ---------------
+  // Every partial of this workgroup was stored by this wave with device-coherent write-through
+  // stores; vmcnt(0) returns once they are acknowledged, and only then is the ticket taken.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  int32_t* ticket = p.ws_cnt + ((int64_t)b * gridDim.x + hrow) * p.ticket_stride;
+  int tk = 0;
+  if (lane == 0) tk = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  tk = __builtin_amdgcn_readfirstlane(tk);
+  if (tk != n_splits - 1) return;
+
+  float pm = kNegBig, pl = 0.f;  // (m, l) of split `lane`
+  {
+    const int sidx = lane < n_splits ? lane : n_splits - 1;
+    float a, c;
+    load_coherent(p.ws_ml + (part0 + sidx) * 2, a, c);
+    if (lane < n_splits) { pm = a; pl = c; }
+  }
+  constexpr int PRE = 16;  // partial loads in flight
+  float pa[PRE], pb[PRE];
+  auto issue = [&](int base) {
+#pragma unroll
+    for (int u = 0; u < PRE; ++u) {
+      int sidx = base + u;
+      sidx = sidx < n_splits ? sidx : n_splits - 1;
+      load_coherent(p.ws_o + (part0 + sidx) * D + 2 * lane, pa[u], pb[u]);
+    }
+  };
+  issue(0);
+  const float Mx = rows_max(row16_max(pm));
+  const float pf = fast_exp2(pm - Mx);  // scale of split `lane` (0 for lanes past the splits: pl = 0)
+  const float Lx = rows_sum(group_sum<16>(pl * pf));
+  float ra = 0.f, rb = 0.f;
+  for (int base = 0; base < n_splits; base += PRE) {
+    if (base) issue(base);
+#pragma unroll
+    for (int u = 0; u < PRE; ++u) {
+      const int sidx = base + u;  // uniform
+      if (sidx < n_splits) {
+        const float f = __builtin_bit_cast(
+            float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, pf), sidx));
+        ra = fmaf(pa[u], f, ra);
+        rb = fmaf(pb[u], f, rb);
+      }
+    }
+  }
+  const float inv = Lx > 0.f ? 1.f / Lx : 0.f;
+  *o32 = pack2<T>(ra * inv, rb * inv);
+  if (lse_out && lane == 0) *lse_out = Lx > 0.f ? (Mx + fast_log2(Lx)) * kLn2 : -INFINITY;
+  if (lane == 0) __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Shapes of the sparse-layer kernel: waves per workgroup x K (and V) rows per lane.
+static bool sparse_shape_supported(int nw, int rows) {
+  return (nw == 4 || nw == 8) && (rows == 8 || rows == 16);
+}
+
+template <typename T>
+static int launch_sparse(const DecodeParams& p, int nw, int rows, bool probe, dim3 grid, hipStream_t st) {
+#define TD_SPARSE_CASE(N_, U_)                                                                   \
+  if (nw == N_ && rows == U_) {                                                                  \
+    if (probe)                                                                                   \
+      hipLaunchKernelGGL((sparse_attn_kernel<T, N_, U_, false, true>), grid, dim3(N_ * 64), 0,   \
+                         st, p);                                                                 \
+    else if (p.fresh_k)                                                                          \
+      hipLaunchKernelGGL((sparse_attn_kernel<T, N_, U_, true>), grid, dim3(N_ * 64), 0, st, p);  \
+    else                                                                                         \
+      hipLaunchKernelGGL((sparse_attn_kernel<T, N_, U_, false>), grid, dim3(N_ * 64), 0, st, p); \
+    return TD_OK;                                                                                \
+  }
+  TD_SPARSE_CASE(8, 8)
+  TD_SPARSE_CASE(4, 8)
+  TD_SPARSE_CASE(4, 16)
+  TD_SPARSE_CASE(8, 16)
+#undef TD_SPARSE_CASE
+  return fail(TD_ERR_UNSUPPORTED, "sparse decode attention: no kernel for %d waves x %d rows", nw, rows);
+}
+
+// Launches the sparse-layer kernel (and, when the plan asks for it, the second-launch merge);
+// defined once per element type in sparse_attn_f16.hip / sparse_attn_bf16.hip.
+int launch_sparse_f16(const DecodeParams& p, int nw, int rows, bool probe, bool merge_kernel, dim3 grid,
+                      hipStream_t st);
+int launch_sparse_bf16(const DecodeParams& p, int nw, int rows, bool probe, bool merge_kernel, dim3 grid,
+                       hipStream_t st);
+
+}  // namespace tidal
