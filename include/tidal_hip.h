@@ -224,6 +224,26 @@ int td_decode_attn(const td_paged_kv* kv, const td_index_list* list, const td_de
                    void* stream);
 
 /*
+ * td_decode_attn for callers that cannot allocate device memory or be handed a workspace -- code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc: the ticket
+ * counters and split partials live in TD_STATIC_SCRATCH_BYTES of device memory inside the library
+ * image (one copy per GPU, held until the process ends).  Same arguments, kernels and results as
+ * td_decode_attn without `workspace` / `workspace_bytes`; a plan whose workspace_bytes exceeds
+ * TD_STATIC_SCRATCH_BYTES is rejected with TD_ERR_STATE.  Calls no hipMalloc / hipFree.  All calls
+ * on one GPU share that GPU's scratch: they must be ordered on one stream (calls that overlap
+ * race), and they must not be mixed on another stream with in-flight calls of this entry point.
+ * The scratch starts zeroed and every launch leaves its counters zeroed, so nothing is cleared per
+ * call.  No counterpart in the reference, whose handler allocates its scratch in every
+ * BeginForward (kernels/include/decode/decode_handler.cuh:39-121).
+ */
+#define TD_STATIC_SCRATCH_BYTES (4 << 20)
+int td_decode_attn_noalloc(const td_paged_kv* kv, const td_index_list* list,
+                           const td_decode_plan* plan, const void* q, void* o, int32_t batch,
+                           int32_t num_qo_heads, float sm_scale, void* scores, int32_t scores_dtype,
+                           int64_t score_stride, float* lse, const td_fresh_token* fresh,
+                           void* stream);
+
+/*
  * cos[b, j] / sin[b, j] of positions[b] / rope_scale * rope_theta^(-2j/head_dim), j < head_dim/2
  * (angles formed in double precision, as td_rope_in_place does).  One launch per decode step
  * serves every layer's fused td_decode_attn.

@@ -485,6 +485,9 @@ class BatchDecodeWithPagedKVCachePyTorchWrapper:
         self.tile_rows = 0        # 0 = library default
         self.sparse_waves = 0     # short-list kernel: 0 = library default, -1 = never
         self.sparse_rows = 0
+        # True: forward() goes through td_decode_attn_noalloc (scratch inside the library image,
+        # no workspace tensor) -- for callers that must not allocate
+        self.static_scratch = False
 
     def begin_forward(self, indptr: torch.Tensor, num_qo_heads: int, num_kv_heads: int,
                       head_dim: int, page_size: int, empty_data: torch.Tensor) -> None:
@@ -601,7 +604,7 @@ class BatchDecodeWithPagedKVCachePyTorchWrapper:
         max_items = lst.n_list_host * (page if kind == TD_IDX_PAGES else 1) + max_last
         has_scores = qk_product is not None and qk_product.numel() > 0
         plan = self._plan(batch, rows, max_items, kind == TD_IDX_SLOTS and not has_scores)
-        if plan.workspace_bytes > 0 and (self._workspace is None or
+        if not self.static_scratch and plan.workspace_bytes > 0 and (self._workspace is None or
                                          self._workspace.numel() < plan.workspace_bytes or
                                          self._workspace.device != q.device):
             self._workspace = torch.zeros(int(plan.workspace_bytes), dtype=torch.uint8,
@@ -641,6 +644,11 @@ class BatchDecodeWithPagedKVCachePyTorchWrapper:
                 raise RuntimeError("fresh dst_slot must hold one entry per sequence")
             fresh_arg = FreshToken(fk.data_ptr(), fv.data_ptr(), fcos.data_ptr(), fsin.data_ptr(),
                                    fslot.data_ptr())
+        if self.static_scratch:
+            check(lib.td_decode_attn_noalloc(pool, lst, plan, q.data_ptr(), o.data_ptr(), batch, hq,
+                                             1.0 / math.sqrt(d), scores_ptr, scores_dtype,
+                                             score_stride, lse_ptr, fresh_arg, _stream()))
+            return
         ws = self._workspace
         check(lib.td_decode_attn(pool, lst, plan, q.data_ptr(), o.data_ptr(), batch, hq,
                                  1.0 / math.sqrt(d), scores_ptr, scores_dtype, score_stride,

@@ -16,6 +16,7 @@ TD_F16, TD_BF16, TD_F32 = 0, 1, 2
 TD_NHD, TD_HND = 0, 1
 TD_IDX_PAGES, TD_IDX_SLOTS = 0, 1
 TD_REDUCE_HEAD_SUM, TD_REDUCE_GROUP_SUM = 0, 1
+TD_STATIC_SCRATCH_BYTES = 4 << 20  # scratch inside the library image (td_decode_attn_noalloc)
 # words of the device-resident step state (td_step_advance)
 (TD_STEP_SEQ_LEN, TD_STEP_PAGES_BEFORE_LAST, TD_STEP_LAST_PAGE_LEN, TD_STEP_LAST_PAGE_IDX,
  TD_STEP_DST_SLOT, TD_STEP_POSITION, TD_STEP_N_SELECTED, TD_STEP_COUNT, TD_STEP_WORDS) = range(9)
@@ -109,6 +110,11 @@ SIGNATURES = {
         [POINTER(PagedKV), POINTER(IndexList), POINTER(DecodePlan), c_void_p, c_void_p, c_int32,
          c_int32, c_float, c_void_p, c_int32, c_int64, c_void_p, POINTER(FreshToken), c_void_p,
          c_int64, c_void_p],
+    ),
+    "td_decode_attn_noalloc": (
+        c_int32,
+        [POINTER(PagedKV), POINTER(IndexList), POINTER(DecodePlan), c_void_p, c_void_p, c_int32,
+         c_int32, c_float, c_void_p, c_int32, c_int64, c_void_p, POINTER(FreshToken), c_void_p],
     ),
     "td_merge_states": (
         c_int32,

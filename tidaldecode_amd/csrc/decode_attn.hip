@@ -37,6 +37,35 @@ static bool is_pow2(int64_t x) { return x > 0 && (x & (x - 1)) == 0; }
 
 }  // namespace tidal
 
+// Scratch of td_decode_attn_noalloc: ticket counters and split partials in device memory that
+// belongs to the library image, for callers that must not allocate.  Zero when the image is
+// loaded; every launch leaves the ticket counters zero again.
+static __device__ __align__(256) unsigned char scratch[TD_STATIC_SCRATCH_BYTES];
+
+namespace tidal {
+
+// Device address of `scratch` on the current device.  The array's name is a host-side handle, not
+// a device address: the address is looked up once per device (each device holds its own copy)
+// and that pointer is what the launches get.
+static int static_scratch(void** out) {
+  constexpr int kMaxDevices = 64;
+  static void* ptr_of[kMaxDevices] = {};
+  int dev = 0;
+  TD_HIP_CHECK(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices)
+    return fail(TD_ERR_UNSUPPORTED, "td_decode_attn_noalloc: device %d (at most %d devices)", dev, kMaxDevices);
+  void* ptr = __atomic_load_n(&ptr_of[dev], __ATOMIC_ACQUIRE);
+  if (ptr == nullptr) {
+    TD_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (ptr == nullptr) return fail(TD_ERR_HIP, "hipGetSymbolAddress returned a NULL scratch address");
+    __atomic_store_n(&ptr_of[dev], ptr, __ATOMIC_RELEASE);
+  }
+  *out = ptr;
+  return TD_OK;
+}
+
+}  // namespace tidal
+
 using namespace tidal;
 
 extern "C" int td_num_cus(void) { return num_cus(); }
@@ -61,6 +90,13 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
   const int qpg = qpg_for(num_qo_heads, num_kv_heads, idx_rows, head_dim);
   const int subs = qpg > 1 ? (num_qo_heads / num_kv_heads + qpg - 1) / qpg : 1;
   const int n_hrows = qpg > 1 ? num_kv_heads * subs : num_qo_heads;
+  {
+    // Planning happens before the launches it serves (and outside any stream capture): a good
+    // moment to look up this device's static scratch for td_decode_attn_noalloc.  Without a
+    // device the lookup fails and is simply tried again by that entry point.
+    void* unused = nullptr;
+    (void)static_scratch(&unused);
+  }
 
   // ---- short lists: the sparse-layer kernel -------------------------------------------------------
   // Chunks are a power of two (the kernel divides by shifting) and a multiple of the workgroup
@@ -369,6 +405,24 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
   if (rc != TD_OK) return rc;
   TD_HIP_CHECK(hipGetLastError());
   return TD_OK;
+}
+
+extern "C" int td_decode_attn_noalloc(const td_paged_kv* kv, const td_index_list* list,
+                                      const td_decode_plan* plan, const void* q, void* o,
+                                      int32_t batch, int32_t num_qo_heads, float sm_scale,
+                                      void* scores, int32_t scores_dtype, int64_t score_stride,
+                                      float* lse, const td_fresh_token* fresh, void* stream) {
+  TD_REQUIRE(plan != nullptr, "td_decode_attn_noalloc: plan is NULL");
+  if (plan->workspace_bytes > (int64_t)TD_STATIC_SCRATCH_BYTES)
+    return fail(TD_ERR_STATE,
+                "td_decode_attn_noalloc: the plan needs %lld bytes of scratch, the built-in scratch holds "
+                "%lld (fewer sequences, heads or splits, or td_decode_attn with a workspace)",
+                (long long)plan->workspace_bytes, (long long)TD_STATIC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  const int rc = static_scratch(&ws);
+  if (rc != TD_OK) return rc;
+  return td_decode_attn(kv, list, plan, q, o, batch, num_qo_heads, sm_scale, scores, scores_dtype,
+                        score_stride, lse, fresh, ws, (int64_t)TD_STATIC_SCRATCH_BYTES, stream);
 }
 
 // ---------------------------------------------------------------------------------------------
