@@ -3,7 +3,7 @@ selection and one sparse layer through the operator surface, against the CPU ora
 
   cfg1  Llama-2-7B shape: 32/32 heads x 128, bf16, page 16, 32768 (+1) tokens, top_k 2048
   cfg2  GQA 32/8, 102400 tokens, top_k 4096
-  cfg4  40/40 heads, 32768 tokens, top_k 2048
+  cfg4  40/40 heads, 10240 / 32768 / 102400 tokens, top_k 2048
 
 The oracle's sparse layer gathers the selected rows (equal to the reference's masked dense form,
 pinned in tests/test_oracle.py), so it finishes in seconds at these sizes.  Index sets are
@@ -25,6 +25,8 @@ pytestmark = pytest.mark.gpu
     ("cfg2", 32, 8, 102400, 4096, "per_head", torch.bfloat16),
     ("cfg2-group", 32, 8, 102400, 4096, "group_sum", torch.float16),
     ("cfg4", 40, 40, 32768, 2048, "per_head", torch.float16),
+    ("cfg4-10k", 40, 40, 10240, 2048, "per_head", torch.bfloat16),
+    ("cfg4-100k", 40, 40, 102400, 2048, "per_head", torch.bfloat16),
 ])
 def test_selection_topk_sparse_at_full_size(cuda, name, hq, hkv, n, k, mode, dtype):
     from oracle import tidal_oracle as orc

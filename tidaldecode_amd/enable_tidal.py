@@ -14,8 +14,13 @@ on the model, and the persisted selection is the token list inside that state:
     decode, layer == sparse_layer_start / correction   full attention + logits -> top-k
     decode, other layers                               sparse attention over the persisted list
 
-Rotary embedding uses the cos/sin the model computes, so every RoPE variant of the model works.
-Batch size 1, as the reference's kernel path (tidal/ops/csrc/approx_attn.cu:33,78).
+Rotary embedding uses the cos/sin the model computes, so every RoPE variant of the model works;
+in decode steps they go, with the un-rotated q and k, into the fused launch (RoPE + cache append +
+attention in one kernel) wherever the cache geometry allows it.  Batch size 1 and no padding, as
+the reference's kernel path (tidal/ops/csrc/approx_attn.cu:33,78): ``attention_mask`` is not
+consulted, the attention is causal over everything cached.  As in the reference
+(modify_llama.py:365-367) ``forward`` is replaced only for ``attn_type == "tidal"``; any other value
+just leaves the original under ``flash_forward``.
 """
 import types
 from typing import Optional
@@ -41,6 +46,7 @@ class TidalState:
         self.first_layer = None
         self.last_layer = None
         self.step_len = 0
+        self.dst_slot = None   # device int32 [1]: slot of the token being decoded (fused step)
 
     def layer_kind(self, layer_idx: int) -> str:
         if layer_idx < self.sparse_layer_start:
@@ -84,35 +90,53 @@ def _tidal_attention_forward(self, hidden_states, position_embeddings=None, atte
     k = self.k_proj(hidden_states).view(q_len, hkv, d)
     v = self.v_proj(hidden_states).view(q_len, hkv, d).contiguous()
     cos, sin = position_embeddings  # [1, q_len, D]
-    cos, sin = cos[0].unsqueeze(1), sin[0].unsqueeze(1)
-    q = (q * cos + _rotate_half(q) * sin).contiguous()
-    k = (k * cos + _rotate_half(k) * sin).contiguous()
 
     if self.layer_idx == state.first_layer:
-        # a model forward starts: a fresh prompt restarts the cache
-        if q_len > 1 and (past_key_values is None
-                          or past_key_values.get_seq_length(self.layer_idx) == 0):
+        # a model forward starts; whenever the framework's cache is empty (or absent) it is a new
+        # sequence and the paged cache starts over, whatever the length of the input
+        if past_key_values is None or past_key_values.get_seq_length(self.layer_idx) == 0:
             state.reset()
         ctrl.prepare_metadata(q_len)
         ctrl.begin_forward(q_len)
         state.step_len = q_len
+        if q_len == 1 and ctrl.fused_step_ok:
+            pos = ctrl.kv_cache.seqlen - 1
+            slot = ctrl.kv_cache.indicies[pos // ctrl.page_size] * ctrl.page_size + pos % ctrl.page_size
+            state.dst_slot = torch.tensor([slot], dtype=torch.int32, device=hidden_states.device)
+    fused = q_len == 1 and ctrl.fused_step_ok
+    if fused:
+        # the launch rotates q and k itself, with the model's own cos/sin (first half of the
+        # duplicated table), and writes k, v into the cache
+        half = d // 2
+        fresh = (k.contiguous(), v, cos[0, :, :half].float().contiguous(),
+                 sin[0, :, :half].float().contiguous(), state.dst_slot)
+        k_cache = k
+        q = q.contiguous()
+    else:
+        fresh = None
+        cos, sin = cos[0].unsqueeze(1), sin[0].unsqueeze(1)
+        q = (q * cos + _rotate_half(q) * sin).contiguous()
+        k = (k * cos + _rotate_half(k) * sin).contiguous()
+        k_cache = k
     if past_key_values is not None:
         # keep the framework's cache length in step (generation code derives positions from it);
         # one element per row is enough for that, the real K/V live in the paged cache
-        past_key_values.update(k.transpose(0, 1)[None, :, :, :1], v.transpose(0, 1)[None, :, :, :1],
-                               self.layer_idx)
+        past_key_values.update(k_cache.transpose(0, 1)[None, :, :, :1],
+                               v.transpose(0, 1)[None, :, :, :1], self.layer_idx)
 
-    tidal_utils.append_kv(k, v, ctrl, self.layer_idx)
+    if not fused:
+        tidal_utils.append_kv(k, v, ctrl, self.layer_idx)
     if q_len > 1:
         o = tidal_utils.prefill_forward(q, ctrl, self.layer_idx)
     else:
         kind = state.layer_kind(self.layer_idx)
         if kind == "sparse":
             o = tidal_utils.decode_sparse_attn(q, ctrl, self.layer_idx, ctrl.topk_dindices_buffer,
-                                               False)
+                                               False, fresh=fresh)
         else:
             o = tidal_utils.decode_sparse_attn(q, ctrl, self.layer_idx,
-                                               ctrl.kv_indices_without_last, kind == "select")
+                                               ctrl.kv_indices_without_last, kind == "select",
+                                               fresh=fresh)
             if kind == "select":
                 tidal_utils.decode_topk(ctrl)
     if self.layer_idx == state.last_layer:
@@ -122,8 +146,10 @@ def _tidal_attention_forward(self, hidden_states, position_embeddings=None, atte
 
 
 def enable_llama_tidal_attention(model, top_k, attn_type="tidal", sparse_layer_start=2,
-                                 correction_layer=13, *, page_size=16, max_seq_len=None,
+                                 correction_layer=9, *, page_size=16, max_seq_len=None,
                                  select_mode="per_head"):
+    """Arguments and defaults of the reference's function of this name (modify_llama.py:331-333:
+    ``correction_layer=9`` here, 13 in ``enable_tidal``)."""
     state = TidalState(top_k, sparse_layer_start, correction_layer, page_size, max_seq_len,
                        select_mode)
     layers = []
@@ -137,7 +163,8 @@ def enable_llama_tidal_attention(model, top_k, attn_type="tidal", sparse_layer_s
     for module in layers:
         module._tidal_state = state
         module.flash_forward = module.forward  # the reference keeps the original under this name
-        module.forward = types.MethodType(_tidal_attention_forward, module)
+        if attn_type == "tidal":                # modify_llama.py:365-367
+            module.forward = types.MethodType(_tidal_attention_forward, module)
     model._tidal_state = state
     return state
 
