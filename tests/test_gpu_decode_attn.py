@@ -170,11 +170,18 @@ def test_full_attention_with_scores(cuda, dtype, hq, hkv, n):
     err = (got_logits - logits).abs()
     if err.max() > bound:   # say where, and whether a second launch gives the same value
         h, i = divmod(int(err.argmax()), n)
+        # where the kernel computed it: workgroup tiles of 8 waves x 16 tokens are dealt to the
+        # splits round robin, a wave keeps its logits in a strip of tiles until it is flushed
+        plan = w._plan(1, 1, (case.n_pages - 1) * page_size + case.last_page_len, False)
+        wg_tokens = plan.waves_per_block * plan.tile_rows * 4
+        n_splits = -(-n // plan.chunk_tokens)
+        where = (f"split {(i // wg_tokens) % n_splits} of {n_splits}, wave {(i % wg_tokens) // (plan.tile_rows * 4)}, "
+                 f"tile {(i // wg_tokens) // n_splits} of that wave, row {i % (plan.tile_rows * 4)} of the tile")
         scores2 = torch.full_like(scores, float("nan"))
         w.forward(qd, od, case.pool.to(cuda), table.to(cuda), None, case.last_page_len,
                   int(case.page_table[-1]), scores2, lse=lse)
         torch.cuda.synchronize()
-        raise AssertionError(f"logit of head {h}, token {i}: {got_logits[h, i].item()!r}, oracle "
+        raise AssertionError(f"logit of head {h}, token {i} ({where}): {got_logits[h, i].item()!r}, oracle "
                              f"{logits[h, i].item()!r}, second launch {scores2[h, i].item()!r}; "
                              f"{int((err > bound).sum())} entries beyond {bound:.2e}")
     assert torch.isnan(scores[:, n:]).all()  # nothing written past the sequence
@@ -336,6 +343,38 @@ def test_out_of_range_indices_are_clamped_not_faulting(cuda):
     w.forward(qd, od, case.pool.to(cuda), bad, None, 0, 0, None, index_kind="slots")
     torch.cuda.synchronize()
     assert torch.isfinite(od.float()).all()
+
+
+@pytest.mark.parametrize("index_kind", ["pages", "slots"])
+def test_poisoned_device_lengths_leave_the_tickets_clean(cuda, index_kind):
+    """Lengths that live on the device are not trusted: a last-page fill beyond the page size is
+    read as a full page (both kernels), every workgroup that runs finds its ticket taken care
+    of, and the counters are zero again afterwards -- a later call is not disturbed."""
+    from oracle import tidal_oracle as orc
+
+    dtype, h, d, page_size, n = torch.float16, 8, 128, 16, 3000
+    case = PagedCase(n, h, d, page_size, dtype, seed=41)
+    pool = case.pool.to(cuda)
+    qd = randn((1, h, d), 1, dtype).to(dtype).to(cuda)
+    w = _wrapper(0, h, h, d, page_size, dtype)
+    if index_kind == "pages":
+        lists = case.page_table[:-1].to(torch.int32).unsqueeze(0).to(cuda)
+    else:
+        g = torch.Generator().manual_seed(7)
+        pos = torch.stack([torch.randperm((case.n_pages - 1) * page_size, generator=g)[:500] for _ in range(h)])
+        lists = case.slots_of(pos).to(torch.int32).to(cuda)
+    indptr = torch.tensor([0, lists.shape[1]], dtype=torch.int32, device=cuda)
+    li = torch.tensor([int(case.page_table[-1])], dtype=torch.int32, device=cuda)
+    outs = []
+    for fill in (10 ** 6, page_size, -3, 0):
+        ll = torch.tensor([fill], dtype=torch.int32, device=cuda)
+        o = torch.full_like(qd, float("nan"))
+        w.forward(qd, o, pool, lists, indptr, ll, li, None, index_kind=index_kind)
+        torch.cuda.synchronize()
+        assert torch.isfinite(o.float()).all()
+        assert int(w._workspace[: 1 << 20].view(torch.int32).abs().sum()) == 0
+        outs.append(o)
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[2], outs[3])
 
 
 def test_error_paths(cuda):

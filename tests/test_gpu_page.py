@@ -163,6 +163,27 @@ def test_multi_turn_append_round_trip(cuda):
     assert torch.equal(kk, case.k) and torch.equal(vv, case.v)
 
 
+def test_fused_rope_append_keeps_a_bad_slot_inside_the_pool(cuda):
+    """A destination slot beyond the pool is written into the pool's last page (the clamp the
+    attention launch applies as well) and nowhere else."""
+    from tidaldecode_amd import _kernels
+
+    dtype, hq, hkv, d, page_size, pages = torch.float16, 8, 8, 128, 16, 4
+    pool = torch.full((pages, 2, page_size, hkv, d), 3.0, dtype=dtype, device=cuda)
+    q = randn((1, hq, d), 1, dtype).to(dtype).to(cuda)
+    k = randn((1, hkv, d), 2, dtype).to(dtype).to(cuda)
+    v = randn((1, hkv, d), 3, dtype).to(dtype).to(cuda)
+    pos = torch.zeros(1, dtype=torch.int32, device=cuda)           # position 0: the rotation is the identity
+    bad = torch.tensor([1000 * page_size + 5], dtype=torch.int32, device=cuda)
+    _kernels.rope_append_decode(q, k, v, pool, pos, bad, 0, 1.0, 1e4)
+    torch.cuda.synchronize()
+    assert (pool[: pages - 1] == 3.0).all()
+    assert torch.equal(pool[pages - 1, 0, 5], k[0]) and torch.equal(pool[pages - 1, 1, 5], v[0])
+    untouched = torch.ones(page_size, dtype=torch.bool)
+    untouched[5] = False
+    assert (pool[pages - 1][:, untouched] == 3.0).all()
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("layout", [0, 1])
 def test_fused_rope_append_equals_the_two_calls(cuda, dtype, layout):

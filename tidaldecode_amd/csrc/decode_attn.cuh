@@ -483,6 +483,12 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
   const int emit_step = n_splits * NW * TILE;  // tokens between two tiles of this wave
   auto emit_flush = [&]() {
     if constexpr (EMIT) {
+      // The strip was written by other lanes of this wave than the ones that now read it.  LDS
+      // accesses of one wave complete in issue order, so the reads below see those writes; the
+      // explicit wait and the wave barrier say so to the reader and pin the order for the
+      // compiler as well (one wait per flush, that is per 16-64 tiles).
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_wave_barrier();
       // a store instruction covers 64 / TILE tiles of one head: lane -> (tile, token)
       constexpr int TPS = 64 / TILE >= 1 ? 64 / TILE : 1;  // tiles per store (TILE <= 64)
       const int lt = lane / TILE, ltok = lane % TILE;

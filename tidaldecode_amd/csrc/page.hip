@@ -107,8 +107,9 @@ __global__ __launch_bounds__(256) void rope_append_decode_kernel(
   const int slots = 256 / half;
   if (slot >= slots) return;
   const uint32_t dst = (uint32_t)dst_slot[b];
-  const uint32_t page = dst / (uint32_t)g.page_size;
+  uint32_t page = dst / (uint32_t)g.page_size;
   const int entry = (int)(dst - page * (uint32_t)g.page_size);
+  page = page > g.max_page ? g.max_page : page;  // a bad slot lands inside the pool, as in the fused step
   float sn, cs;
   rope_sincos((double)positions[b] * inv_scale, log2_theta, j, D, sn, cs);
   uint16_t* pool = reinterpret_cast<uint16_t*>(g.data);
