@@ -285,3 +285,99 @@ def test_plans_of_both_kernels_share_one_workspace(cuda):
         assert tolerance_report(od[0], want_full) <= ATOL[dtype], k
         assert tolerance_report(os_[0], want) <= ATOL[dtype], k
         assert int(w._workspace[: 1 << 20].view(torch.int32).abs().sum()) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("hq,hkv,rows", [(8, 4, 4), (16, 4, 4), (32, 4, 4), (16, 4, 1), (32, 8, 8), (64, 8, 8)])
+@pytest.mark.parametrize("sw", [4, 8])
+def test_shared_kv_rows(cuda, dtype, hq, hkv, rows, sw):
+    """Grouped queries whose 2, 4 or 8 query heads share the list of their KV head (or one list for
+    all): one walk of the list per KV head, the group's heads scored against every loaded row,
+    p.V on the matrix cores.  Lengths around the tile edges, forced last page, both merges, several
+    tiles per wave; oracle and streaming kernel as above."""
+    from oracle import tidal_oracle as orc
+
+    d, page, n = 128, 16, 3000 + 7
+    case = PagedCase(n, hkv, d, page, dtype, seed=hq + hkv + rows)
+    pool = case.pool.to(cuda)
+    q = randn((hq, d), 3, dtype)
+    qd = q.to(dtype).to(cuda).unsqueeze(0)
+    before_last = (case.n_pages - 1) * page
+    g = torch.Generator().manual_seed(2)
+    gen = _wrapper(0, hq, hkv, d, page, dtype, sparse_waves=-1)
+    tile = sw * 32
+    for k, knobs in [(1, {}), (31, {}), (tile, {}), (tile + 1, {}), (700, {}), (700, dict(fused_merge=0)),
+                     (2500, dict(chunk_tokens=1024)), (2048, {})]:
+        w = _wrapper(0, hq, hkv, d, page, dtype, sparse_waves=sw, sparse_rows=8, **knobs)
+        pos = torch.stack([torch.randperm(before_last, generator=g)[:k] for _ in range(rows)])
+        assert _uses_short_list_kernel(w, 1, rows, k + case.last_page_len)
+        slots = case.slots_of(pos).to(torch.int32).to(cuda).contiguous()
+        allpos = torch.cat([pos, torch.arange(before_last, n).repeat(rows, 1)], 1)
+        want = orc.sparse_layer_gather(q, case.k, case.v, allpos)
+        od = torch.full_like(qd, float("nan"))
+        lse = torch.full((1, hq), float("nan"), dtype=torch.float32, device=cuda)
+        og = torch.full_like(qd, float("nan"))
+        for _ in range(2):   # twice: the tickets and partial buffers are reused
+            w.forward(qd, od, pool, slots, None, case.last_page_len, int(case.page_table[-1]), None,
+                      index_kind="slots", lse=lse)
+        gen.forward(qd, og, pool, slots, None, case.last_page_len, int(case.page_table[-1]), None,
+                    index_kind="slots")
+        torch.cuda.synchronize()
+        assert tolerance_report(od[0], want) <= ATOL[dtype], (k, knobs)
+        assert (od.float() - og.float()).abs().max().item() <= ATOL[dtype] / 2, (k, knobs)
+        logits = orc.attn_logits(q, case.k)
+        rows_of_heads = torch.arange(hq) * rows // hq
+        want_lse = torch.logsumexp(torch.gather(logits, 1, allpos[rows_of_heads]), -1)
+        assert (lse[0].cpu() - want_lse).abs().max() <= 1e-3, (k, knobs)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("hq,hkv", [(8, 4), (16, 4), (32, 4)])
+def test_fused_decode_step_with_shared_kv_rows(cuda, dtype, hq, hkv):
+    from tidaldecode_amd import _kernels
+
+    d, page, n, b = 128, 16, 1500, 2
+    for k in (1, 40, 700):
+        cases = [PagedCase(n, hkv, d, page, dtype, seed=40 + i, spare=0, shuffle=False) for i in range(b)]
+        npg = cases[0].n_pages
+        pool = torch.cat([c.pool for c in cases]).to(cuda)
+        offs = [0, npg]
+        q = randn((b, hq, d), 1, dtype).to(dtype).to(cuda)
+        knew = randn((b, hkv, d), 2, dtype).to(dtype).to(cuda)
+        vnew = randn((b, hkv, d), 3, dtype).to(dtype).to(cuda)
+        positions = torch.tensor([n - 1, 31000], dtype=torch.int32, device=cuda)
+        last_len = (n - 1) % page + 1
+        last_idx = torch.tensor([offs[i] + npg - 1 for i in range(b)], dtype=torch.int32, device=cuda)
+        dst = (last_idx * page + last_len - 1).to(torch.int32)
+        g = torch.Generator().manual_seed(5 + k)
+        lists = []
+        for i in range(b):
+            pos = torch.stack([torch.randperm(n - 1, generator=g)[: k - 1] for _ in range(hkv)])
+            pos = torch.cat([pos, torch.full((hkv, 1), n - 1)], 1)[:, torch.randperm(k, generator=g)]
+            lists.append(pos + offs[i] * page)
+        idx = torch.cat(lists, 1).to(torch.int32).to(cuda).contiguous()
+        indptr = torch.tensor([0, k, 2 * k], dtype=torch.int32, device=cuda)
+        zeros = torch.zeros(b, dtype=torch.int32, device=cuda)
+        w = _wrapper(0, hq, hkv, d, page, dtype)
+        assert _uses_short_list_kernel(w, b, hkv, k)
+
+        def run(fused):
+            pl, qq, o = pool.clone(), q.clone(), torch.full_like(q, float("nan"))
+            if fused:
+                cos, sin = _kernels.rope_table(positions, d, 1.0, 5e5)
+                w.forward(qq, o, pl, idx, indptr, zeros, zeros, None, index_kind="slots", n_list=k,
+                          fresh=(knew, vnew, cos, sin, dst))
+                assert torch.equal(qq, q)
+            else:
+                _kernels.rope_append_decode(qq, knew, vnew, pl, positions, dst, 0, 1.0, 5e5)
+                w.forward(qq, o, pl, idx, indptr, zeros, zeros, None, index_kind="slots", n_list=k)
+            torch.cuda.synchronize()
+            return o, pl
+
+        o1, p1 = run(False)
+        o2, p2 = run(True)
+        assert (o1.float() - o2.float()).abs().max().item() <= ATOL[dtype], k
+        ulp = {torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}[dtype]
+        assert ((p2.float() - p1.float()).abs() <= ulp * p1.float().abs() + 1e-6).all()
+        changed = (p1 != pool).any(dim=(1, 2, 3, 4)).nonzero().flatten().tolist()
+        assert changed == sorted(set(last_idx.tolist()))

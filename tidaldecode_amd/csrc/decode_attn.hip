@@ -103,9 +103,14 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
   // tile; the streaming kernel at 8 waves x 4 rows (tile 128) can run the same plan when a call
   // turns out not to fit the short-list kernel (page lists, score output, large pools).
   int sw = plan->sparse_waves, sr = plan->sparse_rows;
-  bool sparse = sw >= 0 && sr >= 0 && head_dim == 128 && qpg == 1 &&
-                is_pow2(num_qo_heads / num_kv_heads) && max_items > 0 && max_items <= kSparseMaxItems &&
+  // one query head per list walk with a power-of-two group size, or exactly 2, 4 or 8 query heads
+  // sharing their KV head's list (no padding heads)
+  const int group = num_qo_heads / num_kv_heads;
+  const bool heads_fit = qpg == 1 ? is_pow2(group) : (qpg == group && subs == 1);
+  bool sparse = sw >= 0 && sr >= 0 && head_dim == 128 && heads_fit && max_items > 0 &&
+                max_items <= kSparseMaxItems &&
                 (plan->chunk_tokens == 0 || is_pow2(plan->chunk_tokens));
+  if (qpg > 1 && sr == 16) sparse = false;  // shared rows: 8 rows per lane only
   if (sparse) {
     // Chunk: the smallest power of two from 128 tokens up that leaves at most 9/8 workgroups per
     // compute unit, but no more than 512 tokens -- the waves of this kernel do not pipeline their
@@ -121,7 +126,7 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
     while (ceil_div64(max_items, chunk) > 64) chunk <<= 1;
     if (sr == 0) sr = 8;
     if (sw == 0) sw = (chunk < 256 || sr == 16) ? 4 : 8;
-    if (!sparse_shape_supported(sw, sr))
+    if (!sparse_shape_supported(sw, sr, qpg))
       return fail(TD_ERR_UNSUPPORTED,
                   "td_decode_make_plan: no short-list kernel with %d waves x %d rows (4 or 8 waves, 8 or "
                   "16 rows)", sw, sr);
@@ -141,10 +146,10 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
   if (sparse) {
     if (plan->fused_merge < 0) plan->fused_merge = 1;
     plan->fused_merge = plan->fused_merge ? 1 : 0;
-    TD_REQUIRE((int64_t)batch * n_hrows * kTicketStride * 4 <= kTicketBytes,
-               "td_decode_make_plan: batch %d x %d head rows exceeds the %lld ticket counters", batch,
-               n_hrows, (long long)(kTicketBytes / (kTicketStride * 4)));
-    const int64_t n_part = (int64_t)batch * n_hrows * plan->max_splits;
+    TD_REQUIRE((int64_t)batch * n_hrows * qpg * kTicketStride * 4 <= kTicketBytes,
+               "td_decode_make_plan: batch %d x %d heads exceeds the %lld ticket counters", batch,
+               n_hrows * qpg, (long long)(kTicketBytes / (kTicketStride * 4)));
+    const int64_t n_part = (int64_t)batch * n_hrows * qpg * plan->max_splits;
     plan->workspace_bytes = kTicketBytes + align256(n_part * head_dim * 4) + align256(n_part * 2 * 4);
     return TD_OK;
   }
@@ -362,11 +367,12 @@ static int build_params(const td_paged_kv* kv, const td_index_list* list, const 
 // score output, chunks that are a power-of-two multiple of the kernel's workgroup tile.
 static bool sparse_kernel_fits(const DecodeParams& p, const td_decode_plan* plan,
                                const td_index_list* list, int qpg, int head_dim, bool emit) {
-  if (plan->sparse_waves <= 0 || !sparse_shape_supported(plan->sparse_waves, plan->sparse_rows))
+  if (plan->sparse_waves <= 0 || !sparse_shape_supported(plan->sparse_waves, plan->sparse_rows, qpg))
     return false;
   const int stile = plan->sparse_waves * 4 * plan->sparse_rows;
-  return list->kind == TD_IDX_SLOTS && p.lean && !emit && qpg == 1 && head_dim == 128 &&
-         p.chunk_shift >= 0 && p.qpk_shift >= 0 && plan->chunk_tokens % stile == 0 &&
+  const bool heads_fit = qpg == 1 ? p.qpk_shift >= 0 : (p.q_per_kv == qpg && p.subs == 1);
+  return list->kind == TD_IDX_SLOTS && p.lean && !emit && heads_fit && head_dim == 128 &&
+         p.chunk_shift >= 0 && plan->chunk_tokens % stile == 0 &&
          p.page_stride_b < (1u << 24) && p.entry_stride_b < (1u << 24);
 }
 
@@ -388,7 +394,13 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
   const bool merge_kernel = plan->max_splits > 1 && !plan->fused_merge;
   int rc;
   if (sparse_kernel_fits(p, plan, list, qpg, D, scores != nullptr)) {
-    if (kv->dtype == TD_F16)
+    TD_REQUIRE((int64_t)batch * n_hrows * qpg * kTicketStride * 4 <= kTicketBytes,
+               "td_decode_attn: batch %d x %d heads exceeds the ticket counters", batch, n_hrows * qpg);
+    if (qpg > 1)
+      rc = kv->dtype == TD_F16
+               ? launch_sparse_shared_f16(p, plan->sparse_waves, qpg, merge_kernel, grid, st)
+               : launch_sparse_shared_bf16(p, plan->sparse_waves, qpg, merge_kernel, grid, st);
+    else if (kv->dtype == TD_F16)
       rc = launch_sparse_f16(p, plan->sparse_waves, plan->sparse_rows, false, merge_kernel, grid, st);
     else
       rc = launch_sparse_bf16(p, plan->sparse_waves, plan->sparse_rows, false, merge_kernel, grid, st);
@@ -484,8 +496,8 @@ extern "C" int td_gather_probe(const td_paged_kv* kv, const td_index_list* list,
                                nullptr, nullptr, out, (int64_t)1 << 40, p, qpg, n_hrows);
   if (prc != TD_OK) return prc;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  if (sparse_kernel_fits(p, plan, list, qpg, kv->head_dim, false) && list->last_page_len == 0 &&
-      !list->last_page_len_arr) {
+  if (qpg == 1 && sparse_kernel_fits(p, plan, list, qpg, kv->head_dim, false) &&
+      list->last_page_len == 0 && !list->last_page_len_arr) {
     // the short-list kernel's own loads-only form; it reads `out` as q and writes nothing
     TD_REQUIRE(out_bytes >= (int64_t)batch * num_qo_heads * kv->head_dim * 2,
                "td_gather_probe: out holds %lld bytes, %lld needed", (long long)out_bytes,

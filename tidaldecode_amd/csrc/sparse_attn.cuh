@@ -135,8 +135,87 @@ __device__ __forceinline__ void scalar_load4(const int32_t* a0, const int32_t* a
       : "memory");
 }
 
-template <typename T, int NW, int U, bool FRESH, bool PROBE = false>
+// The tail of a head's computation, run by ONE wave that holds the workgroup's partial result of
+// that head (lane: dimensions 2 lane, 2 lane + 1; M, L uniform): write the result if the head was
+// not split, else publish the partial, take the head's ticket and, as the last of the splits to
+// arrive, merge all partials.
+template <typename T>
+__device__ __forceinline__ void finish_head(const DecodeParams& p, int lane, int n_splits, int split,
+                                            int64_t part0, int32_t* ticket, uint32_t* o32,
+                                            float* lse_out, float o0, float o1, float M, float L) {
+  constexpr int D = 128;
+  if (n_splits == 1) {
+    const float inv = L > 0.f ? 1.f / L : 0.f;
+    *o32 = pack2<T>(o0 * inv, o1 * inv);
+    if (lse_out && lane == 0) *lse_out = L > 0.f ? (M + fast_log2(L)) * kLn2 : -INFINITY;
+    return;
+  }
+  store_coherent(p.ws_o + (part0 + split) * D + 2 * lane, o0, o1);
+  if (lane == 0) store_coherent(p.ws_ml + (part0 + split) * 2, M, L);
+  if (!p.fused_merge) return;  // a second launch (merge_partials_kernel) reduces the partials
+
+  // Ordering.  The partial was stored by this wave alone, with device-scope write-through stores
+  // (sc1): such a store is acknowledged -- vmcnt decremented -- only once it has reached memory, the
+  // point where all XCDs meet, so after s_waitcnt vmcnt(0) the partial is visible device-wide.
+  // Only then is the ticket taken; the increment is a device-scope atomic performed at memory,
+  // so a wave that draws the last ticket knows that every other partial of the head had been
+  // acknowledged before its own ticket was even issued.  It reads them with device-scope loads
+  // (sc1), which do not hit lines a non-coherent cache level may still hold from earlier
+  // launches.  What would break this: a plain (non-sc1) store or load on ws_o / ws_ml, a compiler
+  // that moved the ticket above the wait (hence asm volatile with a memory clobber), or partials
+  // stored by several waves without a barrier between their waits and the ticket.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  int tk = 0;
+  if (lane == 0) tk = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  tk = __builtin_amdgcn_readfirstlane(tk);
+  if (tk != n_splits - 1) return;
+
+  float pm = kNegBig, pl = 0.f;  // (m, l) of split `lane`
+  {
+    const int sidx = lane < n_splits ? lane : n_splits - 1;
+    float a, c;
+    load_coherent(p.ws_ml + (part0 + sidx) * 2, a, c);
+    if (lane < n_splits) { pm = a; pl = c; }
+  }
+  constexpr int PRE = 16;  // partial loads in flight
+  float pa[PRE], pb[PRE];
+  auto issue = [&](int base) {
+#pragma unroll
+    for (int u = 0; u < PRE; ++u) {
+      int sidx = base + u;
+      sidx = sidx < n_splits ? sidx : n_splits - 1;
+      load_coherent(p.ws_o + (part0 + sidx) * D + 2 * lane, pa[u], pb[u]);
+    }
+  };
+  issue(0);
+  const float Mx = rows_max(row16_max(pm));
+  const float pf = fast_exp2(pm - Mx);  // scale of split `lane` (0 for lanes past the splits: pl = 0)
+  const float Lx = rows_sum(group_sum<16>(pl * pf));
+  float ra = 0.f, rb = 0.f;
+  for (int base = 0; base < n_splits; base += PRE) {
+    if (base) issue(base);
+#pragma unroll
+    for (int u = 0; u < PRE; ++u) {
+      const int sidx = base + u;  // uniform
+      if (sidx < n_splits) {
+        const float f = __builtin_bit_cast(
+            float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, pf), sidx));
+        ra = fmaf(pa[u], f, ra);
+        rb = fmaf(pb[u], f, rb);
+      }
+    }
+  }
+  const float inv = Lx > 0.f ? 1.f / Lx : 0.f;
+  *o32 = pack2<T>(ra * inv, rb * inv);
+  if (lse_out && lane == 0) *lse_out = Lx > 0.f ? (Mx + fast_log2(Lx)) * kLn2 : -INFINITY;
+  if (lane == 0) __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// QPG query heads per loaded K/V row: 1 (every head row is a query head with its own walk of a
+// list) or the 2, 4 or 8 query heads of a KV head that share one list (a head row is a KV head).
+template <typename T, int NW, int U, bool FRESH, bool PROBE = false, int QPG = 1>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U == 16 ? 2 : 4))) void sparse_attn_kernel(const DecodeParams p) {
+  static_assert(QPG == 1 || U == 8, "shared KV rows: 8 rows per lane");
   constexpr int D = 128;
   constexpr int LPR = 16;       // lanes per K/V row
   constexpr int TILE = 4 * U;   // tokens of a wave tile: lane group g holds tokens g U .. g U + U - 1
@@ -158,15 +237,17 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
     TD_TOUCH(p.fresh_slot);
   }
 #undef TD_TOUCH
-  const int kv_head = hrow >> p.qpk_shift;  // the host sends only power-of-two group sizes here
-  const int own = g * U + (li & (U - 1));   // the token of the tile this lane owns
+  // the host sends only power-of-two group sizes here
+  const int kv_head = QPG > 1 ? hrow : hrow >> p.qpk_shift;
+  const int rq0 = hrow * QPG;              // first query head of the head row
+  const int own = g * U + (li & (U - 1));  // the token of the tile this lane owns
 
   // ---- everything that depends on the kernel arguments only is requested at once ---------------
   // The list entries of the first tile are read before the length of the list is known: the
   // position is clamped to the row's capacity (n_list_host), which the host has checked against
   // the row stride.
   const int t0 = (split * NW + wave) * TILE;
-  const int idx_row = p.idx_per_kv ? kv_head : hrow;
+  const int idx_row = (QPG > 1 || p.idx_per_kv) ? kv_head : hrow;
   int list_beg = 0, list_end = 0;
   if (p.indptr) scalar_load2(p.indptr + b, p.indptr + b + 1, list_beg, list_end);
   const int32_t* row = p.idx + (int64_t)idx_row * p.idx_row_stride + list_beg;
@@ -178,10 +259,12 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
   };
   int32_t ent = fetch_entry(t0);
 
-  uint32_t qp[4];
-  {
-    const u32x4 v = reinterpret_cast<const u32x4*>(p.q)[((int64_t)b * p.num_qo_heads + hrow) * LPR + li];
-    qp[0] = v.x; qp[1] = v.y; qp[2] = v.z; qp[3] = v.w;
+  uint32_t qp[QPG][4];
+#pragma unroll
+  for (int j = 0; j < QPG; ++j) {
+    const u32x4 v =
+        reinterpret_cast<const u32x4*>(p.q)[((int64_t)b * p.num_qo_heads + rq0 + j) * LPR + li];
+    qp[j][0] = v.x; qp[j][1] = v.y; qp[j][2] = v.z; qp[j][3] = v.w;
   }
   uint32_t knew[4] = {0, 0, 0, 0}, vnew[4] = {0, 0, 0, 0};
   // slot of the token being decoded: requested now, waited for after the K/V rows are on their way
@@ -204,7 +287,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
     const float sgn = li < HALF ? -1.f : 1.f;  // y_lo = x_lo c - x_hi s,  y_hi = x_hi c + x_lo s
     rsn[0] = sgn * s0.x; rsn[1] = sgn * s0.y; rsn[2] = sgn * s0.z; rsn[3] = sgn * s0.w;
     rsn[4] = sgn * s1.x; rsn[5] = sgn * s1.y; rsn[6] = sgn * s1.z; rsn[7] = sgn * s1.w;
-    const int64_t fresh_off = ((int64_t)b * (p.num_qo_heads >> p.qpk_shift) + kv_head) * LPR + li;
+    const int n_kv = QPG > 1 ? p.num_qo_heads / QPG : p.num_qo_heads >> p.qpk_shift;
+    const int64_t fresh_off = ((int64_t)b * n_kv + kv_head) * LPR + li;
     const u32x4 kn = reinterpret_cast<const u32x4*>(p.fresh_k)[fresh_off];
     const u32x4 vn = reinterpret_cast<const u32x4*>(p.fresh_v)[fresh_off];
     knew[0] = kn.x; knew[1] = kn.y; knew[2] = kn.z; knew[3] = kn.w;
@@ -259,14 +343,24 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
   float acc[8];
 #pragma unroll
   for (int d = 0; d < 8; ++d) acc[d] = 0.f;
+  // Shared KV rows (QPG > 1): per-head maxima and denominators, and p.V on the matrix cores:
+  // accm[e][r] = o[head 4 g + r][li 8 + e], already summed over the four lane groups.
+  float mh[QPG], lh[QPG];
+#pragma unroll
+  for (int j = 0; j < QPG; ++j) { mh[j] = kNegBig; lh[j] = 0.f; }
+  f32x4 accm[8];
+#pragma unroll
+  for (int d = 0; d < 8; ++d) accm[d] = f32x4{0.f, 0.f, 0.f, 0.f};
+  __shared__ __attribute__((aligned(16))) float sm_p[QPG > 1 ? NW * QPG * TILE : 4];
   // Decode-step fusion: q arrives un-rotated and is rotated in registers, once per wave.  The new
   // token's key is rotated by the wave that writes it into the cache (one per KV head) and by
   // every wave whose tokens include its slot.
   bool q_rot = false, k_rot = false, wrote = false;  // wave-uniform
-  const bool writer = FRESH && split == 0 && wave == 0 && hrow == (kv_head << p.qpk_shift);
+  const bool writer = FRESH && split == 0 && wave == 0 && (QPG > 1 || hrow == (kv_head << p.qpk_shift));
   auto fresh_duties = [&](bool any_hit) {
     if (!q_rot) {
-      rotate(qp);
+#pragma unroll
+      for (int j = 0; j < QPG; ++j) rotate(qp[j]);
       q_rot = true;
     }
     if ((any_hit || (writer && !wrote)) && !k_rot) {
@@ -353,14 +447,88 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
       }
     }
 
+    if constexpr (QPG > 1) {
+      // The lane ends with the logits of ITS token for all QPG heads; maxima per head are made
+      // wave-uniform.  The weights then go through a strip of LDS private to the wave into the
+      // A-operand layout of a 16x16x16 matrix product (row = head, inner index = the 16 tokens
+      // 4c..4c+3 of the four lane groups), B = the four V rows a lane holds, one 16-bit element each.
+      constexpr bool kSplit = std::is_same<T, BF16>::value;  // bf16 weights travel as value + remainder
+      float* sp = sm_p + wave * (QPG * TILE);
+      float alpha[QPG];
+#pragma unroll
+      for (int j = 0; j < QPG; ++j) {
+        float part[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          float a = dot2<T>(qp[j][0], kb[u].x, 0.f);
+          a = dot2<T>(qp[j][1], kb[u].y, a);
+          a = dot2<T>(qp[j][2], kb[u].z, a);
+          part[u] = dot2<T>(qp[j][3], kb[u].w, a);
+        }
+        const float red = reduce_scatter_rows<U>(part, li);
+        const float sv = valid ? red * p.scale_log2 : kNegBig;
+        const float m_new = fmaxf(mh[j], rows_max(row16_max(sv)));
+        alpha[j] = fast_exp2(mh[j] - m_new);
+        mh[j] = m_new;
+        const float pr = valid ? fast_exp2(sv - m_new) : 0.f;
+        lh[j] = lh[j] * alpha[j] + (li < 8 ? pr : 0.f);  // lanes li and li ^ 8 hold the same token
+        if (li < 8) sp[j * TILE + own] = pr;
+      }
+      if (t != t0) {  // later tiles: rescale what the earlier ones left (row r of group g: head 4 g + r)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float f = (QPG == 8 && g == 1) ? alpha[(4 + r) % QPG] : alpha[r % QPG];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) accm[e][r] *= f;
+        }
+      }
+      // the strip was written by other lanes of this wave: LDS accesses of a wave complete in
+      // issue order; the wait and the wave barrier pin that order for the compiler too
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int c = 0; c < U / 4; ++c) {
+        f32x4 pa = *reinterpret_cast<const f32x4*>(sp + (li < QPG ? li : 0) * TILE + g * U + 4 * c);
+        if (li >= QPG) pa = f32x4{0.f, 0.f, 0.f, 0.f};  // rows past the heads of the group
+        const uint32_t ah0 = pack2<T>(pa.x, pa.y), ah1 = pack2<T>(pa.z, pa.w);
+        uint32_t al0 = 0, al1 = 0;
+        if constexpr (kSplit) {
+          float r0, r1, r2, r3;
+          unpack2<T>(ah0, r0, r1);
+          unpack2<T>(ah1, r2, r3);
+          al0 = pack2<T>(pa.x - r0, pa.y - r1);
+          al1 = pack2<T>(pa.z - r2, pa.w - r3);
+        }
+        const uint32_t vw[4][4] = {
+            {vb[4 * c].x, vb[4 * c].y, vb[4 * c].z, vb[4 * c].w},
+            {vb[4 * c + 1].x, vb[4 * c + 1].y, vb[4 * c + 1].z, vb[4 * c + 1].w},
+            {vb[4 * c + 2].x, vb[4 * c + 2].y, vb[4 * c + 2].z, vb[4 * c + 2].w},
+            {vb[4 * c + 3].x, vb[4 * c + 3].y, vb[4 * c + 3].z, vb[4 * c + 3].w}};
+#pragma unroll
+        for (int w2 = 0; w2 < 4; ++w2) {
+          const uint32_t lo0 = __builtin_amdgcn_perm(vw[1][w2], vw[0][w2], 0x05040100u);
+          const uint32_t lo1 = __builtin_amdgcn_perm(vw[3][w2], vw[2][w2], 0x05040100u);
+          const uint32_t hi0 = __builtin_amdgcn_perm(vw[1][w2], vw[0][w2], 0x07060302u);
+          const uint32_t hi1 = __builtin_amdgcn_perm(vw[3][w2], vw[2][w2], 0x07060302u);
+          accm[2 * w2] = mfma_16x16x16<T>(ah0, ah1, lo0, lo1, accm[2 * w2]);
+          accm[2 * w2 + 1] = mfma_16x16x16<T>(ah0, ah1, hi0, hi1, accm[2 * w2 + 1]);
+          if constexpr (kSplit) {
+            accm[2 * w2] = mfma_16x16x16<T>(al0, al1, lo0, lo1, accm[2 * w2]);
+            accm[2 * w2 + 1] = mfma_16x16x16<T>(al0, al1, hi0, hi1, accm[2 * w2 + 1]);
+          }
+        }
+      }
+      asm volatile("" ::: "memory");  // the strip is rewritten by the next tile only after these reads
+      continue;
+    }
     // q.k: U partial sums per lane, reduce-scattered so that the lane ends with its own token
     float part[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      float a = dot2<T>(qp[0], kb[u].x, 0.f);
-      a = dot2<T>(qp[1], kb[u].y, a);
-      a = dot2<T>(qp[2], kb[u].z, a);
-      part[u] = dot2<T>(qp[3], kb[u].w, a);
+      float a = dot2<T>(qp[0][0], kb[u].x, 0.f);
+      a = dot2<T>(qp[0][1], kb[u].y, a);
+      a = dot2<T>(qp[0][2], kb[u].z, a);
+      part[u] = dot2<T>(qp[0][3], kb[u].w, a);
     }
     const float red = reduce_scatter_rows<U>(part, li);  // every lane takes part: no branch around it
     const float sv = valid ? red * p.scale_log2 : kNegBig;
@@ -399,115 +567,80 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
   }
 
   if constexpr (PROBE) return;
-  // ---- the four lane groups of the wave: the maximum is shared, so the sums simply add ----------
-  // reduce-scatter over the groups: lane (g, li) ends with dimensions li 8 + g 2 + {0, 1}
-  float r0, r1;
-  {
-    float x, y, h[4];
+  __shared__ __attribute__((aligned(16))) float sm_o[NW][QPG][D];
+  __shared__ float sm_ml[NW][QPG][2];
+  if constexpr (QPG > 1) {
+    // the matrix product already summed the lane groups: the lanes of group g hold heads 4g..4g+3
 #pragma unroll
-    for (int i2 = 0; i2 < 4; ++i2) {
-      swap32(acc[i2], acc[i2 + 4], x, y);
-      h[i2] = x + y;  // lower half: dimension i2, upper half: dimension i2 + 4
-    }
-    swap16(h[0], h[2], x, y);
-    r0 = x + y;
-    swap16(h[1], h[3], x, y);
-    r1 = x + y;
-  }
-  float l_w = rows_sum(group_sum<16>(l_lane));
-
-  // ---- the waves of the workgroup meet in LDS; wave 0 carries on alone ---------------------------
-  __shared__ __attribute__((aligned(16))) float sm_o[NW][D];
-  __shared__ float sm_ml[NW][2];
-  {
-    f32x2 v = {r0, r1};
-    *reinterpret_cast<f32x2*>(&sm_o[wave][li * 8 + g * 2]) = v;
-    if (lane == 0) {
-      sm_ml[wave][0] = m_run;
-      sm_ml[wave][1] = l_w;
-    }
-  }
-  __syncthreads();
-  if (wave != 0) return;
-  float M = kNegBig;
-#pragma unroll
-  for (int w = 0; w < NW; ++w) M = fmaxf(M, sm_ml[w][0]);
-  float L = 0.f, o0 = 0.f, o1 = 0.f;  // this lane: dimensions 2 lane, 2 lane + 1
-#pragma unroll
-  for (int w = 0; w < NW; ++w) {
-    const float f = fast_exp2(sm_ml[w][0] - M);
-    L = fmaf(sm_ml[w][1], f, L);
-    const f32x2 v = *reinterpret_cast<const f32x2*>(&sm_o[w][2 * lane]);
-    o0 = fmaf(v.x, f, o0);
-    o1 = fmaf(v.y, f, o1);
-  }
-  uint32_t* o32 = reinterpret_cast<uint32_t*>(p.o) + ((int64_t)b * p.num_qo_heads + hrow) * (D / 2) + lane;
-  float* lse_out = p.lse ? p.lse + (int64_t)b * p.num_qo_heads + hrow : nullptr;
-  if (n_splits == 1) {
-    const float inv = L > 0.f ? 1.f / L : 0.f;
-    *o32 = pack2<T>(o0 * inv, o1 * inv);
-    if (lse_out && lane == 0) *lse_out = L > 0.f ? (M + fast_log2(L)) * kLn2 : -INFINITY;
-    return;
-  }
-  const int64_t part0 = ((int64_t)b * p.vheads + hrow) * p.max_splits;
-  store_coherent(p.ws_o + (part0 + split) * D + 2 * lane, o0, o1);
-  if (lane == 0) store_coherent(p.ws_ml + (part0 + split) * 2, M, L);
-  if (!p.fused_merge) return;
-
-  // ---- the last workgroup of this (sequence, head) to arrive reduces the partials ---------------
-  // Every partial of this workgroup was stored by this wave with device-coherent write-through
-  // stores; vmcnt(0) returns once they are acknowledged, and only then is the ticket taken.
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  int32_t* ticket = p.ws_cnt + ((int64_t)b * gridDim.x + hrow) * p.ticket_stride;
-  int tk = 0;
-  if (lane == 0) tk = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  tk = __builtin_amdgcn_readfirstlane(tk);
-  if (tk != n_splits - 1) return;
-
-  float pm = kNegBig, pl = 0.f;  // (m, l) of split `lane`
-  {
-    const int sidx = lane < n_splits ? lane : n_splits - 1;
-    float a, c;
-    load_coherent(p.ws_ml + (part0 + sidx) * 2, a, c);
-    if (lane < n_splits) { pm = a; pl = c; }
-  }
-  constexpr int PRE = 16;  // partial loads in flight
-  float pa[PRE], pb[PRE];
-  auto issue = [&](int base) {
-#pragma unroll
-    for (int u = 0; u < PRE; ++u) {
-      int sidx = base + u;
-      sidx = sidx < n_splits ? sidx : n_splits - 1;
-      load_coherent(p.ws_o + (part0 + sidx) * D + 2 * lane, pa[u], pb[u]);
-    }
-  };
-  issue(0);
-  const float Mx = rows_max(row16_max(pm));
-  const float pf = fast_exp2(pm - Mx);  // scale of split `lane` (0 for lanes past the splits: pl = 0)
-  const float Lx = rows_sum(group_sum<16>(pl * pf));
-  float ra = 0.f, rb = 0.f;
-  for (int base = 0; base < n_splits; base += PRE) {
-    if (base) issue(base);
-#pragma unroll
-    for (int u = 0; u < PRE; ++u) {
-      const int sidx = base + u;  // uniform
-      if (sidx < n_splits) {
-        const float f = __builtin_bit_cast(
-            float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, pf), sidx));
-        ra = fmaf(pa[u], f, ra);
-        rb = fmaf(pb[u], f, rb);
+    for (int r = 0; r < 4; ++r) {
+      const int head = 4 * g + r;
+      if (head < QPG) {
+        *reinterpret_cast<f32x4*>(&sm_o[wave][head][li * 8]) =
+            f32x4{accm[0][r], accm[1][r], accm[2][r], accm[3][r]};
+        *reinterpret_cast<f32x4*>(&sm_o[wave][head][li * 8 + 4]) =
+            f32x4{accm[4][r], accm[5][r], accm[6][r], accm[7][r]};
       }
     }
+#pragma unroll
+    for (int j = 0; j < QPG; ++j) {
+      const float lw = rows_sum(group_sum<16>(lh[j]));
+      if (lane == 0) {
+        sm_ml[wave][j][0] = mh[j];
+        sm_ml[wave][j][1] = lw;
+      }
+    }
+  } else {
+    // ---- the four lane groups of the wave: the maximum is shared, so the sums simply add --------
+    // reduce-scatter over the groups: lane (g, li) ends with dimensions li 8 + g 2 + {0, 1}
+    float r0, r1;
+    {
+      float x, y, h[4];
+#pragma unroll
+      for (int i2 = 0; i2 < 4; ++i2) {
+        swap32(acc[i2], acc[i2 + 4], x, y);
+        h[i2] = x + y;  // lower half: dimension i2, upper half: dimension i2 + 4
+      }
+      swap16(h[0], h[2], x, y);
+      r0 = x + y;
+      swap16(h[1], h[3], x, y);
+      r1 = x + y;
+    }
+    const float l_w = rows_sum(group_sum<16>(l_lane));
+    *reinterpret_cast<f32x2*>(&sm_o[wave][0][li * 8 + g * 2]) = f32x2{r0, r1};
+    if (lane == 0) {
+      sm_ml[wave][0][0] = m_run;
+      sm_ml[wave][0][1] = l_w;
+    }
   }
-  const float inv = Lx > 0.f ? 1.f / Lx : 0.f;
-  *o32 = pack2<T>(ra * inv, rb * inv);
-  if (lse_out && lane == 0) *lse_out = Lx > 0.f ? (Mx + fast_log2(Lx)) * kLn2 : -INFINITY;
-  if (lane == 0) __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  // ---- the waves of the workgroup meet in LDS; wave j carries on alone with head j --------------
+  __syncthreads();
+  for (int j = wave; j < QPG; j += NW) {
+    float M = kNegBig;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) M = fmaxf(M, sm_ml[w][j][0]);
+    float L = 0.f, o0 = 0.f, o1 = 0.f;  // this lane: dimensions 2 lane, 2 lane + 1
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      const float f = fast_exp2(sm_ml[w][j][0] - M);
+      L = fmaf(sm_ml[w][j][1], f, L);
+      const f32x2 v = *reinterpret_cast<const f32x2*>(&sm_o[w][j][2 * lane]);
+      o0 = fmaf(v.x, f, o0);
+      o1 = fmaf(v.y, f, o1);
+    }
+    const int qh = rq0 + j;
+    uint32_t* o32 = reinterpret_cast<uint32_t*>(p.o) + ((int64_t)b * p.num_qo_heads + qh) * (D / 2) + lane;
+    float* lse_out = p.lse ? p.lse + (int64_t)b * p.num_qo_heads + qh : nullptr;
+    const int64_t part0 = ((int64_t)b * p.vheads + qh) * p.max_splits;
+    int32_t* ticket = p.ws_cnt + (((int64_t)b * gridDim.x + hrow) * QPG + j) * p.ticket_stride;
+    finish_head<T>(p, lane, n_splits, split, part0, ticket, o32, lse_out, o0, o1, M, L);
+  }
 }
 
-// Shapes of the sparse-layer kernel: waves per workgroup x K (and V) rows per lane.
-static bool sparse_shape_supported(int nw, int rows) {
-  return (nw == 4 || nw == 8) && (rows == 8 || rows == 16);
+// Shapes of the sparse-layer kernel: waves per workgroup x K (and V) rows per lane; with shared
+// KV rows (2, 4 or 8 query heads per list walk) 8 rows per lane.
+static bool sparse_shape_supported(int nw, int rows, int qpg = 1) {
+  if (qpg == 1) return (nw == 4 || nw == 8) && (rows == 8 || rows == 16);
+  return (qpg == 2 || qpg == 4 || qpg == 8) && (nw == 4 || nw == 8) && rows == 8;
 }
 
 template <typename T>
@@ -531,11 +664,39 @@ static int launch_sparse(const DecodeParams& p, int nw, int rows, bool probe, di
   return fail(TD_ERR_UNSUPPORTED, "sparse decode attention: no kernel for %d waves x %d rows", nw, rows);
 }
 
+// shared KV rows: QPG query heads per list walk
+template <typename T>
+static int launch_sparse_shared(const DecodeParams& p, int nw, int qpg, dim3 grid, hipStream_t st) {
+#define TD_SPARSE_CASE(N_, Q_)                                                                  \
+  if (nw == N_ && qpg == Q_) {                                                                  \
+    if (p.fresh_k)                                                                              \
+      hipLaunchKernelGGL((sparse_attn_kernel<T, N_, 8, true, false, Q_>), grid, dim3(N_ * 64),  \
+                         0, st, p);                                                             \
+    else                                                                                        \
+      hipLaunchKernelGGL((sparse_attn_kernel<T, N_, 8, false, false, Q_>), grid, dim3(N_ * 64), \
+                         0, st, p);                                                             \
+    return TD_OK;                                                                               \
+  }
+  TD_SPARSE_CASE(4, 2)
+  TD_SPARSE_CASE(4, 4)
+  TD_SPARSE_CASE(4, 8)
+  TD_SPARSE_CASE(8, 2)
+  TD_SPARSE_CASE(8, 4)
+  TD_SPARSE_CASE(8, 8)
+#undef TD_SPARSE_CASE
+  return fail(TD_ERR_UNSUPPORTED,
+              "sparse decode attention: no kernel for %d waves with %d query heads per shared row", nw, qpg);
+}
+
 // Launches the sparse-layer kernel (and, when the plan asks for it, the second-launch merge);
-// defined once per element type in sparse_attn_f16.hip / sparse_attn_bf16.hip.
+// defined once per element type (and once more for shared KV rows) in sparse_attn_*.hip.
 int launch_sparse_f16(const DecodeParams& p, int nw, int rows, bool probe, bool merge_kernel, dim3 grid,
                       hipStream_t st);
 int launch_sparse_bf16(const DecodeParams& p, int nw, int rows, bool probe, bool merge_kernel, dim3 grid,
                        hipStream_t st);
+int launch_sparse_shared_f16(const DecodeParams& p, int nw, int qpg, bool merge_kernel, dim3 grid,
+                             hipStream_t st);
+int launch_sparse_shared_bf16(const DecodeParams& p, int nw, int qpg, bool merge_kernel, dim3 grid,
+                              hipStream_t st);
 
 }  // namespace tidal
