@@ -347,10 +347,11 @@ int td_topk(const void* values, int32_t values_dtype, int64_t values_stride, int
             void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
- * Bytes of device scratch that lets td_topk spread a row over several workgroups (rows of more
- * than 8192 elements; three launches; about 56 KiB per row).  The scratch must be zero-filled once
- * before its first use;
- * every call leaves it ready for the next.  Without it (NULL) one workgroup handles each row.
+ * Bytes of device scratch for td_topk.  Rows of up to 40960 elements never touch it (one launch,
+ * every workgroup of a row selects on the whole row and emits a slice).  A few longer rows are
+ * shared between workgroups through it (three launches; about 56 KiB per row); without it (NULL),
+ * or with many long rows, the one-launch kernel re-reads such rows from L2 in every pass.  The
+ * scratch must be zero-filled once before its first use; every call leaves it ready for the next.
  * Plays the part of the `buf` argument of topk_filtering (tidal/utils/controller.py:164-168).
  */
 int64_t td_topk_workspace_bytes(int32_t rows);

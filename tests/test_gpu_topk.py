@@ -16,7 +16,8 @@ _scratch = {}
 
 def _shared_scratch(cuda, rows):
     """One scratch tensor for the whole module: zeroed at allocation only, so every cooperative
-    call after the first relies on the previous call having left it clean."""
+    call after the first (rows of more than 40960 elements) relies on the previous call having
+    left it clean."""
     from tidaldecode_amd import _kernels
 
     need = _kernels.topk_workspace_bytes(64)
@@ -51,7 +52,7 @@ def _check(values, k, cuda):
     assert np.array_equal(got.numpy(), want_c)
     expect = torch.gather(values, 1, want)  # values travel with their index (NaN == NaN here)
     assert torch.equal(torch.nan_to_num(vals.float(), nan=1e38), torch.nan_to_num(expect.float(), nan=1e38))
-    # the several-workgroups-per-row path (taken for rows longer than 8192 when scratch is given)
+    # with scratch: rows of more than 40960 elements take the three cooperative launches
     got2, vals2 = _gpu_topk(values, k, cuda, scratch=True)
     assert torch.equal(got2, got), "cooperative path differs"
     assert torch.equal(torch.nan_to_num(vals2.float(), nan=1e38), torch.nan_to_num(vals.float(), nan=1e38))
@@ -105,6 +106,40 @@ def test_long_rows_with_crowded_threshold_bins(cuda, dtype):
     _check(v.to(dtype), 20000, cuda)
     _check(v.to(dtype), 1, cuda)
     _check(v.to(dtype), n, cuda)
+
+
+@pytest.mark.parametrize("n", [5000, 32768, 30000 + 77, 50000])
+def test_score_distributions_that_steer_the_radix_levels(cuda, n):
+    """The one-launch kernel maps scores to d = distance below the row maximum and starts its radix
+    select 64 binades below that maximum.  Rows that leave the usual road: all negative; fewer
+    non-negative scores than k (threshold below zero); a threshold 100 binades below the maximum
+    (second pass over the rest of the range); +0 / -0 ties at the threshold; denormals; a threshold
+    bin with hundreds of members (radix levels on the gathered list) and with thousands (another
+    level over the row before anything is gathered)."""
+    g = torch.Generator().manual_seed(n)
+    k = max(1, n // 16)
+    neg = -10.0 + 2.0 * torch.randn((2, n), generator=g)
+    few_pos = -3.0 + torch.randn((2, n), generator=g)
+    assert ((few_pos >= 0).sum(1) < k).all()
+    wide = torch.rand((2, n), generator=g) * 1e-30
+    wide[:, torch.randperm(n, generator=g)[: k // 2]] = 0.5 + 0.5 * torch.rand((2, k // 2), generator=g)
+    zeros = -torch.rand((2, n), generator=g)
+    idx = torch.randperm(n, generator=g)
+    zeros[:, idx[: k // 4]] = torch.rand((2, k // 4), generator=g) + 0.1
+    zeros[:, idx[k // 4: 2 * k]] = 0.0
+    zeros[:, idx[k // 2: 2 * k: 3]] = -0.0
+    den = torch.randn((2, n), generator=g) * 1e-41
+    for v in (neg, few_pos, wide, zeros, den):
+        _check(v, k, cuda)
+    # one bin at 1.0 is 2^16 ulps = 0.0078 wide
+    for members in (600, 3000):
+        if 2 * members > n:
+            continue
+        v = torch.rand((2, n), generator=g) * 0.9
+        idx = torch.randperm(n, generator=g)
+        v[:, idx[:members]] = 1.0 + torch.rand((2, members), generator=g) * 0.007
+        v[:, idx[members: members + 300]] = 1.01 + torch.rand((2, 300), generator=g)
+        _check(v, 300 + members // 2, cuda)
 
 
 def test_sorted_and_blocky_long_rows(cuda):

@@ -165,8 +165,9 @@ def topk_filtering(estimated_value: torch.Tensor, estimated_indices: Optional[to
     """bsk_ops.h:34-39 / topk.cu:7-44.  Row-wise top-``page_budget`` of ``estimated_value``
     ``[H, len]``; ``indices_out[h, j]`` is ``estimated_indices[h, p]`` of the selected position
     ``p``.  ``buf`` is scratch, as in the reference (there: RAFT's): a zero-initialised uint8 /
-    any-dtype device tensor of at least ``topk_workspace_bytes(H)`` bytes lets rows longer than
-    8192 elements be spread over several workgroups; smaller or ``None``: one workgroup per row.
+    any-dtype device tensor of at least ``topk_workspace_bytes(H)`` bytes through which the
+    workgroups of a row of more than 40960 elements share the work; shorter rows never touch it,
+    and without it (smaller or ``None``) every workgroup of a long row goes through the whole row.
     The call leaves ``buf`` zeroed where it must be for the next call.
 
     Deterministic where the reference is not: ties at the threshold go to the lower position

@@ -1,16 +1,22 @@
 // Row-wise top-k selection and the cross-head score reduction for gfx950 (MI355X).
 //
-// One 1024-thread workgroup (16 wavefronts) per row (rows of up to 65536 elements are held in
-// registers, longer ones are re-read from L2 per pass; given scratch memory, rows of more than
-// 8192 elements are split over several workgroups, see topk_coop_select_kernel) runs an MSB-first radix select over
-// order-preserving integer keys with LDS histograms (11/11/10-bit digits for fp32 keys, 8/8 for
-// fp16/bf16 keys), which yields the exact k-th largest key T and the number r of elements equal
-// to T that still fit.  A final ordered pass emits every element above T plus the first r
-// elements equal to T, so ties go to the lower position and the output is sorted by position:
-// the result is a pure function of the input row.
+// Exact selection by radix select over order-preserving integer images of the fp32 scores (fp16 /
+// bf16 scores are widened first): the k-th largest key T and the number r of elements equal to T
+// that still fit, then an ordered pass that emits every element above T plus the first r elements
+// equal to T.  Ties go to the lower position and each output row is sorted by position: the
+// result is a pure function of the input row.  -0 equals +0, every NaN ranks above +inf.
+//
+// Two routes:
+//   * topk_slice_kernel, one launch: every workgroup (1024 threads) of a row runs the selection on
+//     the whole row -- up to 40K elements from registers -- and emits its own slice of it.  All
+//     rows of up to 40960 elements, and longer ones when there are many rows or no scratch.
+//   * topk_coop_{hist,select,emit}_kernel, three launches over a zeroed scratch: the workgroups of
+//     a row share the row.  A few rows of more than 40960 elements.
 //
 // Replaces decode_select_k (kernels/include/topk/decode_select_k.cuh:25-62 of the reference),
 // which launches RAFT's radix_topk_one_block_kernel, one 512-thread block per head.
+
+#include <type_traits>
 
 #include "common.cuh"
 
@@ -18,7 +24,6 @@ namespace tidal {
 
 constexpr int kTopkThreads = 1024;
 constexpr int kTopkWaves = kTopkThreads / 64;
-constexpr int kMaxBins = 2048;
 
 struct TopkParams {
   const void* values;
@@ -67,9 +72,6 @@ template <>
 struct KeyTraits<F32> {
   typedef uint32_t key_t;
   typedef float elem_t;
-  static constexpr int kBits = 32;
-  static constexpr int kPasses = 3;
-  __device__ static constexpr int digit_bits(int pass) { return pass < 2 ? 11 : 10; }
   __device__ static key_t key(float f) {
     uint32_t u = __builtin_bit_cast(uint32_t, f);
     if ((u & 0x7fffffffu) == 0u) u = 0u;
@@ -77,35 +79,6 @@ struct KeyTraits<F32> {
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
   }
 };
-template <>
-struct KeyTraits<F16> {
-  typedef uint32_t key_t;
-  typedef uint16_t elem_t;
-  static constexpr int kBits = 16;
-  static constexpr int kPasses = 2;
-  __device__ static constexpr int digit_bits(int) { return 8; }
-  __device__ static key_t key(uint16_t h) {
-    uint32_t u = h;
-    if ((u & 0x7fffu) == 0u) u = 0u;
-    if ((u & 0x7fffu) > 0x7c00u) return 0xffffu;
-    return (u & 0x8000u) ? (~u & 0xffffu) : (u | 0x8000u);
-  }
-};
-template <>
-struct KeyTraits<BF16> {
-  typedef uint32_t key_t;
-  typedef uint16_t elem_t;
-  static constexpr int kBits = 16;
-  static constexpr int kPasses = 2;
-  __device__ static constexpr int digit_bits(int) { return 8; }
-  __device__ static key_t key(uint16_t h) {
-    uint32_t u = h;
-    if ((u & 0x7fffu) == 0u) u = 0u;
-    if ((u & 0x7fffu) > 0x7f80u) return 0xffffu;
-    return (u & 0x8000u) ? (~u & 0xffffu) : (u | 0x8000u);
-  }
-};
-
 // inclusive suffix sum inside a wavefront: lane i gets the sum over lanes >= i
 __device__ __forceinline__ uint32_t wave_suffix_sum(uint32_t x, int lane) {
 #pragma unroll
@@ -114,131 +87,6 @@ __device__ __forceinline__ uint32_t wave_suffix_sum(uint32_t x, int lane) {
     if (lane + off < 64) x += y;
   }
   return x;
-}
-
-template <typename T>
-__global__ __launch_bounds__(kTopkThreads) void topk_kernel(const TopkParams p) {
-  typedef KeyTraits<T> KT;
-  typedef typename KT::elem_t elem_t;
-  const int row = blockIdx.x;
-  const int32_t* table = table_of(p, row);
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int len = row_len(p, row);
-  const int k = row_k(p, len);  // 1 <= k <= len
-  const elem_t* vals = reinterpret_cast<const elem_t*>(p.values) + (int64_t)row * p.values_stride;
-
-  __shared__ uint32_t hist[kMaxBins];
-  __shared__ uint32_t wave_tot[kTopkWaves];
-  __shared__ uint32_t sh_bin, sh_krem;
-  __shared__ uint32_t seg_gt[kTopkWaves], seg_eq[kTopkWaves];
-
-  uint32_t prefix = 0, mask = 0, krem = (uint32_t)k;
-  int shift = KT::kBits;
-#pragma unroll
-  for (int pass = 0; pass < KT::kPasses; ++pass) {
-    const int bits = KT::digit_bits(pass);
-    const int nb = 1 << bits;
-    shift -= bits;
-    for (int i = tid; i < nb; i += kTopkThreads) hist[i] = 0;
-    __syncthreads();
-    for (int i = tid; i < len; i += kTopkThreads) {
-      const uint32_t key = KT::key(vals[i]);
-      if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & (nb - 1)], 1u);
-    }
-    __syncthreads();
-    // locate the digit whose bin holds the krem-th largest remaining key
-    const int bpt = nb >= kTopkThreads ? nb / kTopkThreads : 1;  // bins per thread
-    const int my_bin = tid * bpt;
-    uint32_t local = 0;
-    if (my_bin < nb)
-      for (int j = 0; j < bpt; ++j) local += hist[my_bin + j];
-    const uint32_t suf = wave_suffix_sum(local, lane);
-    if (lane == 0) wave_tot[wave] = suf;
-    __syncthreads();
-    uint32_t above = suf - local;  // keys in bins above this thread's bins
-    for (int w = wave + 1; w < kTopkWaves; ++w) above += wave_tot[w];
-    if (my_bin < nb) {
-      for (int j = bpt - 1; j >= 0; --j) {
-        const uint32_t c = hist[my_bin + j];
-        if (above < krem && krem <= above + c) {
-          sh_bin = (uint32_t)(my_bin + j);
-          sh_krem = krem - above;
-        }
-        above += c;
-      }
-    }
-    __syncthreads();
-    prefix |= sh_bin << shift;
-    mask |= (uint32_t)(nb - 1) << shift;
-    krem = sh_krem;
-    __syncthreads();
-  }
-  const uint32_t thr = prefix;  // the k-th largest key
-  const uint32_t r = krem;      // elements equal to thr that are selected (lowest positions)
-
-  // ordered emission: each wave owns a contiguous segment of the row
-  int seg = (len + kTopkWaves - 1) / kTopkWaves;
-  seg = (seg + 63) & ~63;
-  const int s0 = wave * seg;
-  int s1 = s0 + seg;
-  s1 = s1 > len ? len : s1;
-  uint32_t n_gt = 0, n_eq = 0;
-  for (int base = s0; base < s1; base += 64) {
-    const int i = base + lane;
-    uint32_t key = 0;
-    const bool in = i < s1;
-    if (in) key = KT::key(vals[i]);
-    n_gt += __popcll(__ballot(in && key > thr));
-    n_eq += __popcll(__ballot(in && key == thr));
-  }
-  if (lane == 0) {
-    seg_gt[wave] = n_gt;
-    seg_eq[wave] = n_eq;
-  }
-  __syncthreads();
-  uint32_t eq_run = 0, out_run = 0;
-  for (int w = 0; w < wave; ++w) {
-    const uint32_t e = seg_eq[w];
-    const uint32_t room = r > eq_run ? r - eq_run : 0u;
-    out_run += seg_gt[w] + (e < room ? e : room);
-    eq_run += e;
-  }
-  const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
-  int32_t* out_idx = p.out_idx + (int64_t)row * p.out_stride;
-  elem_t* out_val =
-      p.out_values ? reinterpret_cast<elem_t*>(p.out_values) + (int64_t)row * p.out_stride : nullptr;
-  for (int base = s0; base < s1; base += 64) {
-    const int i = base + lane;
-    const bool in = i < s1;
-    elem_t v = 0;
-    uint32_t key = 0;
-    if (in) {
-      v = vals[i];
-      key = KT::key(v);
-    }
-    const bool gt = in && key > thr;
-    const bool eq = in && key == thr;
-    const uint64_t eq_mask = __ballot(eq);
-    const uint32_t eq_rank = eq_run + (uint32_t)__popcll(eq_mask & lt_mask);
-    const bool sel = gt || (eq && eq_rank < r);
-    const uint64_t sel_mask = __ballot(sel);
-    const uint32_t pos = out_run + (uint32_t)__popcll(sel_mask & lt_mask);
-    if (sel && pos < (uint32_t)k) {
-      int32_t payload;
-      if (p.in_idx)
-        payload = p.in_idx[(int64_t)row * p.in_idx_stride + i];
-      else if (p.page_table)
-        payload = slot_of(p, table, i);
-      else
-        payload = i;
-      out_idx[pos] = payload;
-      if (out_val) out_val[pos] = v;
-    }
-    eq_run += (uint32_t)__popcll(eq_mask);
-    out_run += (uint32_t)__popcll(sel_mask);
-  }
 }
 
 // inclusive prefix sum inside a wavefront
@@ -268,138 +116,6 @@ __device__ __forceinline__ uint32_t block_exclusive_sum(uint32_t x, int lane, in
   __syncthreads();
   total = all;
   return before + incl - x;
-}
-
-// Register-resident variant for rows of up to 1024 * IPT elements: thread t owns elements
-// j * 1024 + t (j < IPT), so the row is read from memory exactly once (coalesced, IPT loads in
-// flight per thread) and every radix pass and the ordered emission work on registers.  In index
-// order the row is a sequence of 64-element runs (j, wave); per-run counts are prefix-summed in
-// LDS and the lanes of a run rank themselves with ballots.
-template <typename T, int IPT>
-__global__ __launch_bounds__(kTopkThreads) void topk_reg_kernel(const TopkParams p) {
-  typedef KeyTraits<T> KT;
-  typedef typename KT::elem_t elem_t;
-  const int row = blockIdx.x;
-  const int32_t* table = table_of(p, row);
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int len = row_len(p, row);
-  const int k = row_k(p, len);  // 1 <= k <= len <= 1024 * IPT (host-checked for p.len)
-  const elem_t* vals = reinterpret_cast<const elem_t*>(p.values) + (int64_t)row * p.values_stride;
-
-  __shared__ uint32_t hist[kMaxBins];
-  __shared__ uint32_t wave_tot[kTopkWaves];
-  __shared__ uint32_t sh_bin, sh_krem;
-  __shared__ uint32_t run_eq[IPT * kTopkWaves], run_out[IPT * kTopkWaves];
-
-  // key 0 is below every real key (it would be the image of a negative NaN, which maps to the
-  // maximum instead), so it marks the slots past the end of the row
-  uint32_t key[IPT];
-#pragma unroll
-  for (int j = 0; j < IPT; ++j) {
-    const int i = j * kTopkThreads + tid;
-    const uint32_t kv = KT::key(vals[i < len ? i : len - 1]);  // unconditional load: all IPT in flight
-    key[j] = i < len ? kv : 0u;
-  }
-
-  uint32_t prefix = 0, mask = 0, krem = (uint32_t)k;
-  int shift = KT::kBits;
-#pragma unroll
-  for (int pass = 0; pass < KT::kPasses; ++pass) {
-    const int bits = KT::digit_bits(pass);
-    const int nb = 1 << bits;
-    shift -= bits;
-    for (int i = tid; i < nb; i += kTopkThreads) hist[i] = 0;
-    __syncthreads();
-#pragma unroll
-    for (int j = 0; j < IPT; ++j)
-      if ((key[j] & mask) == prefix && key[j] != 0u)
-        atomicAdd(&hist[(key[j] >> shift) & (nb - 1)], 1u);
-    __syncthreads();
-    const int bpt = nb >= kTopkThreads ? nb / kTopkThreads : 1;
-    const int my_bin = tid * bpt;
-    uint32_t local = 0;
-    if (my_bin < nb)
-      for (int j = 0; j < bpt; ++j) local += hist[my_bin + j];
-    const uint32_t suf = wave_suffix_sum(local, lane);
-    if (lane == 0) wave_tot[wave] = suf;
-    __syncthreads();
-    uint32_t above = suf - local;
-    for (int w = wave + 1; w < kTopkWaves; ++w) above += wave_tot[w];
-    if (my_bin < nb) {
-      for (int j = bpt - 1; j >= 0; --j) {
-        const uint32_t c = hist[my_bin + j];
-        if (above < krem && krem <= above + c) {
-          sh_bin = (uint32_t)(my_bin + j);
-          sh_krem = krem - above;
-        }
-        above += c;
-      }
-    }
-    __syncthreads();
-    prefix |= sh_bin << shift;
-    mask |= (uint32_t)(nb - 1) << shift;
-    krem = sh_krem;
-    __syncthreads();
-  }
-  const uint32_t thr = prefix;
-  const uint32_t r = krem;
-
-  // per-run counts: run (j, wave) covers elements j*1024 + wave*64 .. +64
-#pragma unroll
-  for (int j = 0; j < IPT; ++j) {
-    const uint32_t n_gt = (uint32_t)__popcll(__ballot(key[j] > thr));
-    const uint32_t n_eq = (uint32_t)__popcll(__ballot(key[j] == thr));
-    if (lane == 0) {
-      run_eq[j * kTopkWaves + wave] = n_eq;
-      run_out[j * kTopkWaves + wave] = n_gt;
-    }
-  }
-  __syncthreads();
-  // thread x handles run x (IPT * 16 <= 1024 runs): ties taken from each run, then output offsets
-  {
-    const bool has = tid < IPT * kTopkWaves;
-    const uint32_t e = has ? run_eq[tid] : 0u;
-    const uint32_t g = has ? run_out[tid] : 0u;
-    uint32_t total;
-    const uint32_t eq_before = block_exclusive_sum(e, lane, wave, wave_tot, total);
-    const uint32_t room = r > eq_before ? r - eq_before : 0u;
-    const uint32_t take = e < room ? e : room;
-    const uint32_t out_before = block_exclusive_sum(g + take, lane, wave, wave_tot, total);
-    if (has) {
-      run_eq[tid] = eq_before;
-      run_out[tid] = out_before;
-    }
-  }
-  __syncthreads();
-
-  const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
-  int32_t* out_idx = p.out_idx + (int64_t)row * p.out_stride;
-  elem_t* out_val =
-      p.out_values ? reinterpret_cast<elem_t*>(p.out_values) + (int64_t)row * p.out_stride : nullptr;
-#pragma unroll
-  for (int j = 0; j < IPT; ++j) {
-    const bool gt = key[j] > thr;
-    const bool eq = key[j] == thr;
-    const uint64_t eq_mask = __ballot(eq);
-    const uint32_t eq_rank = run_eq[j * kTopkWaves + wave] + (uint32_t)__popcll(eq_mask & lt_mask);
-    const bool sel = gt || (eq && eq_rank < r);
-    const uint64_t sel_mask = __ballot(sel);
-    const uint32_t pos = run_out[j * kTopkWaves + wave] + (uint32_t)__popcll(sel_mask & lt_mask);
-    if (sel && pos < (uint32_t)k) {
-      const int i = j * kTopkThreads + tid;
-      int32_t payload;
-      if (p.in_idx)
-        payload = p.in_idx[(int64_t)row * p.in_idx_stride + i];
-      else if (p.page_table)
-        payload = slot_of(p, table, i);
-      else
-        payload = i;
-      out_idx[pos] = payload;
-      if (out_val) out_val[pos] = vals[i];
-    }
-  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -893,28 +609,563 @@ __global__ __launch_bounds__(kTopkThreads) void topk_coop_emit_kernel(const Topk
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Sliced variant: one launch, no scratch, no exchange between workgroups.  A row is served by
+// n_slices workgroups that ALL run the selection on the whole row (the row is small: 128 KiB at
+// 32K fp32 scores, read once from HBM and again from the XCD's L2 by the other workgroups of the
+// row) and then each emit their own slice of it in position order.  Every workgroup of a row
+// computes the same threshold from the same data, so the slices agree.
+//
+// The selection is a radix select on d = kmax - key (kmax: the row's largest key; the k-th largest
+// key is the k-th smallest d) that starts at the first bit the row actually uses:
+//   1. the row as fp32-order keys in registers (IPT per thread; IPT == 0: rows that do not fit are
+//      re-read from L2 in every pass), kmax and kmin by reduction;
+//   2. an 8192-bin LDS histogram of (d - lo) >> s over the window [lo, lo + limit): first the
+//      8191 << 16 smallest d (values within 2^-64 of the maximum: 128 bins per binade, so the
+//      scores around the threshold spread over hundreds of bins and same-address LDS atomics are
+//      rare), or all of [0, kmax - kmin] with the smallest s that fits when that is narrower;
+//      what lies beyond the window is not counted at all;
+//   3. a scan finds the bin of the k-th smallest d; if it lies beyond the window, or the bin holds
+//      more keys than the LDS list, step 2 runs again on that narrower range;
+//   4. the bin's members (a few dozen) are gathered in LDS and ranked against each other by all
+//      threads (larger lists: further radix levels on the list): exact threshold T and the number
+//      r of keys equal to T that are taken, those at the lowest positions;
+//   5. one pass counts the selected elements in front of the slice and per 64-element run of the
+//      slice, a scan turns that into output offsets, and the slice is emitted.
+// ---------------------------------------------------------------------------------------------
+constexpr int kSliceBins = 8192;
+constexpr int kSliceCand = 1024;    // list entries in LDS; a fuller bin gets another level instead
+constexpr int kSliceRank = 128;     // lists up to this size are ranked directly
+constexpr int kSliceMaxRuns = 64;   // 1024-element runs a slice may hold
+
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t x) {  // 0 where the source lane does not exist
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, CTRL, 0xf, 0xf, true);
+}
+// inclusive prefix sum inside every row of 16 lanes (row_shr:1,2,4,8)
+__device__ __forceinline__ uint32_t row_prefix_sum(uint32_t x) {
+  x += dpp_u32<0x111>(x);
+  x += dpp_u32<0x112>(x);
+  x += dpp_u32<0x114>(x);
+  x += dpp_u32<0x118>(x);
+  return x;
+}
+// inclusive prefix sum over the wavefront
+__device__ __forceinline__ uint32_t wave_prefix_sum_dpp(uint32_t x, int lane) {
+  x = row_prefix_sum(x);
+  const uint32_t t0 = __builtin_amdgcn_readlane(x, 15), t1 = __builtin_amdgcn_readlane(x, 31),
+                 t2 = __builtin_amdgcn_readlane(x, 47);
+  return x + (lane >= 16 ? t0 : 0u) + (lane >= 32 ? t1 : 0u) + (lane >= 48 ? t2 : 0u);
+}
+// arr[0] + ... + arr[n - 1], n <= 16 and the same in the whole wavefront; result in a scalar
+__device__ __forceinline__ uint32_t sum_first(const uint32_t* arr, int n, int lane) {
+  const uint32_t v = row_prefix_sum(lane < n ? arr[lane & 15] : 0u);
+  return __builtin_amdgcn_readlane(v, 15);
+}
+// maximum over the wavefront (rows of 16 lanes by DPP, then the four rows); result in a scalar
+__device__ __forceinline__ int32_t wave_max_i32(int32_t x) {
+  int32_t y;
+  y = (int32_t)dpp_u32<0xB1>((uint32_t)x), x = x > y ? x : y;   // quad_perm [1,0,3,2]
+  y = (int32_t)dpp_u32<0x4E>((uint32_t)x), x = x > y ? x : y;   // quad_perm [2,3,0,1]
+  y = (int32_t)dpp_u32<0x141>((uint32_t)x), x = x > y ? x : y;  // row_half_mirror
+  y = (int32_t)dpp_u32<0x140>((uint32_t)x), x = x > y ? x : y;  // row_mirror
+  const int32_t a = __builtin_amdgcn_readlane(x, 0), b = __builtin_amdgcn_readlane(x, 16),
+                c = __builtin_amdgcn_readlane(x, 32), d = __builtin_amdgcn_readlane(x, 48);
+  const int32_t ab = a > b ? a : b, cd = c > d ? c : d;
+  return ab > cd ? ab : cd;
+}
+
+struct SliceLds {
+  uint32_t hist[kSliceBins];
+  uint32_t cd[kSliceCand];   // list: d of the members of the threshold bin
+  int32_t ci[kSliceCand];    //       and their positions
+  uint32_t run_eq[kSliceMaxRuns * kTopkWaves], run_gt[kSliceMaxRuns * kTopkWaves];
+  uint32_t wa[kTopkWaves], wb[kTopkWaves], wc[kTopkWaves];
+  uint32_t sh[4];
+  uint32_t n_cand;
+};
+
+// One radix level: histogram of (d - lo) >> s over the elements with d - lo < limit (for_each
+// hands every d of the row or of the list to its argument), then the bin of the krem-th smallest
+// of them.  True: bin in tb, its count in n_in, krem becomes the rank inside the bin.  False: fewer
+// than krem elements in the window; krem loses their number.  Four barriers; the caller has none
+// to add before the next level.
+template <class ForEach>
+__device__ __forceinline__ bool slice_level(SliceLds& L, ForEach for_each, uint32_t lo, int s,
+                                            uint32_t limit, uint32_t& krem, uint32_t& tb,
+                                            uint32_t& n_in, int tid, int lane, int wave) {
+  uint4* h4 = reinterpret_cast<uint4*>(L.hist);
+  h4[tid] = make_uint4(0, 0, 0, 0);
+  h4[tid + kTopkThreads] = make_uint4(0, 0, 0, 0);
+  __syncthreads();
+  for_each([&](uint32_t d) {
+    const uint32_t x = d - lo;
+    if (x < limit) atomicAdd(&L.hist[x >> s], 1u);
+  });
+  __syncthreads();
+  const uint4 a = h4[2 * tid], b = h4[2 * tid + 1];  // bins 8 tid .. 8 tid + 7
+  const uint32_t c[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+  const uint32_t local = ((a.x + a.y) + (a.z + a.w)) + ((b.x + b.y) + (b.z + b.w));
+  const uint32_t incl = wave_prefix_sum_dpp(local, lane);
+  if (lane == 63) L.wa[wave] = incl;
+  __syncthreads();
+  const uint32_t total = sum_first(L.wa, kTopkWaves, lane);
+  uint32_t before = sum_first(L.wa, wave, lane) + incl - local;
+  if (before < krem && krem <= before + local) {  // one thread of the workgroup, if any
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (before < krem && krem <= before + c[i]) {
+        L.sh[0] = (uint32_t)(8 * tid + i);
+        L.sh[1] = krem - before;
+        L.sh[2] = c[i];
+      }
+      before += c[i];
+    }
+  }
+  __syncthreads();
+  if (krem > total) {
+    krem -= total;
+    return false;
+  }
+  tb = __builtin_amdgcn_readfirstlane(L.sh[0]);
+  krem = __builtin_amdgcn_readfirstlane(L.sh[1]);
+  n_in = __builtin_amdgcn_readfirstlane(L.sh[2]);
+  return true;
+}
+
+// A row of scores behind a buffer descriptor: loads take the descriptor (scalar registers), one
+// 32-bit lane offset that is the same for every run, and the run's offset as a scalar, so dozens
+// of loads are in flight without an address register pair each; reads past the end of the row
+// return 0.  score_bits: bits of the fp32 value of element run * 1024 + tid.
+template <typename T>
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t row_descriptor(const void* row, int len) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(row), 0,
+                                           len * (int)sizeof(typename ElemOf<T>::type), 0x00020000);
+}
+template <typename T>
+__device__ __forceinline__ uint32_t score_bits(__amdgpu_buffer_rsrc_t row, int tid, int run);
+template <>
+__device__ __forceinline__ uint32_t score_bits<F32>(__amdgpu_buffer_rsrc_t row, int tid, int run) {
+  return __builtin_amdgcn_raw_buffer_load_b32(row, tid * 4, run * (kTopkThreads * 4), 0);
+}
+template <>
+__device__ __forceinline__ uint32_t score_bits<F16>(__amdgpu_buffer_rsrc_t row, int tid, int run) {
+  return __builtin_bit_cast(
+      uint32_t, to_float<F16>(__builtin_amdgcn_raw_buffer_load_b16(row, tid * 2, run * (kTopkThreads * 2), 0)));
+}
+template <>
+__device__ __forceinline__ uint32_t score_bits<BF16>(__amdgpu_buffer_rsrc_t row, int tid, int run) {
+  return __builtin_bit_cast(
+      uint32_t, to_float<BF16>(__builtin_amdgcn_raw_buffer_load_b16(row, tid * 2, run * (kTopkThreads * 2), 0)));
+}
+
+constexpr int kOwn = 8;                   // runs of a slice that stay in registers for the emission
+constexpr uint32_t kNoElement = ~0u;      // d of the slots past the end of the row: beyond every window
+
+template <typename T, int IPT>
+__global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(const TopkParams p, int n_slices,
+                                                                  int rps, int rows) {
+  typedef typename ElemOf<T>::type elem_t;
+  int slice, row;
+  if (!coop_decode(n_slices, rows, slice, row)) return;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int len = row_len(p, row);
+  const int k = row_k(p, len);
+  const elem_t* vals = reinterpret_cast<const elem_t*>(p.values) + (int64_t)row * p.values_stride;
+  const int nruns = (len + kTopkThreads - 1) / kTopkThreads;
+  const int j_lo = slice * rps;
+  if (j_lo >= nruns) return;  // a slice past the end of a short row (lengths on the device)
+  const int j_hi = j_lo + rps < nruns ? j_lo + rps : nruns;
+  const int n_own = j_hi - j_lo;
+  const int32_t* table = table_of(p, row);
+  auto payload_of = [&](int i) -> int32_t {
+    if (p.in_idx) return p.in_idx[(int64_t)row * p.in_idx_stride + i];
+    if (p.page_table) return slot_of(p, table, i);
+    return i;
+  };
+
+  __shared__ SliceLds L;
+
+  // ---- 1. the row's scores as raw fp32 bits; the extremes that fix the mapping to d ---------------
+  const __amdgpu_buffer_rsrc_t scores = row_descriptor<T>(vals, len);
+  uint32_t reg[IPT > 0 ? IPT : 1];
+  const uint32_t reg0 = score_bits<T>(scores, 0, 0);  // element 0, which every row has
+  int32_t imax = INT32_MIN;       // largest as signed integers: the largest non-negative score, if any
+  uint32_t umax = 0u, umin = ~0u;  // as unsigned integers: most negative score / smallest non-negative
+  // (only the row's last run has slots past the end; the empty asm keeps the compiler from turning
+  // the scalar branch around that case into selects on every run)
+  auto extremes = [&](int j, uint32_t u) {
+    if ((j + 1) * kTopkThreads > len) {
+      asm volatile("");
+      if (j * kTopkThreads + tid >= len) u = reg0;
+    }
+    imax = (int32_t)u > imax ? (int32_t)u : imax;
+    umax = u > umax ? u : umax;
+    umin = u < umin ? u : umin;
+  };
+  if constexpr (IPT > 0) {
+#pragma unroll
+    for (int j = 0; j < IPT; ++j) reg[j] = score_bits<T>(scores, tid, j);  // all in flight
+  }
+  if constexpr (IPT > 0) {
+#pragma unroll
+    for (int j = 0; j < IPT; ++j) extremes(j, reg[j]);
+  } else {
+    for (int jb = 0; jb < nruns; jb += 16) {
+      uint32_t uu[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) uu[u] = score_bits<T>(scores, tid, jb + u);
+#pragma unroll
+      for (int u = 0; u < 16; ++u) extremes(jb + u, uu[u]);
+    }
+  }
+  imax = wave_max_i32(imax);
+  umax = (uint32_t)wave_max_i32((int32_t)(umax ^ 0x80000000u)) ^ 0x80000000u;
+  umin = ~((uint32_t)wave_max_i32((int32_t)(~umin ^ 0x80000000u)) ^ 0x80000000u);
+  if (lane == 0) {
+    L.wa[wave] = (uint32_t)imax;
+    L.wb[wave] = umax ^ 0x80000000u;
+    L.wc[wave] = ~umin ^ 0x80000000u;
+  }
+  __syncthreads();
+  imax = wave_max_i32((int32_t)L.wa[lane & 15]);
+  umax = (uint32_t)wave_max_i32((int32_t)L.wb[lane & 15]) ^ 0x80000000u;
+  umin = ~((uint32_t)wave_max_i32((int32_t)L.wc[lane & 15]) ^ 0x80000000u);
+
+  // d: 0 for the row's largest score, growing as the scores fall, equal for equal scores (-0 == +0).
+  //   kMixed  some score is >= +0: d = top - u for the non-negative ones (integer order is value
+  //           order there), top + |u| for the negative ones, top = bits of the largest score
+  //   kNeg    all scores negative: d = u - (bits of the one closest to zero)
+  //   kCanon  a NaN in the row: d = kmax - key with the canonical keys (every NaN the maximum)
+  enum { kMixed, kNeg, kCanon };
+  int mode;
+  uint32_t top, dmax;
+  if (imax > 0x7f800000 || umax > 0xff800000u) {
+    mode = kCanon;
+    uint32_t kx = 0u, kn = ~0u;
+    auto key_extremes = [&](int j, uint32_t u) {
+      const uint32_t kv = KeyTraits<F32>::key(__builtin_bit_cast(float, u));
+      if (j * kTopkThreads + tid < len) {
+        kx = kv > kx ? kv : kx;
+        kn = kv < kn ? kv : kn;
+      }
+    };
+    if constexpr (IPT > 0) {
+#pragma unroll
+      for (int j = 0; j < IPT; ++j) key_extremes(j, reg[j]);
+    } else {
+      for (int j = 0; j < nruns; ++j) key_extremes(j, score_bits<T>(scores, tid, j));
+    }
+    kx = (uint32_t)wave_max_i32((int32_t)(kx ^ 0x80000000u));
+    kn = (uint32_t)wave_max_i32((int32_t)(~kn ^ 0x80000000u));
+    __syncthreads();  // wa, wb have been read
+    if (lane == 0) {
+      L.wa[wave] = kx;
+      L.wb[wave] = kn;
+    }
+    __syncthreads();
+    top = (uint32_t)wave_max_i32((int32_t)L.wa[lane & 15]) ^ 0x80000000u;
+    dmax = top - ~((uint32_t)wave_max_i32((int32_t)L.wb[lane & 15]) ^ 0x80000000u);
+  } else if (imax >= 0) {
+    mode = kMixed;
+    top = (uint32_t)imax;
+    dmax = umax >= 0x80000000u ? top + (umax - 0x80000000u) : top - umin;
+  } else {
+    mode = kNeg;
+    top = umin;
+    dmax = umax - umin;
+  }
+  const uint32_t neg_add = top - 0x80000000u;  // kMixed: d = u + neg_add for u with the sign bit
+  auto to_d = [&](uint32_t u) -> uint32_t {
+    if (mode == kMixed) return (int32_t)u >= 0 ? top - u : u + neg_add;
+    if (mode == kNeg) return u - top;
+    return top - KeyTraits<F32>::key(__builtin_bit_cast(float, u));
+  };
+  if constexpr (IPT > 0) {
+    if (mode == kMixed) {
+#pragma unroll
+      for (int j = 0; j < IPT; ++j) reg[j] = (int32_t)reg[j] >= 0 ? top - reg[j] : reg[j] + neg_add;
+    } else if (mode == kNeg) {
+#pragma unroll
+      for (int j = 0; j < IPT; ++j) reg[j] -= top;
+    } else {
+#pragma unroll
+      for (int j = 0; j < IPT; ++j)
+        reg[j] = top - KeyTraits<F32>::key(__builtin_bit_cast(float, reg[j]));
+    }
+#pragma unroll
+    for (int j = 0; j < IPT; ++j)
+      if ((j + 1) * kTopkThreads > len) {  // uniform: only the row's last run has slots past the end
+        asm volatile("");
+        reg[j] = j * kTopkThreads + tid < len ? reg[j] : kNoElement;
+      }
+  }
+  // f(j, d of element j * 1024 + tid) for the runs j0 <= j < j1 (j uniform); all = true: every
+  // run of the row, without the checks (the runs past the end hold nothing)
+  auto for_runs = [&](int j0, int j1, auto all, auto f) {
+    if constexpr (IPT > 0) {
+#pragma unroll
+      for (int j = 0; j < IPT; ++j)
+        if (decltype(all)::value || (j >= j0 && j < j1)) f(j, reg[j]);
+    } else {
+      for (int jb = j0; jb < j1; jb += 16) {
+        uint32_t uu[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) uu[u] = score_bits<T>(scores, tid, jb + u);
+#pragma unroll
+        for (int u = 0; u < 16; ++u)
+          if (jb + u < j1)
+            f(jb + u, (jb + u) * kTopkThreads + tid < len ? to_d(uu[u]) : kNoElement);
+      }
+    }
+  };
+  const std::true_type every_run;
+  const std::false_type some_runs;
+
+  // ---- 2./3. radix levels over the whole row until the threshold bin fits the list --------------
+  auto nbits = [](uint32_t x) { return x ? 32 - __builtin_clz(x) : 0; };
+  uint32_t lo = 0, krem = (uint32_t)k, tb = 0, n_in = 0;
+  int s = nbits(dmax) - 13;
+  uint32_t limit = dmax + 1u;  // dmax <= 0xff800000
+  if (s < 0) s = 0;
+  if (s > 16) {  // the 8191 << 16 smallest d first: 128 bins per binade
+    s = 16;
+    limit = (uint32_t)(kSliceBins - 1) << 16;
+  }
+  while (dmax != 0u) {  // (all scores equal: the first k positions, nothing to search)
+    const bool found = slice_level(
+        L, [&](auto f) { for_runs(0, nruns, every_run, [&](int, uint32_t d) { f(d); }); }, lo, s, limit,
+        krem, tb,
+        n_in, tid, lane, wave);
+    if (!found) {  // the threshold lies beyond the window: the rest of the range, as finely as fits
+      lo += limit;
+      const uint32_t rem = dmax - lo;
+      s = nbits(rem) - 13;
+      if (s < 0) s = 0;
+      limit = rem + 1u;
+      continue;
+    }
+    lo += tb << s;
+    if (s == 0 || n_in <= (uint32_t)kSliceCand) break;
+    limit = 1u << s;  // a crowded bin: its own range, 13 bits further down
+    s = s > 13 ? s - 13 : 0;
+  }
+  // the first runs of the own slice once more, as raw bits (they come from L2 while the members are
+  // ranked): the emission works on them with constant register numbers
+  uint32_t own[kOwn];
+#pragma unroll
+  for (int jj = 0; jj < kOwn; ++jj) own[jj] = score_bits<T>(scores, tid, j_lo + jj);
+  // the threshold is among the n_in elements with d - lo < 2^s, as the krem-th smallest of them
+  uint32_t thr = lo, r = krem;  // s == 0: they are all equal
+  if (s > 0) {
+    // ---- 4. the members into LDS, then rank them ---------------------------------------------------
+    if (tid == 0) L.n_cand = 0;
+    if (tid < kSliceRank) L.cd[tid] = kNoElement;  // padding: ranks behind every member
+    __syncthreads();
+    const uint32_t width = 1u << s;
+    for_runs(0, nruns, every_run, [&](int j, uint32_t d) {
+      const uint64_t m = __ballot(d - lo < width);
+      if (m) {  // rare: one LDS reservation per run and wave that holds a member
+        uint32_t at = 0;
+        if (lane == 0) at = atomicAdd(&L.n_cand, (uint32_t)__popcll(m));
+        at = __builtin_amdgcn_readfirstlane(at) + lanes_below(m);
+        if ((m >> lane) & 1ull) {
+          L.cd[at] = d;
+          L.ci[at] = j * kTopkThreads + tid;
+        }
+      }
+    });
+    __syncthreads();
+    if (n_in <= (uint32_t)kSliceRank) {
+      // every member against every other: thread (part, c) compares member c with members
+      // 16 part .. 16 part + 15
+      const int n_parts = ((int)n_in + 15) >> 4;
+      const int c = tid & (kSliceRank - 1), part = tid >> 7;  // part: the same in a wavefront
+      const uint32_t my_d = L.cd[c];
+      const int32_t my_i = L.ci[c];
+      if (part < n_parts) {
+        uint32_t g = 0, e = 0;
+        const uint4* d4 = reinterpret_cast<const uint4*>(L.cd) + part * 4;
+        const int4* i4 = reinterpret_cast<const int4*>(L.ci) + part * 4;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const uint4 dd = d4[u];
+          const int4 ii = i4[u];
+          g += (dd.x < my_d) + (dd.y < my_d) + (dd.z < my_d) + (dd.w < my_d);
+          e += (dd.x == my_d && ii.x < my_i) + (dd.y == my_d && ii.y < my_i) +
+               (dd.z == my_d && ii.z < my_i) + (dd.w == my_d && ii.w < my_i);
+        }
+        L.hist[part * kSliceRank + c] = g | (e << 16);
+      }
+      __syncthreads();
+      if (tid < (int)n_in) {
+        uint32_t t = 0;
+        for (int q = 0; q < n_parts; ++q) t += L.hist[q * kSliceRank + tid];
+        const uint32_t gg = t & 0xffffu, ee = t >> 16;
+        if (gg + ee == krem - 1u) {  // the last element taken: exactly one member
+          L.sh[0] = my_d;
+          L.sh[1] = ee + 1u;
+        }
+      }
+      __syncthreads();
+      thr = __builtin_amdgcn_readfirstlane(L.sh[0]);
+      r = __builtin_amdgcn_readfirstlane(L.sh[1]);
+    } else {
+      // the list stays as it is: every level narrows the window on it
+      const int n_list = (int)n_in;
+      uint32_t range = width;
+      while (s > 0) {
+        const int s2 = s > 13 ? s - 13 : 0;
+        slice_level(
+            L, [&](auto f) { for (int i = tid; i < n_list; i += kTopkThreads) f(L.cd[i]); }, lo, s2,
+            range, krem, tb, n_in, tid, lane, wave);
+        lo += tb << s2;
+        range = 1u << s2;
+        s = s2;
+      }
+      thr = lo;
+      r = krem;
+    }
+  }
+
+  // ---- 5. selected elements in front of this slice and per run of it -----------------------------
+  // selected: d < thr, and the first r (in position order) of d == thr
+  uint32_t bgt = 0, beq = 0;
+  for_runs(0, j_lo, some_runs, [&](int, uint32_t d) {
+    bgt += (uint32_t)__popcll(__ballot(d < thr));
+    beq += (uint32_t)__popcll(__ballot(d == thr));
+  });
+  if (lane == 0) {
+    L.wa[wave] = bgt;
+    L.wb[wave] = beq;
+  }
+  int32_t* out_idx = p.out_idx + (int64_t)row * p.out_stride;
+  elem_t* out_val =
+      p.out_values ? reinterpret_cast<elem_t*>(p.out_values) + (int64_t)row * p.out_stride : nullptr;
+  if (n_own <= kOwn) {
+    // the slice's runs from registers; every wave turns the (run, wave) counts into the offsets of
+    // its own 64-element pieces by itself: run jj, wave w is entry 16 jj + w, two entries per lane
+    uint32_t od[kOwn];
+#pragma unroll
+    for (int jj = 0; jj < kOwn; ++jj) {
+      const bool in = jj < n_own && (j_lo + jj) * kTopkThreads + tid < len;
+      od[jj] = in ? to_d(own[jj]) : kNoElement;
+      const uint32_t ng = (uint32_t)__popcll(__ballot(od[jj] < thr));
+      const uint32_t ne = (uint32_t)__popcll(__ballot(od[jj] == thr));
+      if (lane == 0) {
+        L.run_gt[jj * kTopkWaves + wave] = ng;
+        L.run_eq[jj * kTopkWaves + wave] = ne;
+      }
+    }
+    __syncthreads();
+    const uint32_t slice_gt = sum_first(L.wa, kTopkWaves, lane);
+    const uint32_t slice_eq = sum_first(L.wb, kTopkWaves, lane);
+    const uint2 g2 = reinterpret_cast<const uint2*>(L.run_gt)[lane];
+    const uint2 e2 = reinterpret_cast<const uint2*>(L.run_eq)[lane];
+    // exclusive prefix of the entry this wave reads from the lane: entry 2 lane + (wave & 1)
+    uint32_t xg = wave_prefix_sum_dpp(g2.x + g2.y, lane) - g2.y - ((wave & 1) ? 0u : g2.x);
+    uint32_t xe = wave_prefix_sum_dpp(e2.x + e2.y, lane) - e2.y - ((wave & 1) ? 0u : e2.x);
+#pragma unroll
+    for (int jj = 0; jj < kOwn; ++jj) {
+      if (jj >= n_own) break;
+      const int src = jj * (kTopkWaves / 2) + (wave >> 1);
+      const uint32_t eq_before = slice_eq + __builtin_amdgcn_readlane(xe, src);
+      const uint32_t out_before =
+          slice_gt + __builtin_amdgcn_readlane(xg, src) + (eq_before < r ? eq_before : r);
+      const bool eq = od[jj] == thr;
+      const uint32_t eq_rank = eq_before + lanes_below(__ballot(eq));
+      const bool sel = od[jj] < thr || (eq && eq_rank < r);
+      const uint32_t pos = out_before + lanes_below(__ballot(sel));
+      if (sel && pos < (uint32_t)k) {
+        const int i = (j_lo + jj) * kTopkThreads + tid;
+        out_idx[pos] = payload_of(i);
+        if (out_val) out_val[pos] = vals[i];
+      }
+    }
+    return;
+  }
+  // longer slices: counts per (run, wave), one thread per entry for the offsets
+  for_runs(j_lo, j_hi, some_runs, [&](int j, uint32_t d) {
+    const uint32_t ng = (uint32_t)__popcll(__ballot(d < thr));
+    const uint32_t ne = (uint32_t)__popcll(__ballot(d == thr));
+    if (lane == 0) {
+      L.run_gt[(j - j_lo) * kTopkWaves + wave] = ng;
+      L.run_eq[(j - j_lo) * kTopkWaves + wave] = ne;
+    }
+  });
+  __syncthreads();
+  {
+    const uint32_t slice_gt = sum_first(L.wa, kTopkWaves, lane);
+    const uint32_t slice_eq = sum_first(L.wb, kTopkWaves, lane);
+    const bool has = tid < n_own * kTopkWaves;
+    const uint32_t e = has ? L.run_eq[tid] : 0u, g = has ? L.run_gt[tid] : 0u;
+    const uint32_t ie = wave_prefix_sum_dpp(e, lane), ig = wave_prefix_sum_dpp(g, lane);
+    __syncthreads();  // wa, wb have been read
+    if (lane == 63) {
+      L.wa[wave] = ig;
+      L.wb[wave] = ie;
+    }
+    __syncthreads();
+    const uint32_t eq_before = slice_eq + sum_first(L.wb, wave, lane) + ie - e;
+    const uint32_t gt_before = slice_gt + sum_first(L.wa, wave, lane) + ig - g;
+    if (has) {
+      L.run_eq[tid] = eq_before;
+      L.run_gt[tid] = gt_before + (eq_before < r ? eq_before : r);  // output offset of the run
+    }
+  }
+  __syncthreads();
+  for_runs(j_lo, j_hi, some_runs, [&](int j, uint32_t d) {
+    const bool eq = d == thr;
+    const uint32_t eq_rank = L.run_eq[(j - j_lo) * kTopkWaves + wave] + lanes_below(__ballot(eq));
+    const bool sel = d < thr || (eq && eq_rank < r);
+    const uint32_t pos = L.run_gt[(j - j_lo) * kTopkWaves + wave] + lanes_below(__ballot(sel));
+    if (sel && pos < (uint32_t)k) {
+      const int i = j * kTopkThreads + tid;
+      out_idx[pos] = payload_of(i);
+      if (out_val) out_val[pos] = vals[i];
+    }
+  });
+}
+
+// Slices of a row for the sliced variant: enough workgroups to fill the chip when there are few
+// rows, one workgroup per row when there are many (every workgroup of a row repeats the selection
+// work on the whole row), whole 1024-element runs per slice.
+static void slice_shape(int len, int rows, int& n_slices, int& rps) {
+  const int nruns = (len + kTopkThreads - 1) / kTopkThreads;
+  int want = 256 / (rows < 1 ? 1 : rows);  // a 1024-thread workgroup has a compute unit to itself
+  if (want > nruns / 4) want = nruns / 4;  // at least 4 runs (4096 elements) per slice
+  if (want > kCoopMaxSlices) want = kCoopMaxSlices;
+  if (want < 1) want = 1;
+  rps = (nruns + want - 1) / want;
+  if (rps > kSliceMaxRuns) rps = kSliceMaxRuns;  // many long rows: more slices than wanted
+  n_slices = (nruns + rps - 1) / rps;
+}
+
+template <typename T>
+static void launch_topk_sliced(const TopkParams& p, int rows, hipStream_t st) {
+  int n_slices, rps;
+  slice_shape(p.len, rows, n_slices, rps);
+  const dim3 grid((rows + kXcds - 1) / kXcds * n_slices * kXcds), block(kTopkThreads);
+  if (p.len <= 8 * kTopkThreads)
+    hipLaunchKernelGGL((topk_slice_kernel<T, 8>), grid, block, 0, st, p, n_slices, rps, rows);
+  else if (p.len <= 16 * kTopkThreads)
+    hipLaunchKernelGGL((topk_slice_kernel<T, 16>), grid, block, 0, st, p, n_slices, rps, rows);
+  else if (p.len <= 24 * kTopkThreads)
+    hipLaunchKernelGGL((topk_slice_kernel<T, 24>), grid, block, 0, st, p, n_slices, rps, rows);
+  else if (p.len <= 32 * kTopkThreads)
+    hipLaunchKernelGGL((topk_slice_kernel<T, 32>), grid, block, 0, st, p, n_slices, rps, rows);
+  else if (p.len <= 40 * kTopkThreads)
+    hipLaunchKernelGGL((topk_slice_kernel<T, 40>), grid, block, 0, st, p, n_slices, rps, rows);
+  else  // longer rows would not fit the registers of a 1024-thread workgroup: re-read per pass
+    hipLaunchKernelGGL((topk_slice_kernel<T, 0>), grid, block, 0, st, p, n_slices, rps, rows);
+}
+
 // workgroups per row for the cooperative path, 0 if it does not apply
 static int coop_slices(int len, int rows) {
   const int g = (len + kCoopSlice - 1) / kCoopSlice;
   if (g < 2 || g > kCoopMaxSlices) return 0;  // short rows: one workgroup is as fast
   return g;
-}
-
-template <typename T>
-static void launch_topk(const TopkParams& p, int rows, hipStream_t st) {
-  const dim3 grid(rows), block(kTopkThreads);
-  if (p.len <= 8 * kTopkThreads)
-    hipLaunchKernelGGL((topk_reg_kernel<T, 8>), grid, block, 0, st, p);
-  else if (p.len <= 16 * kTopkThreads)
-    hipLaunchKernelGGL((topk_reg_kernel<T, 16>), grid, block, 0, st, p);
-  else if (p.len <= 32 * kTopkThreads)
-    hipLaunchKernelGGL((topk_reg_kernel<T, 32>), grid, block, 0, st, p);
-  else if (p.len <= 48 * kTopkThreads)
-    hipLaunchKernelGGL((topk_reg_kernel<T, 48>), grid, block, 0, st, p);
-  else if (p.len <= 64 * kTopkThreads)
-    hipLaunchKernelGGL((topk_reg_kernel<T, 64>), grid, block, 0, st, p);
-  else
-    hipLaunchKernelGGL(topk_kernel<T>, grid, block, 0, st, p);
 }
 
 // out[r, i] = sum_{h in row r} exp(logits[h, i] - lse[h])
@@ -992,9 +1243,14 @@ extern "C" int td_topk(const void* values, int32_t values_dtype, int64_t values_
   p.out_idx = out_idx;
   p.out_stride = out_stride;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  TD_REQUIRE(values_dtype == TD_F32 || values_dtype == TD_F16 || values_dtype == TD_BF16,
+             "Top-k filtering failed to dispatch with dtype %d", values_dtype);
+  // A few long rows: the three cooperative launches split each row over workgroups that share the
+  // work through the scratch.  Everything else: one launch in which every workgroup of a row goes
+  // through the whole row (rows up to 40K elements from registers) and emits its slice.
   const int slices = coop_slices(len, rows);
-  if (slices && workspace && workspace_bytes >= (int64_t)rows * kCoopRowWords * 4 &&
-      (values_dtype == TD_F32 || values_dtype == TD_F16 || values_dtype == TD_BF16)) {
+  if (len > 40 * kTopkThreads && slices && rows * slices <= 1024 && workspace &&
+      workspace_bytes >= (int64_t)rows * kCoopRowWords * 4) {
     uint32_t* ws = reinterpret_cast<uint32_t*>(workspace);
     const dim3 grid((rows + kXcds - 1) / kXcds * slices * kXcds), block(kTopkThreads);
     if (values_dtype == TD_F32) {
@@ -1010,16 +1266,12 @@ extern "C" int td_topk(const void* values, int32_t values_dtype, int64_t values_
       hipLaunchKernelGGL(topk_coop_select_kernel<BF16>, grid, block, 0, st, p, ws, slices, rows);
       hipLaunchKernelGGL(topk_coop_emit_kernel<BF16>, grid, block, 0, st, p, ws, slices, rows);
     }
-    TD_HIP_CHECK(hipGetLastError());
-    return TD_OK;
-  }
-  switch (values_dtype) {
-    case TD_F32: launch_topk<F32>(p, rows, st); break;
-    case TD_F16: launch_topk<F16>(p, rows, st); break;
-    case TD_BF16: launch_topk<BF16>(p, rows, st); break;
-    default:
-      return fail(TD_ERR_UNSUPPORTED, "Top-k filtering failed to dispatch with dtype %d",
-                  values_dtype);
+  } else if (values_dtype == TD_F32) {
+    launch_topk_sliced<F32>(p, rows, st);
+  } else if (values_dtype == TD_F16) {
+    launch_topk_sliced<F16>(p, rows, st);
+  } else {
+    launch_topk_sliced<BF16>(p, rows, st);
   }
   TD_HIP_CHECK(hipGetLastError());
   return TD_OK;
