@@ -25,8 +25,9 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # HBM bytes one sparse-layer launch of the default workload moves, from rocprofv3 FETCH_SIZE /
-# WRITE_SIZE scaled by a plain 256 MiB copy (profiles/decode_attn_sparse_llama2-7b_ctx32k_top2048.md)
-TRAFFIC_DEFAULT_WORKLOAD = 35291948
+# WRITE_SIZE scaled by a plain 256 MiB copy (profiles/sparse_attn_kernel_llama2-7b_ctx32k_top2048.md):
+# (16621.0 KiB x 2.00 + 169.0 KiB x 1.00) x 1024
+TRAFFIC_DEFAULT_WORKLOAD = 34212864
 
 
 def parse():
@@ -72,6 +73,8 @@ def parse():
     ap.add_argument("--no-real-prompt", action="store_true",
                     help="end-to-end leg: skip the real prompt (prefill of random tokens through "
                          "the decoder, then greedy decoding)")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the legs of benchmark configurations 2 and 4 and the Quest bar")
     ap.add_argument("--extra-only", action="store_true",
                     help="profile helper: run only the prefill, batch-8 and end-to-end legs and "
                          "print their JSON object")
@@ -84,7 +87,7 @@ def parse():
 class Workload:
     """Controller + synthetic per-layer q/k/v for one decode step at a fixed context length."""
 
-    def __init__(self, args, select_mode):
+    def __init__(self, args, select_mode, sel_layers=(0, 2)):
         import torch
 
         from tidaldecode_amd.utils import InferenceController
@@ -94,7 +97,7 @@ class Workload:
         self.L, self.H, self.D, self.P = args.layers, args.heads, 128, 16
         self.HKV = args.kv_heads
         self.N, self.K = args.ctx, args.top_k
-        self.sel_layers = (0, 2)
+        self.sel_layers = tuple(sel_layers)
         self.dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float16
         c = InferenceController(self.L, self.H, self.D, self.P, self.K, self.N + 64, self.dtype,
                                 self.dev, num_kv_heads=self.HKV, select_mode=select_mode,
@@ -294,8 +297,9 @@ def cpu_baseline(args, budget_s=12.0):
     }
 
 
-def e2e_leg(args):
-    """End-to-end decode of a Llama-2-7B-shape decoder with random bf16 weights (the library's
+def e2e_leg(args, shape=None, ctxs=None, top_k=None, select_mode=None, steps=None,
+            real_prompt=None, n_greedy=None):
+    """End-to-end decode of a Llama-shape decoder with random bf16 weights (the library's
     fused matrix-vector launches around its attention path), TidalDecode schedule vs. the same decoder with
     full attention in every layer, at each context length.  One decode step at that context is
     captured as a hipGraph and replayed (steady-state per-token latency; the cache holds
@@ -304,13 +308,21 @@ def e2e_leg(args):
 
     from tidaldecode_amd.llama import TidalLlama, TidalLlamaConfig
 
-    ctxs = [int(x) for x in args.e2e_ctx.split(",") if x]
-    if args.e2e_shape == "llama3_8b":
-        cfg = TidalLlamaConfig.llama3_8b(top_k=args.top_k, sparse_layer_start=0, correction_layer=13,
-                                         select_mode=args.select_mode)
+    shape = shape or args.e2e_shape
+    ctxs = ctxs or [int(x) for x in args.e2e_ctx.split(",") if x]
+    top_k = top_k or args.top_k
+    select_mode = select_mode or args.select_mode
+    steps = steps or max(10, args.steps // 2)
+    real_prompt = (not args.no_real_prompt) if real_prompt is None else real_prompt
+    if shape == "llama3_8b":
+        cfg = TidalLlamaConfig.llama3_8b(top_k=top_k, sparse_layer_start=0, correction_layer=13,
+                                         select_mode=select_mode)
+    elif shape == "cfg4":
+        cfg = TidalLlamaConfig.cfg4(top_k=top_k, sparse_layer_start=0, correction_layer=2,
+                                    select_mode=select_mode)
     else:
-        cfg = TidalLlamaConfig.llama2_7b(top_k=args.top_k, sparse_layer_start=0, correction_layer=2,
-                                         select_mode=args.select_mode)
+        cfg = TidalLlamaConfig.llama2_7b(top_k=top_k, sparse_layer_start=0, correction_layer=2,
+                                         select_mode=select_mode)
     model = TidalLlama(cfg, "cuda:0", seed=0)
     model.tidal_init(page_size=16, max_seq_len=max(ctxs) + 512, page_order_seed=0)
     out = {}
@@ -320,8 +332,7 @@ def e2e_leg(args):
             cfg.attn_type = kind
             model.tidal_clear()
             model.synthetic_prefill(ctx)
-            dt, how = model.timed_decode(steps=max(10, args.steps // 2), warmup=3,
-                                         use_graph=not args.no_graph)
+            dt, how = model.timed_decode(steps=steps, warmup=3, use_graph=not args.no_graph)
             row[f"{kind}_ms_per_token"] = round(dt * 1e3, 4)
             row[f"{kind}_tokens_per_s"] = round(1.0 / dt, 2)
             row["launch"] = how
@@ -331,8 +342,7 @@ def e2e_leg(args):
         model.use_gemv = False
         model.tidal_clear()
         model.synthetic_prefill(ctx)
-        dt, _ = model.timed_decode(steps=max(10, args.steps // 2), warmup=3,
-                                   use_graph=not args.no_graph)
+        dt, _ = model.timed_decode(steps=steps, warmup=3, use_graph=not args.no_graph)
         model.use_gemv = True
         row["tidal_torch_linear_ms_per_token"] = round(dt * 1e3, 4)
         # a real greedy loop: eager launches, the sequence grows by one token per step, one
@@ -349,7 +359,7 @@ def e2e_leg(args):
             tok = model.decode_step(tok).argmax().view(1)
         torch.cuda.synchronize()
         row["tidal_eager_generate_ms_per_token"] = round((time.perf_counter() - t0) / n_gen * 1e3, 4)
-        if not args.no_real_prompt:
+        if real_prompt:
             # the configuration as written: a random-token prompt runs through the decoder (paged
             # prefill attention, K/V appended to the cache), then greedy decoding, every step real
             model.tidal_clear()
@@ -360,7 +370,7 @@ def e2e_leg(args):
             tok = model.prefill(ids).argmax().view(1)
             torch.cuda.synchronize()
             t1 = time.perf_counter()
-            n_gen = 256 if ctx <= 32768 else 128
+            n_gen = n_greedy or (256 if ctx <= 32768 else 128)
             for _ in range(n_gen):
                 tok = model.decode_step(tok).argmax().view(1)
             torch.cuda.synchronize()
@@ -444,6 +454,159 @@ def sweep(args):
             del w
             torch.cuda.empty_cache()
     return out
+
+
+def attention_path_row(args, layers, heads, kv_heads, ctx, top_k, select_mode, sel_layers):
+    """Attention path of one decode step for one model shape at one context: the sparse-layer
+    launch with its HBM roofline fraction, the whole step, and the same step with full attention in
+    every layer (the ratio the reference plots)."""
+    import copy
+
+    import torch
+
+    a = copy.copy(args)
+    a.layers, a.heads, a.kv_heads, a.ctx, a.top_k = layers, heads, kv_heads, ctx, top_k
+    w = Workload(a, select_mode, sel_layers)
+    w.step()
+    torch.cuda.synchronize()
+    use_graph = not args.no_graph
+    sparse = w.sparse_layers()
+
+    def run_sparse():
+        for layer in sparse:
+            w.sparse_attn(layer, w.fresh(layer) if w.fuse else None)
+
+    r, how = capture(torch, run_sparse, use_graph)
+    sparse_us = time_events(torch, r, 20) * 1e3 / len(sparse)
+    r_step, _ = capture(torch, w.step, use_graph)
+    step_ms = time_events(torch, r_step, 20)
+
+    def full_step():
+        if w.fuse:
+            w.rope_table()
+        for layer in range(w.L):
+            if not w.fuse:
+                w.rope_append(layer)
+            w.full_attn(layer, w.fresh(layer) if w.fuse else None)
+
+    r_full, _ = capture(torch, full_step, use_graph)
+    full_ms = time_events(torch, r_full, 5, warm=1)
+    rows = w.c.index_rows
+    k_eff = w.c.num_selected
+    gathered_heads = w.H if rows == w.H else w.HKV
+    algo = k_eff * gathered_heads * w.D * 2 * 2 + k_eff * rows * 4 + 2 * w.H * w.D * 2
+    n_cached = w.c.kv_cache.seqlen
+    full_bytes = n_cached * w.HKV * w.D * 2 * 2 + 2 * w.H * w.D * 2
+    out = {"ctx": ctx, "top_k": k_eff, "launch": how,
+           "sparse_layer": {"us_per_launch": round(sparse_us, 3), "algorithmic_bytes": algo,
+                            "achieved_gbs": round(algo / sparse_us / 1e3, 1),
+                            "frac": round(algo / sparse_us / 1e3 / HBM_PEAK_GBS, 4)},
+           "full_layer": {"us_per_launch": round(full_ms * 1e3 / w.L, 3), "algorithmic_bytes": full_bytes,
+                          "achieved_gbs": round(full_bytes / (full_ms * 1e3 / w.L) / 1e3, 1),
+                          "frac": round(full_bytes / (full_ms * 1e3 / w.L) / 1e3 / HBM_PEAK_GBS, 4)},
+           "tidal_attention_ms_per_step": round(step_ms, 4),
+           "full_attention_ms_per_step": round(full_ms, 4),
+           "attention_ratio_vs_full": round(step_ms / full_ms, 4)}
+    del w
+    torch.cuda.empty_cache()
+    return out
+
+
+def configs_leg(args):
+    """Benchmark configurations 2 and 4 (configuration 1 is the main line and its end-to-end leg,
+    configuration 3 the batch-of-8 leg):
+    cfg2  Llama-3-8B shape (GQA 32/8), 100K context, 4096 tokens, selection at layers 0 and 13:
+          attention path and the decoder end to end (random-token prompt through the decoder,
+          128 greedy steps);
+    cfg4  64 layers, hidden 5120, 40 heads, 2048 tokens, selection at layers 0 and 2: attention
+          path against full attention at 10K / 32K / 100K, and the decoder end to end at 10K and
+          32K (synthetic cache, 128 timed steps)."""
+    out = {}
+    cfg2 = attention_path_row(args, 32, 32, 8, 102400, 4096, "group_sum", (0, 13))
+    cfg2["shape"] = "32 layers, 32/8 heads x 128, bf16, page 16, group_sum lists, selection at layers 0 and 13"
+    if not args.no_e2e:
+        cfg2["e2e_decode"] = e2e_leg(args, "llama3_8b", [102400], 4096, "group_sum", steps=128,
+                                     n_greedy=128)["102400"]
+    out["cfg2_llama3_8b_ctx100k_top4096"] = cfg2
+    cfg4 = {"shape": "64 layers, 40/40 heads x 128, bf16, page 16, per_head lists, selection at layers 0 and 2",
+            "attention_path": [attention_path_row(args, 64, 40, 40, ctx, 2048, "per_head", (0, 2))
+                               for ctx in (10240, 32768, 102400)]}
+    if not args.no_e2e:
+        cfg4["e2e_decode"] = e2e_leg(args, "cfg4", [10240, 32768], 2048, "per_head", steps=128,
+                                     real_prompt=False)
+    out["cfg4_64layers_hidden5120_40heads_top2048"] = cfg4
+    return out
+
+
+def quest_leg(args):
+    """The reference's comparison bar (README latency figure: Quest 1.24 / 0.66 / 0.41 of full
+    attention at 10K / 32K / 100K against TidalDecode's 0.65 / 0.37 / 0.24): the attention path of
+    a Quest-style decode step built from this library's pieces.  Layers 0 and 1 attend to the whole
+    cache; every later layer estimates an upper bound of the logits per KV page from the page's
+    key max / min (decode_estimate), takes the top pages (topk_filtering over the page bounds) and
+    attends to those pages (page-list mode) plus the page being filled.  The page budget is
+    top_k / page_size pages, the same token budget as the TidalDecode step beside it.  RoPE and
+    append run as their own launches here because the append also updates the page bounds."""
+    import torch
+
+    from tidaldecode_amd import _kernels
+    from tidaldecode_amd import utils as ops
+    from tidaldecode_amd.utils import InferenceController
+
+    dev = torch.device("cuda:0")
+    dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float16
+    layers, h, d, page = 32, 32, 128, 16
+    use_graph = not args.no_graph
+    rows = []
+    for ctx in (10240, 32768, 102400):
+        tidal = attention_path_row(args, layers, h, h, ctx, args.top_k, "per_head", (0, 2))
+        c = InferenceController(layers, h, d, page, args.top_k, ctx + 64, dtype, dev,
+                                with_metadata=True, page_order_seed=0)
+        c.kv_cache.pool.buf.normal_()
+        c.metadata_cache.pool.buf.normal_()
+        c.prepare_metadata(ctx)
+        c.prepare_metadata(1)
+        c.begin_forward(1)
+        g = torch.Generator(device=dev).manual_seed(0)
+        q = torch.randn((layers, 1, h, d), generator=g, device=dev).to(dtype)
+        k = torch.randn((layers, 1, h, d), generator=g, device=dev).to(dtype)
+        v = torch.randn((layers, 1, h, d), generator=g, device=dev).to(dtype)
+        o = torch.empty_like(q[0])
+        n_pages = len(c.kv_cache.indicies)
+        budget = min(args.top_k // page, n_pages - 1)
+        page_ids = c.kv_indices_without_last.expand(h, -1).contiguous()  # physical page per position
+        chosen = torch.zeros((h, budget), dtype=torch.int32, device=dev)
+        pos = c.kv_cache.seqlen - 1
+
+        def quest_step():
+            for layer in range(layers):
+                ops.apply_rope_in_place(q[layer], k[layer], pos)
+                ops.append_kv(k[layer], v[layer], c, layer)
+                kv = c.kv_cache.buf_layer(layer)
+                if layer < 2:
+                    c._decode_handler.forward(q[layer], o, kv, c.kv_indices_without_last, None,
+                                              c.kv_cache.last_page_len, c.kv_last_page_idx, None)
+                    continue
+                est = ops.decode_estimate(q[layer], c, layer)
+                _kernels.topk_filtering(est, page_ids, None, chosen, c.topk_buf, budget)
+                c._decode_handler.forward(q[layer], o, kv, chosen, None, c.kv_cache.last_page_len,
+                                          c.kv_last_page_idx, None, index_kind="pages")
+
+        r, how = capture(torch, quest_step, use_graph)
+        quest_ms = time_events(torch, r, 20)
+        full_ms = tidal["full_attention_ms_per_step"]
+        rows.append({"ctx": ctx, "token_budget": budget * page, "launch": how,
+                     "quest_attention_ms_per_step": round(quest_ms, 4),
+                     "tidal_attention_ms_per_step": tidal["tidal_attention_ms_per_step"],
+                     "full_attention_ms_per_step": full_ms,
+                     "quest_ratio_vs_full": round(quest_ms / full_ms, 4),
+                     "tidal_ratio_vs_full": tidal["attention_ratio_vs_full"]})
+        c.clean_states()
+        del c, q, k, v
+        torch.cuda.empty_cache()
+    return {"shape": f"{layers} layers, {h}/{h} heads x {d}, {args.dtype}, page {page}", "rows": rows,
+            "reference_figure": {"quest": [1.24, 0.66, 0.41], "tidal": [0.65, 0.37, 0.24],
+                                 "note": "README llama_latency_eval figure, other hardware"}}
 
 
 def batch8_leg(args):
@@ -558,6 +721,9 @@ def main():
             extra["batch8_sparse_attn"] = batch8_leg(args)
         if not args.no_e2e:
             extra[f"e2e_decode_{args.e2e_shape}_shape"] = e2e_leg(args)
+        if not args.no_configs:
+            extra["configs"] = configs_leg(args)
+            extra["quest_comparison"] = quest_leg(args)
         print(json.dumps(extra))
         return
     results = {}
@@ -624,8 +790,10 @@ def main():
                 for layer in w.sel_layers:
                     w.select_attn(layer, w.fresh(layer) if w.fuse else None)
 
+            n_topk = 16   # launches per graph replay: the replay's own overhead stays below 1 us each
+
             def run_topk():
-                for _ in w.sel_layers:
+                for _ in range(n_topk):
                     w.topk()
 
             def run_rope():
@@ -635,7 +803,7 @@ def main():
             r, _ = capture(torch, run_select, use_graph)
             entry["selection_attn_us_per_layer"] = time_events(torch, r, 20) * 1e3 / len(w.sel_layers)
             r, _ = capture(torch, run_topk, use_graph)
-            entry["topk_us_per_layer"] = time_events(torch, r, 20) * 1e3 / len(w.sel_layers)
+            entry["topk_us_per_layer"] = time_events(torch, r, 20) * 1e3 / n_topk
             r, _ = capture(torch, run_rope, use_graph)
             entry["rope_append_us_per_layer"] = time_events(torch, r, 20) * 1e3 / w.L
             # the contract's timed region: W warm-up steps, then exactly K steps
@@ -709,7 +877,7 @@ def main():
                         if (args.ctx, args.top_k, args.layers, main_mode, args.heads, args.kv_heads,
                             args.dtype) == (32768, 2048, 32, "per_head", 32, 32, "bf16")
                         else None),
-            "kernel": "decode_attn_kernel (sparse layer, token-slot lists)",
+            "kernel": "sparse_attn_kernel (sparse layer, token-slot lists, fused RoPE + append)",
             "algorithmic_bytes_per_launch": e["algorithmic_bytes"],
         },
         "detail": {m: {k: (round(v, 3) if isinstance(v, float) else v) for k, v in r.items()}
@@ -722,6 +890,9 @@ def main():
         line["batch8_sparse_attn"] = batch8_leg(args)
     if not args.no_e2e and not args.only_sparse:
         line[f"e2e_decode_{args.e2e_shape}_shape"] = e2e_leg(args)
+    if not args.no_configs and not args.only_sparse:
+        line["configs"] = configs_leg(args)
+        line["quest_comparison"] = quest_leg(args)
     if not args.no_cpu and not args.only_sparse:
         line["cpu_baseline"] = cpu_baseline(args)
     print(json.dumps(line))

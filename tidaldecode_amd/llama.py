@@ -51,6 +51,12 @@ class TidalLlamaConfig:
     def llama3_8b(**kw):
         return TidalLlamaConfig(32, 4096, 32, 8, 128, 14336, 128256, 5e5, **kw)
 
+    @staticmethod
+    def cfg4(**kw):
+        """The deep decoder of the latency sweep: 64 layers, hidden 5120, 40 heads (MHA), MLP width
+        of the 13B Llama."""
+        return TidalLlamaConfig(64, 5120, 40, 40, 128, 13824, 32000, 1e4, **kw)
+
     def layer_kind(self, layer: int) -> str:
         if self.attn_type == "full" or layer < self.sparse_layer_start:
             return "full"
