@@ -278,6 +278,65 @@ def test_page_score_estimator(cuda, dtype, hq, hkv, d, page, layout):
         assert ((got.float().cpu() - want).abs() <= tol).all()
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("hq,hkv,page,n,budget", [(32, 32, 16, 4099, 32), (8, 2, 4, 1110, 40),
+                                                  (4, 4, 16, 213, 5)])
+def test_quest_style_step(cuda, dtype, hq, hkv, page, n, budget):
+    """The page-selection step of the reference's ancestor built from the library's pieces, as
+    bench.py times it: decode_estimate (upper bound of the logits per page) -> topk_filtering over
+    the bounds with the physical page of each position as payload -> attention over the chosen
+    pages plus the page being filled.  The chosen pages are bit-exact against the oracle's stable
+    top-k of the oracle's bound on the same rounded scores, the attention output against the
+    oracle's attention over the tokens of those pages."""
+    from oracle import tidal_oracle as orc
+    from tidaldecode_amd import _kernels
+    from tidaldecode_amd import utils as ops
+    from tidaldecode_amd.utils import InferenceController
+
+    d = 128
+    c = InferenceController(1, hq, d, page, 64, n + 64, dtype, cuda, num_kv_heads=hkv,
+                            with_metadata=True, page_order_seed=3)
+    g = torch.Generator().manual_seed(n + budget)
+    k = torch.randn((n, hkv, d), generator=g).to(dtype)
+    v = torch.randn((n, hkv, d), generator=g).to(dtype)
+    q = torch.randn((1, hq, d), generator=g).to(dtype)
+    c.prepare_metadata(n - 1)
+    c.begin_forward(n - 1)
+    ops.append_kv(k[:n - 1].to(cuda), v[:n - 1].to(cuda), c, 0)
+    c.end_forward()
+    c.prepare_metadata(1)
+    c.begin_forward(1)
+    ops.append_kv(k[n - 1:].to(cuda), v[n - 1:].to(cuda), c, 0)
+    est = ops.decode_estimate(q.to(cuda), c, 0)                       # [hq, n_pages - 1]
+    n_pages = (n + page - 1) // page
+    assert est.shape == (hq, n_pages - 1) and budget <= n_pages - 1
+    page_ids = c.kv_indices_without_last.expand(hq, -1).contiguous()
+    chosen = torch.full((hq, budget), -1, dtype=torch.int32, device=cuda)
+    _kernels.topk_filtering(est, page_ids, None, chosen, c.topk_buf, budget)
+    o = torch.empty_like(q, device=cuda)
+    c._decode_handler.forward(q.to(cuda), o, c.kv_cache.buf_layer(0), chosen, None,
+                              c.kv_cache.last_page_len, c.kv_last_page_idx, None, index_kind="pages")
+    torch.cuda.synchronize()
+    # the bound itself (fp32 oracle on the rounded keys), then the selection on the GPU's own scores
+    bound = orc.page_score_bound(q[0].float(), k.float(), page)[:, : n_pages - 1]
+    tol = (2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7) * bound.abs().clamp(min=1.0) + 1e-3
+    assert ((est.float().cpu() - bound).abs() <= tol).all()
+    logical = orc.stable_topk(est.float().cpu(), budget)              # [hq, budget] logical pages
+    table = c.kv_cache.indices_device.cpu().long()
+    assert torch.equal(chosen.cpu().long(), table[logical])
+    # attention over the tokens of the chosen pages and of the last page
+    want = torch.empty((hq, d))
+    last = torch.arange((n_pages - 1) * page, n)
+    for h in range(hq):
+        tok = torch.cat([(logical[h][:, None] * page + torch.arange(page)[None]).flatten(), last])
+        kh, vh = k[tok, h // (hq // hkv)].float(), v[tok, h // (hq // hkv)].float()
+        p = torch.softmax(kh @ q[0, h].float() / d ** 0.5, 0)
+        want[h] = p @ vh
+    tol_o = 2e-3 if dtype == torch.float16 else 1e-2
+    assert (o[0].float().cpu() - want).abs().max().item() <= tol_o
+    c.clean_states()
+
+
 @pytest.mark.parametrize("head_dim", [64, 128])
 @pytest.mark.parametrize("page_size", [1, 3, 7, 16, 32])
 def test_page_score_estimator_reference_grid(cuda, head_dim, page_size):
