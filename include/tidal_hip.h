@@ -347,7 +347,7 @@ int td_topk(const void* values, int32_t values_dtype, int64_t values_stride, int
             void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
- * Bytes of device scratch for td_topk.  Rows of up to 40960 elements never touch it (one launch,
+ * Bytes of device scratch for td_topk.  Rows of up to 65536 elements never touch it (one launch,
  * every workgroup of a row selects on the whole row and emits a slice).  A few longer rows are
  * shared between workgroups through it (three launches; about 56 KiB per row); without it (NULL),
  * or with many long rows, the one-launch kernel re-reads such rows from L2 in every pass.  The

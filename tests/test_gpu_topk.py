@@ -16,7 +16,7 @@ _scratch = {}
 
 def _shared_scratch(cuda, rows):
     """One scratch tensor for the whole module: zeroed at allocation only, so every cooperative
-    call after the first (rows of more than 40960 elements) relies on the previous call having
+    call after the first (rows of more than 65536 elements) relies on the previous call having
     left it clean."""
     from tidaldecode_amd import _kernels
 
@@ -52,7 +52,7 @@ def _check(values, k, cuda):
     assert np.array_equal(got.numpy(), want_c)
     expect = torch.gather(values, 1, want)  # values travel with their index (NaN == NaN here)
     assert torch.equal(torch.nan_to_num(vals.float(), nan=1e38), torch.nan_to_num(expect.float(), nan=1e38))
-    # with scratch: rows of more than 40960 elements take the three cooperative launches
+    # with scratch: rows of more than 65536 elements take the three cooperative launches
     got2, vals2 = _gpu_topk(values, k, cuda, scratch=True)
     assert torch.equal(got2, got), "cooperative path differs"
     assert torch.equal(torch.nan_to_num(vals2.float(), nan=1e38), torch.nan_to_num(vals.float(), nan=1e38))

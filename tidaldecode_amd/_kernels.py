@@ -166,7 +166,7 @@ def topk_filtering(estimated_value: torch.Tensor, estimated_indices: Optional[to
     ``[H, len]``; ``indices_out[h, j]`` is ``estimated_indices[h, p]`` of the selected position
     ``p``.  ``buf`` is scratch, as in the reference (there: RAFT's): a zero-initialised uint8 /
     any-dtype device tensor of at least ``topk_workspace_bytes(H)`` bytes through which the
-    workgroups of a row of more than 40960 elements share the work; shorter rows never touch it,
+    workgroups of a row of more than 65536 elements share the work; shorter rows never touch it,
     and without it (smaller or ``None``) every workgroup of a long row goes through the whole row.
     The call leaves ``buf`` zeroed where it must be for the next call.
 

@@ -8,10 +8,10 @@
 //
 // Two routes:
 //   * topk_slice_kernel, one launch: every workgroup (1024 threads) of a row runs the selection on
-//     the whole row -- up to 40K elements from registers -- and emits its own slice of it.  All
-//     rows of up to 40960 elements, and longer ones when there are many rows or no scratch.
+//     the whole row -- up to 64K elements from registers -- and emits its own slice of it.  All
+//     rows of up to 65536 elements, and longer ones when there are many rows or no scratch.
 //   * topk_coop_{hist,select,emit}_kernel, three launches over a zeroed scratch: the workgroups of
-//     a row share the row.  A few rows of more than 40960 elements.
+//     a row share the row.  A few rows of more than 65536 elements.
 //
 // Replaces decode_select_k (kernels/include/topk/decode_select_k.cuh:25-62 of the reference),
 // which launches RAFT's radix_topk_one_block_kernel, one 512-thread block per head.
@@ -119,9 +119,9 @@ __device__ __forceinline__ uint32_t block_exclusive_sum(uint32_t x, int lane, in
 }
 
 // ---------------------------------------------------------------------------------------------
-// Cooperative variant: G workgroups per row, two launches.  One compute unit needs ~40 us to
-// push a 32K-element row through the single-workgroup kernels above (the row costs ~40K wave
-// instructions); with a handful of rows that leaves the other 200+ compute units idle.
+// Cooperative variant: G workgroups per row, three launches, for rows too long to keep in the
+// registers of one workgroup (more than 65536 elements) when there are few of them: the
+// workgroups of a row split the row instead of each going through all of it.
 //
 //   launch 1 (topk_coop_hist_kernel, grid G x rows): every workgroup histograms the top 11 key
 //     bits of its slice in LDS and adds the non-empty bins to a per-row global histogram.
@@ -759,6 +759,7 @@ __device__ __forceinline__ uint32_t score_bits<BF16>(__amdgpu_buffer_rsrc_t row,
       uint32_t, to_float<BF16>(__builtin_amdgcn_raw_buffer_load_b16(row, tid * 2, run * (kTopkThreads * 2), 0)));
 }
 
+constexpr int kStream = 16;               // loads in flight per thread where a row is re-read per pass
 constexpr int kOwn = 8;                   // runs of a slice that stay in registers for the emission
 constexpr uint32_t kNoElement = ~0u;      // d of the slots past the end of the row: beyond every window
 
@@ -810,14 +811,19 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(const TopkPara
   }
   if constexpr (IPT > 0) {
 #pragma unroll
-    for (int j = 0; j < IPT; ++j) extremes(j, reg[j]);
+    for (int j8 = 0; j8 < IPT; j8 += 8) {
+      if (j8 < nruns) {
+#pragma unroll
+        for (int j = j8; j < j8 + 8; ++j) extremes(j, reg[j]);
+      }
+    }
   } else {
-    for (int jb = 0; jb < nruns; jb += 16) {
-      uint32_t uu[16];
+    for (int jb = 0; jb < nruns; jb += kStream) {
+      uint32_t uu[kStream];
 #pragma unroll
-      for (int u = 0; u < 16; ++u) uu[u] = score_bits<T>(scores, tid, jb + u);
+      for (int u = 0; u < kStream; ++u) uu[u] = score_bits<T>(scores, tid, jb + u);
 #pragma unroll
-      for (int u = 0; u < 16; ++u) extremes(jb + u, uu[u]);
+      for (int u = 0; u < kStream; ++u) extremes(jb + u, uu[u]);
     }
   }
   imax = wave_max_i32(imax);
@@ -906,15 +912,20 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(const TopkPara
   auto for_runs = [&](int j0, int j1, auto all, auto f) {
     if constexpr (IPT > 0) {
 #pragma unroll
-      for (int j = 0; j < IPT; ++j)
-        if (decltype(all)::value || (j >= j0 && j < j1)) f(j, reg[j]);
+      for (int j8 = 0; j8 < IPT; j8 += 8) {
+        if (j8 < nruns) {  // (rows of a batch can be much shorter than the longest one)
+#pragma unroll
+          for (int j = j8; j < j8 + 8; ++j)
+            if (decltype(all)::value || (j >= j0 && j < j1)) f(j, reg[j]);
+        }
+      }
     } else {
-      for (int jb = j0; jb < j1; jb += 16) {
-        uint32_t uu[16];
+      for (int jb = j0; jb < j1; jb += kStream) {
+        uint32_t uu[kStream];
 #pragma unroll
-        for (int u = 0; u < 16; ++u) uu[u] = score_bits<T>(scores, tid, jb + u);
+        for (int u = 0; u < kStream; ++u) uu[u] = score_bits<T>(scores, tid, jb + u);
 #pragma unroll
-        for (int u = 0; u < 16; ++u)
+        for (int u = 0; u < kStream; ++u)
           if (jb + u < j1)
             f(jb + u, (jb + u) * kTopkThreads + tid < len ? to_d(uu[u]) : kNoElement);
       }
@@ -1157,6 +1168,12 @@ static void launch_topk_sliced(const TopkParams& p, int rows, hipStream_t st) {
     hipLaunchKernelGGL((topk_slice_kernel<T, 32>), grid, block, 0, st, p, n_slices, rps, rows);
   else if (p.len <= 40 * kTopkThreads)
     hipLaunchKernelGGL((topk_slice_kernel<T, 40>), grid, block, 0, st, p, n_slices, rps, rows);
+  else if (p.len <= 48 * kTopkThreads)
+    hipLaunchKernelGGL((topk_slice_kernel<T, 48>), grid, block, 0, st, p, n_slices, rps, rows);
+  else if (p.len <= 56 * kTopkThreads)
+    hipLaunchKernelGGL((topk_slice_kernel<T, 56>), grid, block, 0, st, p, n_slices, rps, rows);
+  else if (p.len <= 64 * kTopkThreads)
+    hipLaunchKernelGGL((topk_slice_kernel<T, 64>), grid, block, 0, st, p, n_slices, rps, rows);
   else  // longer rows would not fit the registers of a 1024-thread workgroup: re-read per pass
     hipLaunchKernelGGL((topk_slice_kernel<T, 0>), grid, block, 0, st, p, n_slices, rps, rows);
 }
@@ -1247,9 +1264,9 @@ extern "C" int td_topk(const void* values, int32_t values_dtype, int64_t values_
              "Top-k filtering failed to dispatch with dtype %d", values_dtype);
   // A few long rows: the three cooperative launches split each row over workgroups that share the
   // work through the scratch.  Everything else: one launch in which every workgroup of a row goes
-  // through the whole row (rows up to 40K elements from registers) and emits its slice.
+  // through the whole row (rows up to 64K elements from registers) and emits its slice.
   const int slices = coop_slices(len, rows);
-  if (len > 40 * kTopkThreads && slices && rows * slices <= 1024 && workspace &&
+  if (len > 64 * kTopkThreads && slices && rows * slices <= 1024 && workspace &&
       workspace_bytes >= (int64_t)rows * kCoopRowWords * 4) {
     uint32_t* ws = reinterpret_cast<uint32_t*>(workspace);
     const dim3 grid((rows + kXcds - 1) / kXcds * slices * kXcds), block(kTopkThreads);
