@@ -77,7 +77,6 @@ struct DecodeParams {
   float* ws_ml;     // [batch * H_q * max_splits, 2]
   int32_t* ws_cnt;  // [batch * head rows] ticket counters, ticket_stride words apart
   int32_t ticket_stride;
-  uint64_t* ws_st;  // [batch * H_q * max_splits, 130] stamped partials of the sparse-layer kernel
   // the token being decoded (FRESH kernels): un-rotated k, v, its rotary cos/sin and its slot
   const void* fresh_k;
   const void* fresh_v;

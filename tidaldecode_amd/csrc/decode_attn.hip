@@ -158,8 +158,8 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
   int nw = plan->waves_per_block;
   if (nw == 0) nw = 8;
   if (qpg > 1) nw = 8;  // the shared-row kernels exist for 8 waves only
-  // Short lists (sparse layers) are cut finer: 2 K/V rows per lane group and tile; long ones
-  // stream with 4.
+  // K/V rows per lane group and tile of the streaming kernel: 4 unless the caller presets 2
+  // (short token-slot lists have a kernel of their own, above).
   int rows = plan->tile_rows;
   if (rows == 0) rows = 4;
   if (!shape_supported(head_dim, qpg, nw, rows))
