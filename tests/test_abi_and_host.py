@@ -231,3 +231,31 @@ def test_batch_controller_bookkeeping():
     assert c.batch == 2 and c.pool.num_free_blocks == 30 - 7 - 8
     c.release()
     assert c.batch == 0 and c.pool.num_free_blocks == 30
+
+
+def test_split_partials_are_only_touched_through_the_coherent_accessors():
+    """The split merge is ordered by device-scope write-through stores, a wait, a ticket and
+    device-scope loads (the argument sits next to the code).  A plain load or store on the partial
+    arrays would break it without failing any small test, so every use of ws_o / ws_ml in the
+    kernels must go through store_coherent / load_coherent (or form the pointer those take)."""
+    import re
+    from pathlib import Path
+
+    csrc = Path(__file__).resolve().parents[1] / "tidaldecode_amd" / "csrc"
+    uses = 0
+    for path in sorted(csrc.glob("*.cuh")) + sorted(csrc.glob("*.hip")):
+        lines = path.read_text().splitlines()
+        for no, line in enumerate(lines, 1):
+            code = line.split("//")[0]
+            if not re.search(r"\bws_(o|ml)\b", code):
+                continue
+            uses += 1
+            ok = ("store_coherent(" in code or "load_coherent(" in code
+                  or re.search(r"float\* ws_(o|ml);", code)                       # the field
+                  or re.search(r"p\.ws_(o|ml) = reinterpret_cast<float\*>", code)  # host: carve the workspace
+                  or re.search(r"float\* dst = p\.ws_o \+", code))               # pointer handed to store_coherent
+            assert ok, f"{path.name}:{no}: {line.strip()}"
+            if "float* dst = p.ws_o +" in code:
+                following = " ".join(lines[no: no + 4])
+                assert following.count("store_coherent(dst") == 4, f"{path.name}:{no}"
+    assert uses >= 10

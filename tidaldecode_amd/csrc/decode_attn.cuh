@@ -818,7 +818,17 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
   if (n_splits == 1 || !p.fused_merge) return;
 
   // ---- the last workgroup of this (sequence, head row) to arrive reduces the partials ----------
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // partial stores have left this CU
+  // Ordering.  The partials were stored with device-scope write-through stores (store_coherent,
+  // sc1): such a store is acknowledged -- vmcnt decremented -- only once it has reached memory, the
+  // point where all XCDs meet.  Every wave waits for its own stores, the barrier collects the
+  // waves, and only then does one thread take the ticket, a device-scope atomic performed at
+  // memory.  The workgroup that draws the last ticket therefore knows that every other partial of
+  // the head row was acknowledged before its writer's ticket was issued, and it reads them with
+  // device-scope loads (load_coherent, sc1) that a cache level private to one XCD cannot serve
+  // from a stale line.  What would break this: a plain store or load on ws_o / ws_ml (a test greps
+  // for that), the compiler moving the ticket above the wait (hence asm volatile with a memory
+  // clobber), or dropping the barrier between the waves' waits and the ticket.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   int32_t* ticket = p.ws_cnt + ((int64_t)b * gridDim.x + hrow) * p.ticket_stride;
   if (tid == 0)
