@@ -1,7 +1,5 @@
 """Shared builders for the parity tests: seeded K/V, paged pools with shuffled pages, tolerances."""
-import math
 
-import numpy as np
 import torch
 
 # max-abs tolerances of the attention output against the fp32 oracle on identically rounded inputs

@@ -5,7 +5,6 @@ identically rounded inputs.  The parameter grid follows the reference's own deco
 (kernels/src/test/test_batch_decode.cu:215-267: sequence lengths, page sizes, page budgets, head
 dims; per-head page lists drawn from a shuffled iota with the forced last page, :57-76).
 """
-import math
 
 import numpy as np
 import pytest

@@ -10,7 +10,7 @@ import math
 import pytest
 import torch
 
-from _util import ATOL, PagedCase, randn, tolerance_report
+from _util import ATOL, PagedCase, randn
 
 pytestmark = pytest.mark.gpu
 

@@ -11,7 +11,6 @@ the layer schedule of the PyTorch path of the reference (src/tidal_build/modify_
     layer == sparse_layer_start or correction_layer  full attention + token selection
     otherwise                                         sparse attention over the persisted tokens
 """
-import math
 import time
 from dataclasses import dataclass
 from typing import Optional, Tuple
