@@ -68,13 +68,16 @@ typedef struct {
 /*
  * Per-call description of which tokens each sequence attends to.
  *
- * idx is a 2-D int32 array with `idx_rows` rows of `idx_row_stride` elements.  Sequence b uses
+ * idx is a 2-D int32 array with `idx_rows` rows of `idx_row_stride` elements (a single row:
+ * the number of elements it holds, or 0 if unknown).  Sequence b uses
  * columns [indptr[b], indptr[b+1]) of every row (indptr lives on the device; if indptr is NULL
  * the call is for one sequence that uses columns [0, n_list_host)).  With count_arr (device,
  * [batch]) sequence b uses count_arr[b] columns starting at indptr[b] instead: the rows of a
  * padded table, one fixed-width segment per sequence, which can grow in place.  Row r belongs to query
  * head r (idx_rows == num_qo_heads), to KV head r (idx_rows == num_kv_heads) or to everybody
- * (idx_rows == 1).
+ * (idx_rows == 1).  The kernels read no column of a row outside the sequence's segment
+ * [indptr[b], indptr[b+1]), beyond n_list_host columns from its start, or at idx_row_stride and
+ * beyond; a device-resident count that says otherwise is cut to that.
  *
  * After the listed entries every sequence may attend to one more, partially filled page: the
  * first last_page_len entries of page last_page_idx ("forced last page",

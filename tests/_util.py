@@ -64,5 +64,23 @@ class PagedCase:
         return self.page_table[positions // self.page_size] * self.page_size + positions % self.page_size
 
 
+def rotated(x: torch.Tensor, positions, dtype: torch.dtype, theta: float) -> torch.Tensor:
+    """x [N, H, D] fp32 rotated at `positions` by the oracle's float64 closed form, rounded to
+    `dtype`: what a fused decode step holds in registers (q) or writes to the cache (k)."""
+    import numpy as np
+
+    from oracle import tidal_oracle as orc
+
+    y = orc.rope_closed_form(x.numpy(), np.asarray(positions), theta)
+    return rounded(torch.from_numpy(y).float(), dtype)
+
+
+def within_ulps(got: torch.Tensor, want: torch.Tensor, dtype: torch.dtype, ulps: float = 1.0) -> bool:
+    """|got - want| <= ulps units in the last place of `dtype` at want's magnitude"""
+    ulp = {torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}[dtype]
+    want = want.float().cpu()
+    return bool(((got.float().cpu() - want).abs() <= ulps * ulp * want.abs() + 1e-6).all())
+
+
 def tolerance_report(got: torch.Tensor, want: torch.Tensor) -> float:
     return (got.float().cpu() - want.float().cpu()).abs().max().item()

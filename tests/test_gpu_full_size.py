@@ -8,13 +8,15 @@ selection and one sparse layer through the operator surface, against the CPU ora
 The oracle's sparse layer gathers the selected rows (equal to the reference's masked dense form,
 pinned in tests/test_oracle.py), so it finishes in seconds at these sizes.  Index sets are
 compared bit-exact from the scores the GPU wrote; attention within 2e-3 (fp16) / 1e-2 (bf16).
-Size-independent properties on top: a permuted list gives the same output, and a list naming
-every token equals full attention.
+The sparse layer runs twice: as a plain attention launch, and as the fused decode step the
+benchmark times (RoPE of q and the new key, cache write and attention in one launch) against the
+oracle on float64-rotated, storage-rounded q and K.  Size-independent properties on top: a
+permuted list gives the same output, and a list naming every token equals full attention.
 """
 import pytest
 import torch
 
-from _util import ATOL, PagedCase, randn, tolerance_report
+from _util import ATOL, PagedCase, randn, rotated, tolerance_report, within_ulps
 
 pytestmark = pytest.mark.gpu
 
@@ -70,6 +72,42 @@ def test_selection_topk_sparse_at_full_size(cuda, name, hq, hkv, n, k, mode, dty
     # sparse layer
     want = orc.sparse_layer_gather(q_sp, case.k, case.v, pos_c)
     assert tolerance_report(o_sp[0], want) <= ATOL[dtype]
+
+    # The decode step as the benchmark times it: RoPE of q and of the new key, the cache write and
+    # the attention in ONE launch (fresh=...).  The newest token plays the token being decoded: its
+    # slot is in the lists of the even rows (taken from registers there) and in none of the odd ones.
+    theta = 5e5 if hkv != hq else 1e4
+    new_pos = n - 1
+    pos_f = pos_c.clone()
+    for r in range(rows):
+        hit = (pos_f[r] == new_pos).nonzero().flatten()
+        if r % 2 == 0 and hit.numel() == 0:
+            pos_f[r, -1] = new_pos                       # lists stay sorted: it is the last position
+        elif r % 2 == 1 and hit.numel():
+            listed = set(pos_f[r].tolist())
+            unused = next(x for x in range(n - 1) if x not in listed)
+            pos_f[r, hit[0]] = unused
+    k_new, v_new = randn((1, hkv, d), 21, dtype), randn((1, hkv, d), 22, dtype)
+    k_f, v_f = case.k.clone(), case.v.clone()
+    k_f[new_pos] = rotated(k_new, [new_pos], dtype, theta)[0]
+    v_f[new_pos] = v_new[0]
+    want_f = orc.sparse_layer_gather(rotated(q_sp[None], [new_pos], dtype, theta)[0], k_f, v_f, pos_f)
+    assert w._plan(1, rows, k).sparse_waves > 0          # the short-list kernel, as in the benchmark
+    pool_f = pool.clone()
+    dst = case.slots_of(torch.tensor([new_pos])).to(torch.int32).to(cuda)
+    cos, sin = _kernels.rope_table(torch.tensor([new_pos], dtype=torch.int32, device=cuda), d, 1.0, theta)
+    o_f = torch.empty((1, hq, d), dtype=dtype, device=cuda)
+    w.forward(q_sp.to(dtype).to(cuda)[None], o_f, pool_f, case.slots_of(pos_f).to(torch.int32).to(cuda),
+              None, 0, 0, None, index_kind="slots",
+              fresh=(k_new.to(dtype).to(cuda), v_new.to(dtype).to(cuda), cos, sin, dst))
+    torch.cuda.synchronize()
+    assert tolerance_report(o_f[0], want_f) <= ATOL[dtype]
+    page_f, entry_f = int(dst[0]) // page, int(dst[0]) % page
+    assert within_ulps(pool_f[page_f, 0, entry_f], k_f[new_pos], dtype)     # rotated key, one rounding
+    assert torch.equal(pool_f[page_f, 1, entry_f].cpu(), v_new[0].to(dtype))
+    pool_f[page_f, :, entry_f] = pool[page_f, :, entry_f]
+    assert torch.equal(pool_f, pool)                                        # nothing else was written
+    del pool_f
 
     # a permuted list names the same set: same output up to the summation order
     g = torch.Generator().manual_seed(1)

@@ -1,10 +1,12 @@
-"""GPU: the fused decode step (fresh=...) against the three separate calls it replaces
-(RoPE in place, append, attention): same attention output within the attention tolerance, same
-cache contents up to one rounding of the rotated key, logits of the new token included."""
+"""GPU: the fused decode step (fresh=...) against the CPU oracle on float64-rotated,
+storage-rounded q and K, and against the three separate calls it replaces (RoPE in place, append,
+attention): same attention output far inside the attention tolerance (the two GPU paths share
+every rounding but the rotated key's), same cache contents up to one rounding of the rotated key,
+logits of the new token included."""
 import pytest
 import torch
 
-from _util import ATOL, PagedCase, randn
+from _util import ATOL, PagedCase, randn, rotated, tolerance_report, within_ulps
 
 pytestmark = pytest.mark.gpu
 
@@ -24,6 +26,7 @@ def _ulp_close(a, b, dtype):
                                               # 12 heads per KV head: two head rows (8 + 4) per KV head
                                               (24, 2, 2, "slots"), (24, 2, 1, "pages")])
 def test_fused_equals_separate(cuda, dtype, hq, hkv, rows, mode):
+    from oracle import tidal_oracle as orc
     from tidaldecode_amd import _kernels
 
     d, page, n, k, b = 128, 16, 1000, 96, 2   # n counts the new token
@@ -41,18 +44,21 @@ def test_fused_equals_separate(cuda, dtype, hq, hkv, rows, mode):
     last_idx = torch.tensor([offs[i] + npg - 1 for i in range(b)], dtype=torch.int32, device=cuda)
     dst = (last_idx * page + last_len - 1).to(torch.int32)
     g = torch.Generator().manual_seed(5)
+    attended = []         # per sequence: the positions each list row attends to
     if mode == "pages":   # selection layer: every page in order + last page
         idx = torch.cat([torch.arange(npg - 1) + offs[i] for i in range(b)]).to(torch.int32)[None]
         indptr = torch.tensor([0, npg - 1, 2 * (npg - 1)], dtype=torch.int32, device=cuda)
         ll = torch.full((b,), last_len, dtype=torch.int32, device=cuda)
         li = last_idx
         n_list = npg - 1
+        attended = [torch.arange(n)[None] for _ in range(b)]
     else:                 # sparse layer: k slots per row, the new token's slot among them
         lists = []
         for i in range(b):
             pos = torch.stack([torch.randperm(n - 1, generator=g)[: k - 1] for _ in range(rows)])
             pos = torch.cat([pos, torch.full((rows, 1), n - 1)], 1)[:, torch.randperm(k, generator=g)]
             lists.append(pos + offs[i] * page)
+            attended.append(pos)
         idx = torch.cat(lists, 1).to(torch.int32)
         indptr = torch.tensor([0, k, 2 * k], dtype=torch.int32, device=cuda)
         ll = torch.zeros(b, dtype=torch.int32, device=cuda)
@@ -82,7 +88,26 @@ def test_fused_equals_separate(cuda, dtype, hq, hkv, rows, mode):
 
     o1, p1, s1 = run(False)
     o2, p2, s2 = run(True)
-    assert (o1.float() - o2.float()).abs().max().item() <= ATOL[dtype]
+    q_cpu, knew_cpu, vnew_cpu = q.float().cpu(), knew.float().cpu(), vnew.float().cpu()
+    for i in range(b):
+        p_i = [int(positions[i])]
+        kk, vv = cases[i].k.clone(), cases[i].v.clone()
+        kk[n - 1] = rotated(knew_cpu[i:i + 1], p_i, dtype, theta)[0]
+        vv[n - 1] = vnew_cpu[i]
+        q_rot = rotated(q_cpu[i:i + 1], p_i, dtype, theta)[0]
+        want = orc.sparse_layer_gather(q_rot, kk, vv, attended[i])
+        assert tolerance_report(o2[i], want) <= ATOL[dtype], i
+        page_i, entry_i = int(dst[i]) // page, int(dst[i]) % page
+        assert within_ulps(p2[page_i, 0, entry_i], kk[n - 1], dtype), i
+        assert torch.equal(p2[page_i, 1, entry_i], vnew[i]), i
+        if s2 is not None:
+            logits = orc.attn_logits(q_rot, kk)
+            # a rotated q element that lands on the other side of a rounding boundary than the
+            # float64 rotation moves a head's logits by up to one storage ulp of q times |k| / sqrt(d)
+            ulp = {torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}[dtype]
+            bound = 2e-4 * max(1.0, logits.abs().max().item()) + 0.5 * ulp
+            assert (s2[i * hq:(i + 1) * hq, :n].cpu() - logits).abs().max() <= bound, i
+    assert (o1.float() - o2.float()).abs().max().item() <= ATOL[dtype] / 4
     assert _ulp_close(p2, p1, dtype)                         # the cache got the new token
     changed = (p1 != pool).any(dim=(1, 2, 3, 4)).nonzero().flatten().tolist()
     assert changed == sorted(set(last_idx.tolist()))         # ... and nothing else

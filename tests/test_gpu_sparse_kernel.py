@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 import torch
 
-from _util import ATOL, PagedCase, randn, tolerance_report
+from _util import ATOL, PagedCase, randn, rotated, tolerance_report, within_ulps
 
 pytestmark = pytest.mark.gpu
 
@@ -180,12 +180,17 @@ def test_ragged_batch_with_lengths_on_the_device(cuda, counts_kind):
 def test_fused_decode_step(cuda, dtype, sw, sr):
     """RoPE + append inside the launch: the new token's slot sits somewhere in every list (so some
     wave of every head takes it from registers), the cache gets the rotated key exactly once, and
-    the output equals separate RoPE/append launches followed by the same attention."""
+    the output equals the oracle's attention over float64-rotated, storage-rounded q and K as
+    well as separate RoPE/append launches followed by the same attention (the two GPU paths share
+    every rounding but that of the rotated key).  The last case is the benchmark's head row:
+    32 heads x 2048 tokens."""
+    from oracle import tidal_oracle as orc
     from tidaldecode_amd import _kernels
 
-    h, d, page, n, b = 8, 128, 16, 1500, 2
+    d, page, n, b = 128, 16, 1500, 2
     theta = 1e4
-    for k in (1, 4 * sr + 1, 700):
+    for h, k in ((8, 1), (8, 4 * sr + 1), (8, 700), (32, 2048)):
+        n = 1500 if k < 1000 else 5000
         cases = [PagedCase(n, h, d, page, dtype, seed=40 + i, spare=0, shuffle=False) for i in range(b)]
         npg = cases[0].n_pages
         pool = torch.cat([c.pool for c in cases]).to(cuda)
@@ -198,11 +203,18 @@ def test_fused_decode_step(cuda, dtype, sw, sr):
         last_idx = torch.tensor([offs[i] + npg - 1 for i in range(b)], dtype=torch.int32, device=cuda)
         dst = (last_idx * page + last_len - 1).to(torch.int32)
         g = torch.Generator().manual_seed(5 + k)
-        lists = []
+        lists, wants, k_rot = [], [], []
+        q_cpu, knew_cpu, vnew_cpu = q.float().cpu(), knew.float().cpu(), vnew.float().cpu()
         for i in range(b):
             pos = torch.stack([torch.randperm(n - 1, generator=g)[: k - 1] for _ in range(h)])
             pos = torch.cat([pos, torch.full((h, 1), n - 1)], 1)[:, torch.randperm(k, generator=g)]
             lists.append(pos + offs[i] * page)
+            p_i = [int(positions[i])]
+            kk, vv = cases[i].k.clone(), cases[i].v.clone()
+            kk[n - 1] = rotated(knew_cpu[i:i + 1], p_i, dtype, theta)[0]
+            vv[n - 1] = vnew_cpu[i]
+            k_rot.append(kk[n - 1])
+            wants.append(orc.sparse_layer_gather(rotated(q_cpu[i:i + 1], p_i, dtype, theta)[0], kk, vv, pos))
         idx = torch.cat(lists, 1).to(torch.int32).to(cuda).contiguous()
         indptr = torch.tensor([0, k, 2 * k], dtype=torch.int32, device=cuda)
         zeros = torch.zeros(b, dtype=torch.int32, device=cuda)
@@ -224,7 +236,13 @@ def test_fused_decode_step(cuda, dtype, sw, sr):
 
         o1, p1 = run(False)
         o2, p2 = run(True)
-        assert (o1.float() - o2.float()).abs().max().item() <= ATOL[dtype], k
+        for i in range(b):
+            assert tolerance_report(o2[i], wants[i]) <= ATOL[dtype], (h, k, i)
+            assert tolerance_report(o1[i], wants[i]) <= ATOL[dtype], (h, k, i)
+            page_i, entry_i = int(dst[i]) // page, int(dst[i]) % page
+            assert within_ulps(p2[page_i, 0, entry_i], k_rot[i], dtype), (h, k, i)
+            assert torch.equal(p2[page_i, 1, entry_i], vnew[i]), (h, k, i)
+        assert (o1.float() - o2.float()).abs().max().item() <= ATOL[dtype] / 4, (h, k)
         ulp = {torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}[dtype]
         assert ((p2.float() - p1.float()).abs() <= ulp * p1.float().abs() + 1e-6).all()
         changed = (p1 != pool).any(dim=(1, 2, 3, 4)).nonzero().flatten().tolist()
@@ -334,6 +352,9 @@ def test_shared_kv_rows(cuda, dtype, hq, hkv, rows, sw):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("hq,hkv", [(8, 4), (16, 4), (32, 4)])
 def test_fused_decode_step_with_shared_kv_rows(cuda, dtype, hq, hkv):
+    """The fused decode step on the shared-row kernels, against the oracle on float64-rotated,
+    storage-rounded q and K and against the separate launches."""
+    from oracle import tidal_oracle as orc
     from tidaldecode_amd import _kernels
 
     d, page, n, b = 128, 16, 1500, 2
@@ -350,11 +371,18 @@ def test_fused_decode_step_with_shared_kv_rows(cuda, dtype, hq, hkv):
         last_idx = torch.tensor([offs[i] + npg - 1 for i in range(b)], dtype=torch.int32, device=cuda)
         dst = (last_idx * page + last_len - 1).to(torch.int32)
         g = torch.Generator().manual_seed(5 + k)
-        lists = []
+        lists, wants, k_rot = [], [], []
+        q_cpu, knew_cpu, vnew_cpu = q.float().cpu(), knew.float().cpu(), vnew.float().cpu()
         for i in range(b):
             pos = torch.stack([torch.randperm(n - 1, generator=g)[: k - 1] for _ in range(hkv)])
             pos = torch.cat([pos, torch.full((hkv, 1), n - 1)], 1)[:, torch.randperm(k, generator=g)]
             lists.append(pos + offs[i] * page)
+            p_i = [int(positions[i])]
+            kk, vv = cases[i].k.clone(), cases[i].v.clone()
+            kk[n - 1] = rotated(knew_cpu[i:i + 1], p_i, dtype, 5e5)[0]
+            vv[n - 1] = vnew_cpu[i]
+            k_rot.append(kk[n - 1])
+            wants.append(orc.sparse_layer_gather(rotated(q_cpu[i:i + 1], p_i, dtype, 5e5)[0], kk, vv, pos))
         idx = torch.cat(lists, 1).to(torch.int32).to(cuda).contiguous()
         indptr = torch.tensor([0, k, 2 * k], dtype=torch.int32, device=cuda)
         zeros = torch.zeros(b, dtype=torch.int32, device=cuda)
@@ -376,7 +404,12 @@ def test_fused_decode_step_with_shared_kv_rows(cuda, dtype, hq, hkv):
 
         o1, p1 = run(False)
         o2, p2 = run(True)
-        assert (o1.float() - o2.float()).abs().max().item() <= ATOL[dtype], k
+        for i in range(b):
+            assert tolerance_report(o2[i], wants[i]) <= ATOL[dtype], (k, i)
+            page_i, entry_i = int(dst[i]) // page, int(dst[i]) % page
+            assert within_ulps(p2[page_i, 0, entry_i], k_rot[i], dtype), (k, i)
+            assert torch.equal(p2[page_i, 1, entry_i], vnew[i]), (k, i)
+        assert (o1.float() - o2.float()).abs().max().item() <= ATOL[dtype] / 4, k
         ulp = {torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}[dtype]
         assert ((p2.float() - p1.float()).abs() <= ulp * p1.float().abs() + 1e-6).all()
         changed = (p1 != pool).any(dim=(1, 2, 3, 4)).nonzero().flatten().tolist()

@@ -87,6 +87,18 @@ def test_ties_go_to_the_lower_position(cuda):
     assert torch.equal(got, torch.arange(777, dtype=torch.int32).repeat(4, 1))
 
 
+@pytest.mark.parametrize("n,k", [(64, 5), (1500, 1500), (32768, 2048), (40000, 1), (65536, 4096)])
+def test_rows_of_one_value(cuda, n, k):
+    """Every score of a row equal (zeros, a NaN row, -inf, a denormal): the selection has nothing to
+    rank and goes from the extremes of the row straight to the emission; the first k positions."""
+    first_k = torch.arange(k, dtype=torch.int32)
+    for value in (0.0, -0.0, float("nan"), float("-inf"), float("inf"), 1e-42, -7.25):
+        rows = torch.full((3, n), value)
+        rows[1, 1::2] = -value if value == 0.0 else value      # +0 and -0 are one value
+        got = _check(rows, k, cuda)
+        assert torch.equal(got, first_k.repeat(3, 1)), value
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 def test_long_rows_with_crowded_threshold_bins(cuda, dtype):
     """Rows whose keys share their leading bits (more candidates than the cooperative kernel keeps

@@ -575,7 +575,8 @@ class BatchDecodeWithPagedKVCachePyTorchWrapper:
         lst = IndexList()
         lst.idx = _ptr(paged_kv_indices)
         lst.idx_rows = rows
-        lst.idx_row_stride = paged_kv_indices.stride(0)
+        # what a row holds bounds the kernels' reads; a single row has no meaningful stride
+        lst.idx_row_stride = paged_kv_indices.stride(0) if rows > 1 else budget
         lst.kind = kind
         if paged_kv_indptr is not None:
             _check_i32(paged_kv_indptr, "paged_kv_indptr")
@@ -670,7 +671,7 @@ def gather_probe(wrapper: "BatchDecodeWithPagedKVCachePyTorchWrapper", paged_kv_
     lst = IndexList()
     lst.idx = _ptr(slots)
     lst.idx_rows = rows
-    lst.idx_row_stride = slots.stride(0)
+    lst.idx_row_stride = slots.stride(0) if slots.size(0) > 1 else slots.size(1)
     lst.kind = TD_IDX_SLOTS
     lst.n_list_host = budget
     plan = wrapper._plan(1, rows, budget)

@@ -53,6 +53,7 @@ struct DecodeParams {
   // index list
   const int32_t* idx;
   int32_t idx_row_stride;  // 0 for a shared row
+  int32_t idx_cols;        // elements a row holds (the caller's row stride; 0: unknown): reads stop there
   int32_t idx_per_kv;      // 1: rows are per KV head while QPG == 1
   const int32_t* indptr;
   const int32_t* count_arr;  // per-sequence entry counts of a padded table (else indptr differences)
@@ -223,15 +224,29 @@ __device__ __forceinline__ void head_row_geom(const DecodeParams& p, int hrow, i
   }
 }
 
+// Columns of a sequence's list segment that a kernel may read: the host's bound, cut to the segment
+// [list_beg, list_end) when the call has an indptr and to what is left of the row (row_cols columns;
+// 0: a row of unknown length).  Device-resident counts are clamped to it.
+__device__ __forceinline__ int list_capacity(int n_list_host, bool has_indptr, int list_beg,
+                                             int list_end, int row_cols) {
+  int cap = n_list_host;
+  if (has_indptr) cap = list_end - list_beg < cap ? list_end - list_beg : cap;
+  if (row_cols > 0) cap = row_cols - list_beg < cap ? row_cols - list_beg : cap;
+  return cap < 0 ? 0 : cap;
+}
+
 __device__ __forceinline__ int seq_items(const DecodeParams& p, int b, SeqList& s, int& list_beg) {
   list_beg = 0;
+  int list_end = 0;
   if (p.indptr) {
     list_beg = p.indptr[b];
-    s.n_list = p.count_arr ? p.count_arr[b] : p.indptr[b + 1] - list_beg;
+    list_end = p.indptr[b + 1];
+    s.n_list = p.count_arr ? p.count_arr[b] : list_end - list_beg;
   } else {
     s.n_list = p.n_list_host;
   }
-  s.n_list = s.n_list < 0 ? 0 : (s.n_list > p.n_list_host ? p.n_list_host : s.n_list);
+  const int cap = list_capacity(p.n_list_host, p.indptr != nullptr, list_beg, list_end, p.idx_cols);
+  s.n_list = s.n_list < 0 ? 0 : (s.n_list > cap ? cap : s.n_list);
   s.last_len = p.last_len_arr ? p.last_len_arr[b] : p.last_len;
   s.last_idx = p.last_idx_arr ? p.last_idx_arr[b] : p.last_idx;
   // device-resident lengths are not trusted: a fill beyond the page, or more splits than the

@@ -330,6 +330,7 @@ static int build_params(const td_paged_kv* kv, const td_index_list* list, const 
   p.q_per_kv = num_qo_heads / Hkv;
   p.idx = list->idx;
   p.idx_row_stride = list->idx_rows == 1 ? 0 : list->idx_row_stride;
+  p.idx_cols = list->idx_row_stride > 0 ? list->idx_row_stride : 0;
   p.idx_per_kv = (qpg == 1 && list->idx_rows == Hkv && Hkv != num_qo_heads) ? 1 : 0;
   p.page_mode = list->kind == TD_IDX_PAGES ? 1 : 0;
   p.max_page = (uint32_t)(kv->max_pages - 1);

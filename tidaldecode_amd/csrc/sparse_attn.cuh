@@ -228,7 +228,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
 #define TD_TOUCH(x) asm volatile("" ::"s"(x))
   TD_TOUCH(p.q); TD_TOUCH(p.kv); TD_TOUCH(p.v_offset); TD_TOUCH(p.idx); TD_TOUCH(p.indptr);
   TD_TOUCH(p.count_arr); TD_TOUCH(p.last_len_arr); TD_TOUCH(p.last_idx_arr);
-  TD_TOUCH(p.idx_row_stride); TD_TOUCH(p.n_list_host); TD_TOUCH(p.qpk_shift);
+  TD_TOUCH(p.idx_row_stride); TD_TOUCH(p.idx_cols); TD_TOUCH(p.n_list_host); TD_TOUCH(p.qpk_shift);
   TD_TOUCH(p.chunk_shift); TD_TOUCH(p.max_splits); TD_TOUCH(p.page_shift); TD_TOUCH(p.max_slot);
   TD_TOUCH(p.page_stride_b); TD_TOUCH(p.entry_stride_b); TD_TOUCH(p.head_stride);
   TD_TOUCH(p.last_len); TD_TOUCH(p.last_idx); TD_TOUCH(p.scale_log2); TD_TOUCH(p.num_qo_heads);
@@ -243,19 +243,21 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
   const int own = g * U + (li & (U - 1));  // the token of the tile this lane owns
 
   // ---- everything that depends on the kernel arguments only is requested at once ---------------
-  // The list entries of the first tile are read before the length of the list is known: the
-  // position is clamped to the row's capacity (n_list_host), which the host has checked against
-  // the row stride.
+  // The list entries of the first tile are read before the length of the list is known.  The
+  // position is clamped to what the sequence's segment of the row is known to hold whatever the
+  // device-resident count says: at most n_list_host columns (which the host has checked against
+  // the row stride for a segment that starts at column 0), no further than the segment's end
+  // indptr[b + 1], and never beyond the row itself.
   const int t0 = (split * NW + wave) * TILE;
   const int idx_row = (QPG > 1 || p.idx_per_kv) ? kv_head : hrow;
   int list_beg = 0, list_end = 0;
   if (p.indptr) scalar_load2(p.indptr + b, p.indptr + b + 1, list_beg, list_end);
   const int32_t* row = p.idx + (int64_t)idx_row * p.idx_row_stride + list_beg;
-  const bool has_cap = p.n_list_host > 0;
+  const int cap = list_capacity(p.n_list_host, p.indptr != nullptr, list_beg, list_end, p.idx_cols);
   auto fetch_entry = [&](int t) -> int32_t {
     int pos = t + own;
-    pos = pos < p.n_list_host ? pos : p.n_list_host - 1;
-    return has_cap ? row[pos] : 0;
+    pos = pos < cap ? pos : cap - 1;
+    return cap > 0 ? row[pos] : 0;
   };
   int32_t ent = fetch_entry(t0);
 
@@ -267,15 +269,6 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
     qp[j][0] = v.x; qp[j][1] = v.y; qp[j][2] = v.z; qp[j][3] = v.w;
   }
   uint32_t knew[4] = {0, 0, 0, 0}, vnew[4] = {0, 0, 0, 0};
-  // slot of the token being decoded: requested now, waited for after the K/V rows are on their way
-  // (only the comparison with the list needs it)
-  int32_t new_slot_raw = -1;
-  if constexpr (FRESH)
-    asm volatile("s_load_dword %0, %1, 0x0" : "=s"(new_slot_raw) : "s"(p.fresh_slot + b) : "memory");
-  auto new_slot_wait = [&]() -> uint32_t {
-    if constexpr (FRESH) asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(new_slot_raw)::"memory");
-    return (uint32_t)new_slot_raw;
-  };
   float rcs[8], rsn[8];
   if constexpr (FRESH) {
     constexpr int HALF = LPR / 2;
@@ -301,19 +294,26 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
   s.n_list = p.n_list_host;
   s.last_len = p.last_len;
   s.last_idx = p.last_idx;
-  if (p.count_arr || p.last_len_arr || p.last_idx_arr) {
+  // slot of the token being decoded (FRESH): it travels with the other state words, load and wait
+  // inside one asm statement, so that no register allocation can read it before it has landed; the
+  // list entry, which the row loads wait for anyway, is in flight over the same round trip
+  uint32_t new_slot = 0xffffffffu;
+  if (FRESH || p.count_arr || p.last_len_arr || p.last_idx_arr) {
     // absent arrays read a dummy word (q is never NULL) and keep the host value
     const int32_t* dummy = reinterpret_cast<const int32_t*>(p.q);
-    int32_t cnt, ll, lx, unused;
+    int32_t cnt, ll, lx, ns;
     scalar_load4(p.count_arr ? p.count_arr + b : dummy, p.last_len_arr ? p.last_len_arr + b : dummy,
-                 p.last_idx_arr ? p.last_idx_arr + b : dummy, dummy, cnt, ll, lx, unused);
+                 p.last_idx_arr ? p.last_idx_arr + b : dummy, FRESH ? p.fresh_slot + b : dummy, cnt, ll,
+                 lx, ns);
     if (p.indptr) s.n_list = p.count_arr ? cnt : list_end - list_beg;
     if (p.last_len_arr) s.last_len = ll;
     if (p.last_idx_arr) s.last_idx = lx;
+    if constexpr (FRESH) new_slot = (uint32_t)ns;
   } else if (p.indptr) {
     s.n_list = list_end - list_beg;
   }
-  s.n_list = s.n_list < 0 ? 0 : (s.n_list > p.n_list_host ? p.n_list_host : s.n_list);
+  // a count beyond what the first fetch was clamped to would pair tokens with the wrong entries
+  s.n_list = s.n_list < 0 ? 0 : (s.n_list > cap ? cap : s.n_list);
   s.last_len = s.last_len < 0 ? 0 : (s.last_len > p.page_size ? p.page_size : s.last_len);
   const int c1 = s.n_list + s.last_len;
   int n_splits = (c1 + p.chunk_tokens - 1) >> p.chunk_shift;
@@ -368,7 +368,6 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
       k_rot = true;
     }
     if (writer && !wrote) {
-      const uint32_t new_slot = new_slot_wait();  // outside the lane branch: the wait is wave-wide
       if (g == 0) {
         const uint32_t ns = new_slot > p.max_slot ? p.max_slot : new_slot;
         char* dst = reinterpret_cast<char*>(const_cast<void*>(p.kv)) +
@@ -423,7 +422,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
     }
     bool hit = false;
     if constexpr (FRESH) {
-      hit = slot == new_slot_wait();
+      hit = slot == new_slot;
       const uint32_t hit_first = __builtin_amdgcn_readfirstlane(hit ? 1u : 0u);
       hit = valid ? hit : (hit_first != 0);
     }

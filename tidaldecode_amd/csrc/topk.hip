@@ -1047,6 +1047,9 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(const TopkPara
     bgt += (uint32_t)__popcll(__ballot(d < thr));
     beq += (uint32_t)__popcll(__ballot(d == thr));
   });
+  // wa / wb still hold the waves' extremes from step 1: a row of one value (dmax == 0) comes here
+  // without passing another barrier, and a slow wave may not have read them yet
+  __syncthreads();
   if (lane == 0) {
     L.wa[wave] = bgt;
     L.wb[wave] = beq;
