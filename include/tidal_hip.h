@@ -112,10 +112,11 @@ typedef struct {
   int32_t tile_rows;       /* K/V load instructions per wave tile: 2 or 4 */
   int32_t fused_merge;     /* 1: last workgroup merges in-kernel; 0: second kernel */
   /* Shape of the short-list kernel that serves calls with token-slot lists, head_dim 128, one
-   * list row per query head (or one shared row without grouped queries), power-of-two pages, a
-   * pool below 4 GiB and no score output: waves per workgroup (4 or 8) x K rows per lane (8 or
-   * 16).  0 on input: the planner decides; -1 on input: never use that kernel.  On output 0
-   * means the streaming kernel (waves_per_block x tile_rows) serves every call of this plan. */
+   * list row per query head (or one shared row without grouped queries) and no score output:
+   * waves per workgroup (4 or 8) x K rows per lane (8 or 16; pools of 4 GiB and more and pages
+   * that are not a power of two: 8).  0 on input: the planner decides; -1 on input: never use
+   * that kernel.  On output 0 means the streaming kernel (waves_per_block x tile_rows) serves
+   * every call of this plan. */
   int32_t sparse_waves;
   int32_t sparse_rows;
   int64_t workspace_bytes; /* device scratch the call needs (partials + tickets) */
@@ -209,8 +210,9 @@ int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t num_kv_head
  *              writes it and fresh->v into the cache at fresh->dst_slot, and attends to that
  *              token wherever the list names its slot -- one launch instead of
  *              td_rope_append_decode + td_decode_attn (tidal/models/SearchAttention.py:131-176 runs
- *              three).  Needs a power-of-two page_size and a pool below 4 GiB
- *              (TD_ERR_UNSUPPORTED otherwise).
+ *              three).  Calls served by the streaming kernel (page lists, score output, lists of
+ *              more than 16384 entries, head_dim 64 / 256) need a power-of-two page_size and a
+ *              pool below 4 GiB for it (TD_ERR_UNSUPPORTED otherwise).
  *   workspace  device scratch of at least plan->workspace_bytes whose first 1 MiB (ticket
  *              counters, 64 bytes apart) was zero-filled once before first use; every call
  *              leaves them zero again, so one workspace serves plans of any shape.  Calls that
@@ -225,6 +227,17 @@ int td_decode_attn(const td_paged_kv* kv, const td_index_list* list, const td_de
                    void* scores, int32_t scores_dtype, int64_t score_stride, float* lse,
                    const td_fresh_token* fresh, void* workspace, int64_t workspace_bytes,
                    void* stream);
+
+/*
+ * Which kernel family served the calling thread's last successful td_decode_attn call:
+ * "short-list" (the sparse layer's kernel: token-slot lists of up to 16384 entries, head_dim 128, no
+ * score output), "streaming" (everything else), each with ", 64-bit offsets" for pools of 4 GiB and
+ * more or pages that are not a power of two; "none" before the first call.  No counterpart in the
+ * reference (one kernel there, dispatched by SWITCH_HEAD_DIM,
+ * kernels/include/decode/decode_attn.cuh:1150-1154); tests and benchmarks use it to say which code
+ * they measured.
+ */
+const char* td_last_decode_kernel(void);
 
 /*
  * td_decode_attn for callers that cannot allocate device memory or be handed a workspace -- code

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 import torch
 
-from _util import ATOL, randn, tolerance_report
+from _util import ATOL, randn, rotated, tolerance_report, within_ulps
 
 pytestmark = pytest.mark.gpu
 
@@ -65,7 +65,11 @@ def test_decode_attention_beyond_4gib(cuda, dtype, hq, hkv, pool_pages):
     w = _wrapper(hq, hkv, d, page, dtype)
     g = torch.Generator().manual_seed(3)
 
-    # token-slot lists: one per query head, and one per KV head
+    # token-slot lists: one per query head, and one per KV head -- the short-list kernel with 64-bit
+    # row offsets; then the same call as a fused decode step (the newest token is the one being
+    # decoded: RoPE of q and its key, the cache write at the far end of the pool, attention)
+    from tidaldecode_amd import _kernels
+
     for rows in (hq, hkv):
         pos = torch.stack([torch.randperm(n, generator=g)[:k] for _ in range(rows)])
         want = orc.sparse_layer_gather(q, case.k, case.v, pos)
@@ -73,7 +77,34 @@ def test_decode_attention_beyond_4gib(cuda, dtype, hq, hkv, pool_pages):
         w.forward(qd, od, case.pool, case.slots_of(pos).to(torch.int32).to(cuda), None, 0, 0, None,
                   index_kind="slots")
         torch.cuda.synchronize()
+        assert _kernels.last_decode_kernel() == "short-list, 64-bit offsets"
         assert tolerance_report(od[0], want) <= ATOL[dtype], rows
+
+        pos[::2, 0] = n - 1                                   # every second list names the new token
+        for r in range(1, rows, 2):
+            pos[r][pos[r] == n - 1] = int((set(range(n - 1)) - set(pos[r].tolist())).pop())
+        for r in range(0, rows, 2):                           # ... once
+            dup = (pos[r, 1:] == n - 1).nonzero().flatten()
+            if dup.numel():
+                pos[r, 1 + int(dup[0])] = int((set(range(n - 1)) - set(pos[r].tolist())).pop())
+        theta, new_pos = 5e5, 70001
+        k_new, v_new = randn((1, hkv, d), 31, dtype), randn((1, hkv, d), 32, dtype)
+        k_f, v_f = case.k.clone(), case.v.clone()
+        k_f[n - 1] = rotated(k_new, [new_pos], dtype, theta)[0]
+        v_f[n - 1] = v_new[0]
+        want = orc.sparse_layer_gather(rotated(q[None], [new_pos], dtype, theta)[0], k_f, v_f, pos)
+        dst = case.slots_of(torch.tensor([n - 1])).to(torch.int32).to(cuda)
+        cos, sin = _kernels.rope_table(torch.tensor([new_pos], dtype=torch.int32, device=cuda), d, 1.0, theta)
+        page_f, entry_f = int(dst[0]) // page, int(dst[0]) % page
+        before = case.pool[page_f].clone()
+        w.forward(qd, od, case.pool, case.slots_of(pos).to(torch.int32).to(cuda), None, 0, 0, None,
+                  index_kind="slots", fresh=(k_new.to(dtype).to(cuda), v_new.to(dtype).to(cuda), cos, sin, dst))
+        torch.cuda.synchronize()
+        assert _kernels.last_decode_kernel() == "short-list, 64-bit offsets"
+        assert tolerance_report(od[0], want) <= ATOL[dtype], rows
+        assert within_ulps(case.pool[page_f, 0, entry_f], k_f[n - 1], dtype)
+        assert torch.equal(case.pool[page_f, 1, entry_f].cpu(), v_new[0].to(dtype))
+        case.pool[page_f] = before                            # the later checks use the original token
 
     # the whole page table in order, logits and log-sum-exp out (selection layer)
     logits = orc.attn_logits(q, case.k)

@@ -414,3 +414,58 @@ def test_fused_decode_step_with_shared_kv_rows(cuda, dtype, hq, hkv):
         assert ((p2.float() - p1.float()).abs() <= ulp * p1.float().abs() + 1e-6).all()
         changed = (p1 != pool).any(dim=(1, 2, 3, 4)).nonzero().flatten().tolist()
         assert changed == sorted(set(last_idx.tolist()))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("page", [1, 3, 7, 12, 31])
+@pytest.mark.parametrize("hq,hkv,rows", [(8, 8, 8), (16, 4, 4), (8, 2, 8)])
+def test_pages_of_any_size(cuda, dtype, page, hq, hkv, rows):
+    """Page sizes that are not a power of two (the reference tests 3, 7 and 31,
+    kernels/src/test/test_batch_decode.cu:215-267): the short-list kernel divides the slot by the
+    page size once per lane and forms 64-bit row offsets.  Slot lists with the forced last page,
+    then the fused decode step, both against the oracle."""
+    from oracle import tidal_oracle as orc
+    from tidaldecode_amd import _kernels
+
+    d, n = 128, 1000 + page // 2
+    case = PagedCase(n, hkv, d, page, dtype, seed=page + hq)
+    pool = case.pool.to(cuda)
+    q = randn((hq, d), 5, dtype)
+    qd = q.to(dtype).to(cuda).unsqueeze(0)
+    before_last = (case.n_pages - 1) * page
+    g = torch.Generator().manual_seed(page)
+    w = _wrapper(0, hq, hkv, d, page, dtype)
+    kernel = "short-list" if page == 1 else "short-list, 64-bit offsets"
+    for k in (1, 33, 600):
+        pos = torch.stack([torch.randperm(before_last, generator=g)[:k] for _ in range(rows)])
+        allpos = torch.cat([pos, torch.arange(before_last, n).repeat(rows, 1)], 1)
+        want = orc.sparse_layer_gather(q, case.k, case.v, allpos)
+        od = torch.full_like(qd, float("nan"))
+        w.forward(qd, od, pool, case.slots_of(pos).to(torch.int32).to(cuda).contiguous(), None,
+                  case.last_page_len, int(case.page_table[-1]), None, index_kind="slots")
+        torch.cuda.synchronize()
+        assert _kernels.last_decode_kernel() == kernel
+        assert tolerance_report(od[0], want) <= ATOL[dtype], (k, page)
+    # fused step: the newest token is the one being decoded and sits in every list
+    theta, new_pos = 1e4, n - 1
+    pos = torch.stack([torch.randperm(n - 1, generator=g)[:199] for _ in range(rows)])
+    pos = torch.cat([pos, torch.full((rows, 1), n - 1)], 1)
+    k_new, v_new = randn((1, hkv, d), 41, dtype), randn((1, hkv, d), 42, dtype)
+    k_f, v_f = case.k.clone(), case.v.clone()
+    k_f[n - 1] = rotated(k_new, [new_pos], dtype, theta)[0]
+    v_f[n - 1] = v_new[0]
+    want = orc.sparse_layer_gather(rotated(q[None], [new_pos], dtype, theta)[0], k_f, v_f, pos)
+    dst = case.slots_of(torch.tensor([n - 1])).to(torch.int32).to(cuda)
+    cos, sin = _kernels.rope_table(torch.tensor([new_pos], dtype=torch.int32, device=cuda), d, 1.0, theta)
+    pool_f = pool.clone()
+    od = torch.full_like(qd, float("nan"))
+    w.forward(qd, od, pool_f, case.slots_of(pos).to(torch.int32).to(cuda).contiguous(), None, 0, 0, None,
+              index_kind="slots", fresh=(k_new.to(dtype).to(cuda), v_new.to(dtype).to(cuda), cos, sin, dst))
+    torch.cuda.synchronize()
+    assert _kernels.last_decode_kernel() == kernel
+    assert tolerance_report(od[0], want) <= ATOL[dtype], page
+    page_f, entry_f = int(dst[0]) // page, int(dst[0]) % page
+    assert within_ulps(pool_f[page_f, 0, entry_f], k_f[n - 1], dtype)
+    assert torch.equal(pool_f[page_f, 1, entry_f].cpu(), v_new[0].to(dtype))
+    pool_f[page_f, :, entry_f] = pool[page_f, :, entry_f]
+    assert torch.equal(pool_f, pool)

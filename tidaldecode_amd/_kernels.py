@@ -658,6 +658,12 @@ class BatchDecodeWithPagedKVCachePyTorchWrapper:
                                  ws.numel() if ws is not None else 0, _stream()))
 
 
+def last_decode_kernel() -> str:
+    """Kernel family that served this thread's last decode-attention call ("short-list",
+    "streaming", each possibly with ", 64-bit offsets")."""
+    return lib.td_last_decode_kernel().decode()
+
+
 def gather_probe(wrapper: "BatchDecodeWithPagedKVCachePyTorchWrapper", paged_kv_data: torch.Tensor,
                  slots: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Measurement aid: only the memory side of ``wrapper.forward(..., slots, index_kind="slots")``

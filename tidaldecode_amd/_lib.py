@@ -86,6 +86,7 @@ SIGNATURES = {
     "td_last_error": (c_char_p, []),
     "td_version": (c_int32, []),
     "td_num_cus": (c_int32, []),
+    "td_last_decode_kernel": (c_char_p, []),
     "td_rope_in_place": (
         c_int32,
         [c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int64, c_float, c_float,

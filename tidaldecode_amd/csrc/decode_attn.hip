@@ -68,6 +68,11 @@ static int static_scratch(void** out) {
 
 using namespace tidal;
 
+// kernel family that served this thread's last td_decode_attn call
+static thread_local const char* g_last_kernel = "none";
+
+extern "C" const char* td_last_decode_kernel(void) { return g_last_kernel; }
+
 extern "C" int td_num_cus(void) { return num_cus(); }
 
 extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t num_kv_heads,
@@ -312,11 +317,6 @@ static int build_params(const td_paged_kv* kv, const td_index_list* list, const 
   if (fresh) {
     TD_REQUIRE(fresh->k && fresh->v && fresh->cos && fresh->sin && fresh->dst_slot,
                "td_decode_attn: fresh token with a NULL member");
-    if (!p.lean)
-      return fail(TD_ERR_UNSUPPORTED,
-                  "td_decode_attn: the fused decode step needs a power-of-two page_size and a pool "
-                  "below 4 GiB (page_size %d, pool %lld bytes); use td_rope_append_decode first",
-                  P, (long long)(kv->max_pages * p.page_stride * 2));
     p.fresh_k = fresh->k;
     p.fresh_v = fresh->v;
     p.fresh_cos = fresh->cos;
@@ -364,17 +364,24 @@ static int build_params(const td_paged_kv* kv, const td_index_list* list, const 
 }
 
 // Whether a call can run on the short-list kernel of its plan: token-slot lists, head_dim 128, one
-// query head per list walk, 32-bit lean addressing whose strides fit the 24-bit multiplier, no
-// score output, chunks that are a power-of-two multiple of the kernel's workgroup tile.
-static bool sparse_kernel_fits(const DecodeParams& p, const td_decode_plan* plan,
-                               const td_index_list* list, int qpg, int head_dim, bool emit) {
+// query head per list walk or a whole group per shared list, no score output, chunks that are a
+// power-of-two multiple of the kernel's workgroup tile.  Returns 0 (no), kSparseLean (power-of-two
+// pages, pool below 4 GiB, strides within the 24-bit multiplier: 32-bit row offsets) or kSparseWide
+// (any page size, 64-bit row offsets; 8 rows per lane only).
+enum { kSparseNo = 0, kSparseLean = 1, kSparseWide = 2 };
+static int sparse_kernel_fits(const DecodeParams& p, const td_decode_plan* plan,
+                              const td_index_list* list, int qpg, int head_dim, bool emit) {
   if (plan->sparse_waves <= 0 || !sparse_shape_supported(plan->sparse_waves, plan->sparse_rows, qpg))
-    return false;
+    return kSparseNo;
   const int stile = plan->sparse_waves * 4 * plan->sparse_rows;
   const bool heads_fit = qpg == 1 ? p.qpk_shift >= 0 : (p.q_per_kv == qpg && p.subs == 1);
-  return list->kind == TD_IDX_SLOTS && p.lean && !emit && heads_fit && head_dim == 128 &&
-         p.chunk_shift >= 0 && plan->chunk_tokens % stile == 0 &&
-         p.page_stride_b < (1u << 24) && p.entry_stride_b < (1u << 24);
+  if (!(list->kind == TD_IDX_SLOTS && !emit && heads_fit && head_dim == 128 && p.chunk_shift >= 0 &&
+        plan->chunk_tokens % stile == 0))
+    return kSparseNo;
+  if (p.lean && p.page_stride_b < (1u << 24) && p.entry_stride_b < (1u << 24)) return kSparseLean;
+  // a page's bytes and an entry's offset inside it stay 32-bit; the page base is a 64-bit product
+  if (plan->sparse_rows == 8 && p.page_stride * 2 < ((int64_t)1 << 32)) return kSparseWide;
+  return kSparseNo;
 }
 
 extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
@@ -394,21 +401,30 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
   dim3 grid(n_hrows, plan->max_splits, batch);
   const bool merge_kernel = plan->max_splits > 1 && !plan->fused_merge;
   int rc;
-  if (sparse_kernel_fits(p, plan, list, qpg, D, scores != nullptr)) {
+  const int fits = sparse_kernel_fits(p, plan, list, qpg, D, scores != nullptr);
+  if (fits != kSparseNo) {
+    const bool wide = fits == kSparseWide;
     TD_REQUIRE((int64_t)batch * n_hrows * qpg * kTicketStride * 4 <= kTicketBytes,
                "td_decode_attn: batch %d x %d heads exceeds the ticket counters", batch, n_hrows * qpg);
     if (qpg > 1)
       rc = kv->dtype == TD_F16
-               ? launch_sparse_shared_f16(p, plan->sparse_waves, qpg, merge_kernel, grid, st)
-               : launch_sparse_shared_bf16(p, plan->sparse_waves, qpg, merge_kernel, grid, st);
+               ? launch_sparse_shared_f16(p, plan->sparse_waves, qpg, wide, merge_kernel, grid, st)
+               : launch_sparse_shared_bf16(p, plan->sparse_waves, qpg, wide, merge_kernel, grid, st);
     else if (kv->dtype == TD_F16)
-      rc = launch_sparse_f16(p, plan->sparse_waves, plan->sparse_rows, false, merge_kernel, grid, st);
+      rc = launch_sparse_f16(p, plan->sparse_waves, plan->sparse_rows, false, wide, merge_kernel, grid, st);
     else
-      rc = launch_sparse_bf16(p, plan->sparse_waves, plan->sparse_rows, false, merge_kernel, grid, st);
+      rc = launch_sparse_bf16(p, plan->sparse_waves, plan->sparse_rows, false, wide, merge_kernel, grid, st);
     if (rc != TD_OK) return rc;
     TD_HIP_CHECK(hipGetLastError());
+    g_last_kernel = wide ? "short-list, 64-bit offsets" : "short-list";
     return TD_OK;
   }
+  if (fresh && !p.lean)
+    return fail(TD_ERR_UNSUPPORTED,
+                "td_decode_attn: outside the short-list kernel (token-slot lists of up to %lld entries, "
+                "head_dim 128, no score output) the fused decode step needs a power-of-two page_size and "
+                "a pool below 4 GiB (page_size %d, pool %lld bytes); use td_rope_append_decode first",
+                (long long)kSparseMaxItems, kv->page_size, (long long)(kv->max_pages * p.page_stride * 2));
   if (kv->dtype == TD_F16)
     rc = launch_decode_f16(p, D, qpg, plan->waves_per_block, plan->tile_rows, page_mode, scores != nullptr,
                            merge_kernel, grid, st);
@@ -417,6 +433,7 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
                             merge_kernel, grid, st);
   if (rc != TD_OK) return rc;
   TD_HIP_CHECK(hipGetLastError());
+  g_last_kernel = p.lean ? "streaming" : "streaming, 64-bit offsets";
   return TD_OK;
 }
 
@@ -497,16 +514,18 @@ extern "C" int td_gather_probe(const td_paged_kv* kv, const td_index_list* list,
                                nullptr, nullptr, out, (int64_t)1 << 40, p, qpg, n_hrows);
   if (prc != TD_OK) return prc;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  if (qpg == 1 && sparse_kernel_fits(p, plan, list, qpg, kv->head_dim, false) &&
-      list->last_page_len == 0 && !list->last_page_len_arr) {
+  const int fits = qpg == 1 ? sparse_kernel_fits(p, plan, list, qpg, kv->head_dim, false) : kSparseNo;
+  if (fits != kSparseNo && list->last_page_len == 0 && !list->last_page_len_arr) {
     // the short-list kernel's own loads-only form; it reads `out` as q and writes nothing
     TD_REQUIRE(out_bytes >= (int64_t)batch * num_qo_heads * kv->head_dim * 2,
                "td_gather_probe: out holds %lld bytes, %lld needed", (long long)out_bytes,
                (long long)batch * num_qo_heads * kv->head_dim * 2);
     const dim3 sgrid(n_hrows, plan->max_splits, batch);
-    const int src = kv->dtype == TD_F16
-                        ? launch_sparse_f16(p, plan->sparse_waves, plan->sparse_rows, true, false, sgrid, st)
-                        : launch_sparse_bf16(p, plan->sparse_waves, plan->sparse_rows, true, false, sgrid, st);
+    const bool wide = fits == kSparseWide;
+    const int src =
+        kv->dtype == TD_F16
+            ? launch_sparse_f16(p, plan->sparse_waves, plan->sparse_rows, true, wide, false, sgrid, st)
+            : launch_sparse_bf16(p, plan->sparse_waves, plan->sparse_rows, true, wide, false, sgrid, st);
     if (src != TD_OK) return src;
     TD_HIP_CHECK(hipGetLastError());
     return TD_OK;

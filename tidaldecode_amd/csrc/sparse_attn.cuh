@@ -213,7 +213,7 @@ __device__ __forceinline__ void finish_head(const DecodeParams& p, int lane, int
 
 // QPG query heads per loaded K/V row: 1 (every head row is a query head with its own walk of a
 // list) or the 2, 4 or 8 query heads of a KV head that share one list (a head row is a KV head).
-template <typename T, int NW, int U, bool FRESH, bool PROBE = false, int QPG = 1>
+template <typename T, int NW, int U, bool FRESH, bool PROBE = false, int QPG = 1, bool WIDE = false>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U == 16 ? 2 : 4))) void sparse_attn_kernel(const DecodeParams p) {
   static_assert(QPG == 1 || U == 8, "shared KV rows: 8 rows per lane");
   constexpr int D = 128;
@@ -261,31 +261,40 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
   };
   int32_t ent = fetch_entry(t0);
 
+  // ---- q, and in the fused decode step (FRESH) what the workgroup's first wave prepares ----------
+  // FRESH: q arrives un-rotated.  Wave 0 of the workgroup alone loads q, the step's cos / sin and
+  // the new token's k and v, rotates q and k once, and leaves rotated q, rotated k and v in LDS for
+  // the other waves (which then issue no global load besides their list entry and K/V rows: eight
+  // waves per workgroup asking the same few cache lines for cos / sin cost the launch 0.5 us).
   uint32_t qp[QPG][4];
+  const bool prep = FRESH && wave == 0;  // scalar
+  if constexpr (!FRESH) {
 #pragma unroll
-  for (int j = 0; j < QPG; ++j) {
-    const u32x4 v =
-        reinterpret_cast<const u32x4*>(p.q)[((int64_t)b * p.num_qo_heads + rq0 + j) * LPR + li];
-    qp[j][0] = v.x; qp[j][1] = v.y; qp[j][2] = v.z; qp[j][3] = v.w;
+    for (int j = 0; j < QPG; ++j) {
+      const u32x4 v =
+          reinterpret_cast<const u32x4*>(p.q)[((int64_t)b * p.num_qo_heads + rq0 + j) * LPR + li];
+      qp[j][0] = v.x; qp[j][1] = v.y; qp[j][2] = v.z; qp[j][3] = v.w;
+    }
   }
-  uint32_t knew[4] = {0, 0, 0, 0}, vnew[4] = {0, 0, 0, 0};
-  float rcs[8], rsn[8];
+  // What wave 0 loads for the fused step.  Defined in that wave only and read in that wave only:
+  // giving the other waves a value here would make them wait for their list entry first (the
+  // registers are the destination of loads in flight on the other side of the branch).
+  u32x4 q_raw[QPG], kn_raw, vn_raw;
+  f32x4 cos_lo, cos_hi, sin_lo, sin_hi;
   if constexpr (FRESH) {
-    constexpr int HALF = LPR / 2;
-    const f32x4* cp = reinterpret_cast<const f32x4*>(p.fresh_cos + (int64_t)b * (D / 2) + (li % HALF) * 8);
-    const f32x4* sp = reinterpret_cast<const f32x4*>(p.fresh_sin + (int64_t)b * (D / 2) + (li % HALF) * 8);
-    const f32x4 c0 = cp[0], c1v = cp[1], s0 = sp[0], s1 = sp[1];
-    rcs[0] = c0.x; rcs[1] = c0.y; rcs[2] = c0.z; rcs[3] = c0.w;
-    rcs[4] = c1v.x; rcs[5] = c1v.y; rcs[6] = c1v.z; rcs[7] = c1v.w;
-    const float sgn = li < HALF ? -1.f : 1.f;  // y_lo = x_lo c - x_hi s,  y_hi = x_hi c + x_lo s
-    rsn[0] = sgn * s0.x; rsn[1] = sgn * s0.y; rsn[2] = sgn * s0.z; rsn[3] = sgn * s0.w;
-    rsn[4] = sgn * s1.x; rsn[5] = sgn * s1.y; rsn[6] = sgn * s1.z; rsn[7] = sgn * s1.w;
-    const int n_kv = QPG > 1 ? p.num_qo_heads / QPG : p.num_qo_heads >> p.qpk_shift;
-    const int64_t fresh_off = ((int64_t)b * n_kv + kv_head) * LPR + li;
-    const u32x4 kn = reinterpret_cast<const u32x4*>(p.fresh_k)[fresh_off];
-    const u32x4 vn = reinterpret_cast<const u32x4*>(p.fresh_v)[fresh_off];
-    knew[0] = kn.x; knew[1] = kn.y; knew[2] = kn.z; knew[3] = kn.w;
-    vnew[0] = vn.x; vnew[1] = vn.y; vnew[2] = vn.z; vnew[3] = vn.w;
+    if (prep) {
+#pragma unroll
+      for (int j = 0; j < QPG; ++j)
+        q_raw[j] = reinterpret_cast<const u32x4*>(p.q)[((int64_t)b * p.num_qo_heads + rq0 + j) * LPR + li];
+      constexpr int HALF = LPR / 2;
+      const f32x4* cp = reinterpret_cast<const f32x4*>(p.fresh_cos + (int64_t)b * (D / 2) + (li % HALF) * 8);
+      const f32x4* sp = reinterpret_cast<const f32x4*>(p.fresh_sin + (int64_t)b * (D / 2) + (li % HALF) * 8);
+      cos_lo = cp[0]; cos_hi = cp[1]; sin_lo = sp[0]; sin_hi = sp[1];
+      const int n_kv = QPG > 1 ? p.num_qo_heads / QPG : p.num_qo_heads >> p.qpk_shift;
+      const int64_t fresh_off = ((int64_t)b * n_kv + kv_head) * LPR + li;
+      kn_raw = reinterpret_cast<const u32x4*>(p.fresh_k)[fresh_off];
+      vn_raw = reinterpret_cast<const u32x4*>(p.fresh_v)[fresh_off];
+    }
   }
 
   // ---- the sequence: listed entries, forced last page, splits ------------------------------------
@@ -320,23 +329,31 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
   n_splits = n_splits > p.max_splits ? p.max_splits : n_splits;
   n_splits = n_splits < 1 ? 1 : n_splits;
   if (split >= n_splits) return;  // uniform for the workgroup
-  const uint32_t last_base = (uint32_t)s.last_idx << p.page_shift;
-
-  // rotate-half RoPE of 8 elements per lane; the partner dimension (+- 64) sits 8 lanes away
-  auto rotate = [&](uint32_t(&w)[4]) {
-    float x[8], y[8];
-#pragma unroll
-    for (int c = 0; c < 4; ++c) unpack2<T>(w[c], x[2 * c], x[2 * c + 1]);
-#pragma unroll
-    for (int d = 0; d < 8; ++d) y[d] = x[d] * rcs[d] + dpp_move<0x128>(x[d]) * rsn[d];
-#pragma unroll
-    for (int c = 0; c < 4; ++c) w[c] = pack2<T>(y[2 * c], y[2 * c + 1]);
-  };
+  const uint32_t last_base = (uint32_t)s.last_idx * (uint32_t)p.page_size;
 
   const char* kbase = reinterpret_cast<const char*>(p.kv);
   const char* vbase = kbase + p.v_offset * 2;
   const uint32_t head_byte_off = (uint32_t)(kv_head * p.head_stride + li * 8) * 2u;
-  const uint32_t entry_mask = (1u << p.page_shift) - 1u;
+  const uint32_t entry_mask = (1u << (p.page_shift & 31)) - 1u;
+  // Byte offset of a token slot's K row of head 0 in the pool.  Lean form: power-of-two pages, a
+  // pool below 4 GiB and strides that fit the 24-bit multiplier.  Wide form: any page size (one
+  // division per lane and tile) and 64-bit offsets.
+  using off_t = typename std::conditional<WIDE, uint64_t, uint32_t>::type;
+  auto slot_offset = [&](uint32_t slot) -> off_t {
+    if constexpr (WIDE) {
+      uint32_t page, entry;
+      if (p.page_shift >= 0) {
+        page = slot >> p.page_shift;
+        entry = slot & entry_mask;
+      } else {
+        page = slot / (uint32_t)p.page_size;
+        entry = slot - page * (uint32_t)p.page_size;
+      }
+      return (uint64_t)page * (uint64_t)p.page_stride_b + (uint64_t)(entry * p.entry_stride_b);
+    } else {
+      return __umul24(slot >> p.page_shift, p.page_stride_b) + __umul24(slot & entry_mask, p.entry_stride_b);
+    }
+  };
 
   float m_run = kNegBig;  // wave-uniform running maximum (base-2 logits)
   float l_lane = 0.f;     // this lane's share of the denominator
@@ -352,92 +369,88 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
 #pragma unroll
   for (int d = 0; d < 8; ++d) accm[d] = f32x4{0.f, 0.f, 0.f, 0.f};
   __shared__ __attribute__((aligned(16))) float sm_p[QPG > 1 ? NW * QPG * TILE : 4];
-  // Decode-step fusion: q arrives un-rotated and is rotated in registers, once per wave.  The new
-  // token's key is rotated by the wave that writes it into the cache (one per KV head) and by
-  // every wave whose tokens include its slot.
-  bool q_rot = false, k_rot = false, wrote = false;  // wave-uniform
-  const bool writer = FRESH && split == 0 && wave == 0 && (QPG > 1 || hrow == (kv_head << p.qpk_shift));
-  auto fresh_duties = [&](bool any_hit) {
-    if (!q_rot) {
+  // fused decode step: rotated q rows, the new token's rotated key and its value, 256 bytes each
+  __shared__ __attribute__((aligned(16))) uint32_t sm_fresh[FRESH ? (QPG + 2) * 64 : 4];
+  uint32_t* const sm_knew = sm_fresh + (FRESH ? QPG * 64 : 0);
+  uint32_t* const sm_vnew = sm_knew + (FRESH ? 64 : 0);
+
+  // ---- one tile of the wave: slot and row offset of the lane's own token, then every K and V row ----
+  u32x4 kb[U], vb[U];
+  uint32_t slot = 0;   // of this lane's token
+  bool valid = false;  // the token exists
+  auto issue = [&](int t, int32_t entry_raw) {
+    const int i = t + own;
+    valid = i < c1;
+    // entry_raw was read at min(i, capacity - 1), which is i for every listed token (n_list <= capacity)
+    slot = i < s.n_list ? (uint32_t)entry_raw : last_base + (uint32_t)(i - s.n_list);
+    slot = slot > p.max_slot ? p.max_slot : slot;
+    off_t off_own = slot_offset(slot);
+    // lanes past the end of the list repeat the first token of the tile (which exists: t < c1)
+    // with weight 0: a row that holds real data, whatever the unused list entries say
+    if constexpr (WIDE) {
+      const uint32_t lo = (uint32_t)off_own, hi = (uint32_t)(off_own >> 32);
+      const uint32_t lo0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)lo);
+      const uint32_t hi0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)hi);
+      const uint32_t lo_own = valid ? lo : lo0, hi_own = valid ? hi : hi0;
+      const char* ka[U];
+#define TD_ROW_OFF(N)                                                                              \
+  if constexpr (N < U)                                                                             \
+    ka[N] = kbase + ((((uint64_t)row_bcast_u32<N>(hi_own)) << 32) | (uint64_t)row_bcast_u32<N>(lo_own)) + \
+            head_byte_off;
+      TD_ROW_OFF(0) TD_ROW_OFF(1) TD_ROW_OFF(2) TD_ROW_OFF(3) TD_ROW_OFF(4) TD_ROW_OFF(5)
+      TD_ROW_OFF(6) TD_ROW_OFF(7) TD_ROW_OFF(8) TD_ROW_OFF(9) TD_ROW_OFF(10) TD_ROW_OFF(11)
+      TD_ROW_OFF(12) TD_ROW_OFF(13) TD_ROW_OFF(14) TD_ROW_OFF(15)
+#undef TD_ROW_OFF
 #pragma unroll
-      for (int j = 0; j < QPG; ++j) rotate(qp[j]);
-      q_rot = true;
-    }
-    if ((any_hit || (writer && !wrote)) && !k_rot) {
-      rotate(knew);
-      k_rot = true;
-    }
-    if (writer && !wrote) {
-      if (g == 0) {
-        const uint32_t ns = new_slot > p.max_slot ? p.max_slot : new_slot;
-        char* dst = reinterpret_cast<char*>(const_cast<void*>(p.kv)) +
-                    (ns >> p.page_shift) * p.page_stride_b + (ns & entry_mask) * p.entry_stride_b +
-                    head_byte_off;
-        const u32x4 ko = {knew[0], knew[1], knew[2], knew[3]};
-        const u32x4 vo = {vnew[0], vnew[1], vnew[2], vnew[3]};
-        *reinterpret_cast<u32x4*>(dst) = ko;
-        *reinterpret_cast<u32x4*>(dst + p.v_offset * 2) = vo;
-      }
-      wrote = true;
+      for (int u = 0; u < U; ++u)
+        kb[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(ka[u]));
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        vb[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(ka[u] + p.v_offset * 2));
+    } else {
+      off_own = valid ? off_own : (uint32_t)__builtin_amdgcn_readfirstlane((int)off_own);
+      uint32_t offs[U];
+#define TD_ROW_OFF(N) \
+  if constexpr (N < U) offs[N] = row_bcast_u32<N>(off_own) + head_byte_off;
+      TD_ROW_OFF(0) TD_ROW_OFF(1) TD_ROW_OFF(2) TD_ROW_OFF(3) TD_ROW_OFF(4) TD_ROW_OFF(5)
+      TD_ROW_OFF(6) TD_ROW_OFF(7) TD_ROW_OFF(8) TD_ROW_OFF(9) TD_ROW_OFF(10) TD_ROW_OFF(11)
+      TD_ROW_OFF(12) TD_ROW_OFF(13) TD_ROW_OFF(14) TD_ROW_OFF(15)
+#undef TD_ROW_OFF
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        kb[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kbase + offs[u]));
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        vb[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vbase + offs[u]));
     }
   };
 
-  const int STEP = n_splits * NW * TILE;
-  for (int t = t0; t < c1; t += STEP) {
-    if (t != t0) ent = fetch_entry(t);
-    // this lane's token: its slot, whether it exists, whether it is the token being decoded
-    const int i = t + own;
-    const bool valid = i < c1;
-    // ent was read at min(i, capacity - 1), which is i for every listed token (n_list <= capacity)
-    uint32_t slot = i < s.n_list ? (uint32_t)ent : last_base + (uint32_t)(i - s.n_list);
-    slot = slot > p.max_slot ? p.max_slot : slot;
-    uint32_t off_own = __umul24(slot >> p.page_shift, p.page_stride_b) +
-                       __umul24(slot & entry_mask, p.entry_stride_b);
-    // lanes past the end of the list repeat the first token of the tile (which exists: t < c1)
-    // with weight 0: a row that holds real data, whatever the unused list entries say
-    off_own = valid ? off_own : (uint32_t)__builtin_amdgcn_readfirstlane(off_own);
-
-    u32x4 kb[U], vb[U];
-    uint32_t offs[U];
-#define TD_ROW_OFF(N) \
-  if constexpr (N < U) offs[N] = row_bcast_u32<N>(off_own) + head_byte_off;
-    TD_ROW_OFF(0) TD_ROW_OFF(1) TD_ROW_OFF(2) TD_ROW_OFF(3) TD_ROW_OFF(4) TD_ROW_OFF(5)
-    TD_ROW_OFF(6) TD_ROW_OFF(7) TD_ROW_OFF(8) TD_ROW_OFF(9) TD_ROW_OFF(10) TD_ROW_OFF(11)
-    TD_ROW_OFF(12) TD_ROW_OFF(13) TD_ROW_OFF(14) TD_ROW_OFF(15)
-#undef TD_ROW_OFF
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-      kb[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kbase + offs[u]));
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-      vb[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vbase + offs[u]));
-
+  // ---- arithmetic of the tile whose rows `issue` asked for ----------------------------------------
+  auto compute = [&](bool first_tile) {
     if constexpr (PROBE) {  // measurement: the loads alone, no arithmetic and no merge
       u32x4 fold = {0u, 0u, 0u, 0u};
 #pragma unroll
       for (int u = 0; u < U; ++u) fold ^= kb[u] ^ vb[u];
       uint32_t w = fold.x ^ fold.y ^ fold.z ^ fold.w;
       if (w == 0x12345678u) reinterpret_cast<uint32_t*>(p.o)[0] = w;
-      continue;
+      return;
     }
-    bool hit = false;
+    // The token being decoded is used from LDS (where wave 0 left it) wherever the list names its
+    // slot: what the pool holds there is being written by another workgroup of this launch.
     if constexpr (FRESH) {
-      hit = slot == new_slot;
+      bool hit = slot == new_slot;
       const uint32_t hit_first = __builtin_amdgcn_readfirstlane(hit ? 1u : 0u);
-      hit = valid ? hit : (hit_first != 0);
-    }
-    if constexpr (FRESH) fresh_duties(__ballot(hit) != 0);  // behind the loads: hidden by their latency
-    // The token being decoded is used from registers wherever the list names its slot: what the
-    // pool holds there is being written by another workgroup of this launch.
-    if constexpr (FRESH) {
+      hit = valid ? hit : (hit_first != 0);  // lanes without a token hold a copy of the first lane's rows
       if (__ballot(hit)) {
+        const u32x4 kn = *reinterpret_cast<const u32x4*>(sm_knew + li * 4);
+        const u32x4 vn = *reinterpret_cast<const u32x4*>(sm_vnew + li * 4);
         const uint32_t hm = hit ? 1u : 0u;
-#define TD_ROW_FIX(N)                                                                   \
-  if constexpr (N < U) {                                                                \
-    if (row_bcast_u32<N>(hm)) {                                                         \
-      kb[N].x = knew[0]; kb[N].y = knew[1]; kb[N].z = knew[2]; kb[N].w = knew[3];       \
-      vb[N].x = vnew[0]; vb[N].y = vnew[1]; vb[N].z = vnew[2]; vb[N].w = vnew[3];       \
-    }                                                                                   \
+#define TD_ROW_FIX(N)                   \
+  if constexpr (N < U) {                \
+    if (row_bcast_u32<N>(hm)) {         \
+      kb[N] = kn;                       \
+      vb[N] = vn;                       \
+    }                                   \
   }
         TD_ROW_FIX(0) TD_ROW_FIX(1) TD_ROW_FIX(2) TD_ROW_FIX(3) TD_ROW_FIX(4) TD_ROW_FIX(5)
         TD_ROW_FIX(6) TD_ROW_FIX(7) TD_ROW_FIX(8) TD_ROW_FIX(9) TD_ROW_FIX(10) TD_ROW_FIX(11)
@@ -473,7 +486,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
         lh[j] = lh[j] * alpha[j] + (li < 8 ? pr : 0.f);  // lanes li and li ^ 8 hold the same token
         if (li < 8) sp[j * TILE + own] = pr;
       }
-      if (t != t0) {  // later tiles: rescale what the earlier ones left (row r of group g: head 4 g + r)
+      if (!first_tile) {  // later tiles: rescale what the earlier ones left (row r of group g: head 4 g + r)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const float f = (QPG == 8 && g == 1) ? alpha[(4 + r) % QPG] : alpha[r % QPG];
@@ -518,7 +531,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
         }
       }
       asm volatile("" ::: "memory");  // the strip is rewritten by the next tile only after these reads
-      continue;
+      return;
     }
     // q.k: U partial sums per lane, reduce-scattered so that the lane ends with its own token
     float part[U];
@@ -560,9 +573,81 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
     TD_ROW_PV(7) TD_ROW_PV(8) TD_ROW_PV(9) TD_ROW_PV(10) TD_ROW_PV(11) TD_ROW_PV(12)
     TD_ROW_PV(13) TD_ROW_PV(14) TD_ROW_PV(15)
 #undef TD_ROW_PV
+  };
+
+  // ---- the wave's tiles: rows of the first one are asked for before anything else happens --------
+  const int STEP = n_splits * NW * TILE;
+  int t = t0;
+  bool live = t < c1;  // wave-uniform
+  if (!prep && live) issue(t, ent);
+
+  if constexpr (FRESH) {
+    // Wave 0 rotates q and the new key while the other waves' rows are in flight (its own are asked
+    // for right after: what it loaded for the rotation has arrived with its list entry, and the
+    // registers are free again before its K/V rows need them) and leaves them and the new value in
+    // LDS; the cache write of the new token follows after the tiles, from LDS.
+    if (prep) {
+      const float rcs[8] = {cos_lo.x, cos_lo.y, cos_lo.z, cos_lo.w, cos_hi.x, cos_hi.y, cos_hi.z, cos_hi.w};
+      const float sgn = li < LPR / 2 ? -1.f : 1.f;  // y_lo = x_lo c - x_hi s,  y_hi = x_hi c + x_lo s
+      const float rsn[8] = {sgn * sin_lo.x, sgn * sin_lo.y, sgn * sin_lo.z, sgn * sin_lo.w,
+                            sgn * sin_hi.x, sgn * sin_hi.y, sgn * sin_hi.z, sgn * sin_hi.w};
+      // rotate-half RoPE of 8 elements per lane; the partner dimension (+- 64) sits 8 lanes away
+      auto rotate = [&](uint32_t(&w)[4]) {
+        float x[8], y[8];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) unpack2<T>(w[c], x[2 * c], x[2 * c + 1]);
+#pragma unroll
+        for (int d = 0; d < 8; ++d) y[d] = x[d] * rcs[d] + dpp_move<0x128>(x[d]) * rsn[d];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) w[c] = pack2<T>(y[2 * c], y[2 * c + 1]);
+      };
+      uint32_t knew[4] = {kn_raw.x, kn_raw.y, kn_raw.z, kn_raw.w};
+      rotate(knew);
+      if (g == 0) {
+        *reinterpret_cast<u32x4*>(sm_knew + li * 4) = u32x4{knew[0], knew[1], knew[2], knew[3]};
+        *reinterpret_cast<u32x4*>(sm_vnew + li * 4) = vn_raw;
+      }
+#pragma unroll
+      for (int j = 0; j < QPG; ++j) {
+        uint32_t qj[4] = {q_raw[j].x, q_raw[j].y, q_raw[j].z, q_raw[j].w};
+        rotate(qj);
+        if (g == 0) *reinterpret_cast<u32x4*>(sm_fresh + j * 64 + li * 4) = u32x4{qj[0], qj[1], qj[2], qj[3]};
+      }
+      if (live) issue(t, ent);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the LDS writes have landed
+    }
+    // a bare barrier: the fence of __syncthreads would wait for the rows in flight
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    // every wave, the first included: registers that no global load of either branch is still
+    // writing to, so that the wait the compiler puts in front of this read is for LDS only
+#pragma unroll
+    for (int j = 0; j < QPG; ++j) {
+      const u32x4 v = *reinterpret_cast<const u32x4*>(sm_fresh + j * 64 + li * 4);
+      qp[j][0] = v.x; qp[j][1] = v.y; qp[j][2] = v.z; qp[j][3] = v.w;
+    }
+  }
+
+  // the first tile apart from the loop: its rows were asked for above, and the loop then keeps no
+  // K/V registers alive from one pass to the next
+  if (live) {
+    compute(true);
+    for (t += STEP; t < c1; t += STEP) {
+      issue(t, fetch_entry(t));
+      compute(false);
+    }
   }
   if constexpr (FRESH) {
-    if (writer && !wrote) fresh_duties(false);  // a wave without tokens still owes the cache write
+    // One workgroup per KV head writes the new token into the cache, from the copy in LDS and after
+    // the tiles: a store in front of them would have the tiles' first register writes wait for it.
+    // Nobody in this launch reads that slot from memory.
+    if (prep && split == 0 && (QPG > 1 || hrow == (kv_head << p.qpk_shift)) && g == 0) {
+      const uint32_t ns = new_slot > p.max_slot ? p.max_slot : new_slot;
+      char* dst = reinterpret_cast<char*>(const_cast<void*>(p.kv)) + slot_offset(ns) + head_byte_off;
+      *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(sm_knew + li * 4);
+      *reinterpret_cast<u32x4*>(dst + p.v_offset * 2) = *reinterpret_cast<const u32x4*>(sm_vnew + li * 4);
+    }
   }
 
   if constexpr (PROBE) return;
@@ -642,10 +727,12 @@ static bool sparse_shape_supported(int nw, int rows, int qpg = 1) {
   return (qpg == 2 || qpg == 4 || qpg == 8) && (nw == 4 || nw == 8) && rows == 8;
 }
 
+// `wide`: 64-bit row offsets and pages of any size (8 rows per lane only)
 template <typename T>
-static int launch_sparse(const DecodeParams& p, int nw, int rows, bool probe, dim3 grid, hipStream_t st) {
+static int launch_sparse(const DecodeParams& p, int nw, int rows, bool probe, bool wide, dim3 grid,
+                         hipStream_t st) {
 #define TD_SPARSE_CASE(N_, U_)                                                                   \
-  if (nw == N_ && rows == U_) {                                                                  \
+  if (nw == N_ && rows == U_ && !wide) {                                                         \
     if (probe)                                                                                   \
       hipLaunchKernelGGL((sparse_attn_kernel<T, N_, U_, false, true>), grid, dim3(N_ * 64), 0,   \
                          st, p);                                                                 \
@@ -660,28 +747,51 @@ static int launch_sparse(const DecodeParams& p, int nw, int rows, bool probe, di
   TD_SPARSE_CASE(4, 16)
   TD_SPARSE_CASE(8, 16)
 #undef TD_SPARSE_CASE
-  return fail(TD_ERR_UNSUPPORTED, "sparse decode attention: no kernel for %d waves x %d rows", nw, rows);
+#define TD_SPARSE_CASE(N_)                                                                          \
+  if (nw == N_ && rows == 8 && wide) {                                                              \
+    if (probe)                                                                                      \
+      hipLaunchKernelGGL((sparse_attn_kernel<T, N_, 8, false, true, 1, true>), grid, dim3(N_ * 64), \
+                         0, st, p);                                                                 \
+    else if (p.fresh_k)                                                                             \
+      hipLaunchKernelGGL((sparse_attn_kernel<T, N_, 8, true, false, 1, true>), grid, dim3(N_ * 64), \
+                         0, st, p);                                                                 \
+    else                                                                                            \
+      hipLaunchKernelGGL((sparse_attn_kernel<T, N_, 8, false, false, 1, true>), grid,               \
+                         dim3(N_ * 64), 0, st, p);                                                  \
+    return TD_OK;                                                                                   \
+  }
+  TD_SPARSE_CASE(8)
+  TD_SPARSE_CASE(4)
+#undef TD_SPARSE_CASE
+  return fail(TD_ERR_UNSUPPORTED, "sparse decode attention: no kernel for %d waves x %d rows%s", nw, rows,
+              wide ? " with 64-bit offsets" : "");
 }
 
 // shared KV rows: QPG query heads per list walk
 template <typename T>
-static int launch_sparse_shared(const DecodeParams& p, int nw, int qpg, dim3 grid, hipStream_t st) {
-#define TD_SPARSE_CASE(N_, Q_)                                                                  \
-  if (nw == N_ && qpg == Q_) {                                                                  \
-    if (p.fresh_k)                                                                              \
-      hipLaunchKernelGGL((sparse_attn_kernel<T, N_, 8, true, false, Q_>), grid, dim3(N_ * 64),  \
-                         0, st, p);                                                             \
-    else                                                                                        \
-      hipLaunchKernelGGL((sparse_attn_kernel<T, N_, 8, false, false, Q_>), grid, dim3(N_ * 64), \
-                         0, st, p);                                                             \
-    return TD_OK;                                                                               \
+static int launch_sparse_shared(const DecodeParams& p, int nw, int qpg, bool wide, dim3 grid, hipStream_t st) {
+#define TD_SPARSE_CASE(N_, Q_, W_)                                                                  \
+  if (nw == N_ && qpg == Q_ && wide == W_) {                                                        \
+    if (p.fresh_k)                                                                                  \
+      hipLaunchKernelGGL((sparse_attn_kernel<T, N_, 8, true, false, Q_, W_>), grid, dim3(N_ * 64),  \
+                         0, st, p);                                                                 \
+    else                                                                                            \
+      hipLaunchKernelGGL((sparse_attn_kernel<T, N_, 8, false, false, Q_, W_>), grid, dim3(N_ * 64), \
+                         0, st, p);                                                                 \
+    return TD_OK;                                                                                   \
   }
-  TD_SPARSE_CASE(4, 2)
-  TD_SPARSE_CASE(4, 4)
-  TD_SPARSE_CASE(4, 8)
-  TD_SPARSE_CASE(8, 2)
-  TD_SPARSE_CASE(8, 4)
-  TD_SPARSE_CASE(8, 8)
+  TD_SPARSE_CASE(4, 2, false)
+  TD_SPARSE_CASE(4, 4, false)
+  TD_SPARSE_CASE(4, 8, false)
+  TD_SPARSE_CASE(8, 2, false)
+  TD_SPARSE_CASE(8, 4, false)
+  TD_SPARSE_CASE(8, 8, false)
+  TD_SPARSE_CASE(4, 2, true)
+  TD_SPARSE_CASE(4, 4, true)
+  TD_SPARSE_CASE(4, 8, true)
+  TD_SPARSE_CASE(8, 2, true)
+  TD_SPARSE_CASE(8, 4, true)
+  TD_SPARSE_CASE(8, 8, true)
 #undef TD_SPARSE_CASE
   return fail(TD_ERR_UNSUPPORTED,
               "sparse decode attention: no kernel for %d waves with %d query heads per shared row", nw, qpg);
@@ -689,13 +799,13 @@ static int launch_sparse_shared(const DecodeParams& p, int nw, int qpg, dim3 gri
 
 // Launches the sparse-layer kernel (and, when the plan asks for it, the second-launch merge);
 // defined once per element type (and once more for shared KV rows) in sparse_attn_*.hip.
-int launch_sparse_f16(const DecodeParams& p, int nw, int rows, bool probe, bool merge_kernel, dim3 grid,
-                      hipStream_t st);
-int launch_sparse_bf16(const DecodeParams& p, int nw, int rows, bool probe, bool merge_kernel, dim3 grid,
-                       hipStream_t st);
-int launch_sparse_shared_f16(const DecodeParams& p, int nw, int qpg, bool merge_kernel, dim3 grid,
+int launch_sparse_f16(const DecodeParams& p, int nw, int rows, bool probe, bool wide, bool merge_kernel,
+                      dim3 grid, hipStream_t st);
+int launch_sparse_bf16(const DecodeParams& p, int nw, int rows, bool probe, bool wide, bool merge_kernel,
+                       dim3 grid, hipStream_t st);
+int launch_sparse_shared_f16(const DecodeParams& p, int nw, int qpg, bool wide, bool merge_kernel, dim3 grid,
                              hipStream_t st);
-int launch_sparse_shared_bf16(const DecodeParams& p, int nw, int qpg, bool merge_kernel, dim3 grid,
+int launch_sparse_shared_bf16(const DecodeParams& p, int nw, int qpg, bool wide, bool merge_kernel, dim3 grid,
                               hipStream_t st);
 
 }  // namespace tidal

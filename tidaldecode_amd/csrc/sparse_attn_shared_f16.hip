@@ -3,9 +3,9 @@
 #include "sparse_attn.cuh"
 
 namespace tidal {
-int launch_sparse_shared_f16(const DecodeParams& p, int nw, int qpg, bool merge_kernel, dim3 grid,
+int launch_sparse_shared_f16(const DecodeParams& p, int nw, int qpg, bool wide, bool merge_kernel, dim3 grid,
                              hipStream_t st) {
-  const int rc = launch_sparse_shared<F16>(p, nw, qpg, grid, st);
+  const int rc = launch_sparse_shared<F16>(p, nw, qpg, wide, grid, st);
   if (rc == TD_OK && merge_kernel) {
     const dim3 mg(grid.x, grid.z);
     if (qpg == 2) hipLaunchKernelGGL((merge_partials_kernel<F16, 128, 2, 512>), mg, dim3(512), 0, st, p);
