@@ -213,14 +213,10 @@ int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t num_kv_head
  *              three).  Calls served by the streaming kernel (page lists, score output, lists of
  *              more than 16384 entries, head_dim 64 / 256) need a power-of-two page_size and a
  *              pool below 4 GiB for it (TD_ERR_UNSUPPORTED otherwise).
- *   workspace  device scratch of at least plan->workspace_bytes whose first 1 MiB was zero-filled
- *              once before first use: ticket counters, 64 bytes apart, which every call leaves
- *              zero again, so that one workspace serves plans of any shape; behind them (from
- *              byte 983040) words that the library writes once and keeps -- marks of head rows
- *              that one workgroup computes alone and, per hardware queue, the XCC at which the
- *              queue starts dealing out workgroups (csrc/sparse_attn.cuh) -- and that must not
- *              be cleared while launches are in flight.  Calls that share a workspace must be
- *              ordered on one stream.
+ *   workspace  device scratch of at least plan->workspace_bytes whose first 1 MiB (ticket
+ *              counters, 64 bytes apart) was zero-filled once before first use; every call
+ *              leaves them zero again, so one workspace serves plans of any shape.  Calls that
+ *              share a workspace must be ordered on one stream.
  * Replaces BatchDecodeWithPagedKVCachePyTorchWrapper::Forward (bsk_ops.h:104-113,
  * tidal/ops/csrc/approx_attn.cu:68-151), BatchDecodeWithPagedKVCacheKernel
  * (kernels/include/decode/decode_attn.cuh:432-658) including its score output
@@ -236,10 +232,7 @@ int td_decode_attn(const td_paged_kv* kv, const td_index_list* list, const td_de
  * Which kernel family served the calling thread's last successful td_decode_attn call:
  * "short-list" (the sparse layer's kernel: token-slot lists of up to 16384 entries, head_dim 128, no
  * score output), "streaming" (everything else), each with ", 64-bit offsets" for pools of 4 GiB and
- * more or pages that are not a power of two, the first also with ", partials meet in L2" when the
- * split workgroups of a head exchange their partial results inside one XCC's L2 (the device's
- * workgroup placement was probed at planning time and the grid suits it); "none" before the first
- * call.  No counterpart in the
+ * more or pages that are not a power of two; "none" before the first call.  No counterpart in the
  * reference (one kernel there, dispatched by SWITCH_HEAD_DIM,
  * kernels/include/decode/decode_attn.cuh:1150-1154); tests and benchmarks use it to say which code
  * they measured.

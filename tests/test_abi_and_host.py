@@ -251,7 +251,6 @@ def test_split_partials_are_only_touched_through_the_coherent_accessors():
                 continue
             uses += 1
             ok = ("store_coherent(" in code or "load_coherent(" in code
-                  or "store_l2(" in code or "load2(" in code                     # the exchange inside one L2 domain
                   or re.search(r"float\* ws_(o|ml);", code)                       # the field
                   or re.search(r"p\.ws_(o|ml) = reinterpret_cast<float\*>", code)  # host: carve the workspace
                   or re.search(r"float\* dst = p\.ws_o \+", code))               # pointer handed to store_coherent
@@ -260,40 +259,3 @@ def test_split_partials_are_only_touched_through_the_coherent_accessors():
                 following = " ".join(lines[no: no + 4])
                 assert following.count("store_coherent(dst") == 4, f"{path.name}:{no}"
     assert uses >= 10
-
-
-def test_l2_local_exchange_is_fenced_in():
-    """The exchange of split partials through one XCC's L2 (plain stores, a ticket without device
-    scope, loads that only bypass the L1) is valid only among workgroups of one XCC.  The text of
-    the kernel must keep it behind the placement check: the plain accessors appear only in
-    finish_head's `local` branches, and `local` becomes true in exactly one place, the branch
-    taken when the row is not marked, the queue's starting XCC is on record from an earlier launch
-    and the workgroup's own placement agrees with it."""
-    import re
-    from pathlib import Path
-
-    src = (Path(__file__).resolve().parents[1] / "tidaldecode_amd" / "csrc" / "sparse_attn.cuh").read_text()
-    code = "\n".join(line.split("//")[0] for line in src.splitlines())
-    # the plain accessors are defined once and used only inside finish_head
-    fh = code[code.index("void finish_head("):code.index("__global__")]
-    assert code.count("store_l2(") == 1 + fh.count("store_l2(") and fh.count("store_l2(") == 2
-    assert code.count("load_l2(") == 1 + fh.count("load_l2(") and fh.count("load_l2(") == 1
-    # ... and there only under `if (local)`
-    branch = fh[fh.index("if (local) {"):fh.index("} else {")]
-    assert branch.count("store_l2(") == 2 and "__HIP_MEMORY_SCOPE_WORKGROUP" in branch
-    assert "ticket + 1" in branch and "store_coherent" not in branch
-    assert re.search(r"if \(local\)\s+load_l2\(src, a, c\);\s+else\s+load_coherent\(src, a, c\);", fh)
-    # the kernel: one assignment of true, in the last branch of a chain whose earlier branches take
-    # the marked rows, the launches without a record of their queue (or with one of their own
-    # making) and the workgroups whose observed start differs from the recorded one
-    kern = code[code.index("__global__"):]
-    assert kern.count("local = true") == 1 and kern.count("bool local = false") == 1
-    guard = kern[kern.index("if (solo_mark) {"):kern.index("local = true")]
-    assert re.search(r"if \(solo_mark\) \{.*\} else if \(!on_record\) \{.*"
-                     r"\} else if \(\(uint32_t\)rec_start != start \+ 1u\) \{.*\} else \{\s*$", guard, re.S)
-    assert "const bool on_record = rec_start != 0 && (uint32_t)rec_tag != tag;" in kern
-    assert "__builtin_amdgcn_dispatch_ptr()" in kern and "__HIP_MEMORY_SCOPE_AGENT" in guard
-    # no other kernel of the library uses the L2-scope accessors
-    for path in (Path(__file__).resolve().parents[1] / "tidaldecode_amd" / "csrc").glob("*"):
-        if path.suffix in (".cuh", ".hip") and path.name != "sparse_attn.cuh":
-            assert "store_l2(" not in path.read_text() and "load_l2(" not in path.read_text(), path.name

@@ -78,11 +78,6 @@ struct DecodeParams {
   float* ws_ml;     // [batch * H_q * max_splits, 2]
   int32_t* ws_cnt;  // [batch * head rows] ticket counters, ticket_stride words apart
   int32_t ticket_stride;
-  // short-list kernel: exchange of the split partials inside one L2 domain (0: off)
-  int32_t xcc_count;  // XCCs the workgroups of a dispatch are dealt to round-robin (1, 2, 4, 8)
-  int32_t xcc_twist;  // test aid: workgroups 2, 3 (mod 8) take themselves for misplaced
-  int32_t* ws_solo;   // one word per ticket slot: non-zero = computed by one workgroup alone
-  int32_t* ws_queue;  // per hardware queue (128): {starting XCC + 1, tag of the launch that wrote it}
   // the token being decoded (FRESH kernels): un-rotated k, v, its rotary cos/sin and its slot
   const void* fresh_k;
   const void* fresh_v;

@@ -1,8 +1,5 @@
 // Host side of the decode-attention entry points: split planning and argument checks.  The
 // kernels live in decode_attn.cuh and are instantiated in decode_attn_{f16,bf16}.hip.
-#include <cstdlib>
-#include <cstring>
-
 #include "sparse_attn.cuh"
 
 namespace tidal {
@@ -31,15 +28,6 @@ static int64_t align256(int64_t x) { return (x + 255) & ~(int64_t)255; }
 // behind one another at the memory channel (measured: 0.4 us of a 9.7 us launch).
 constexpr int kTicketStride = 16;  // int32 words between counters
 constexpr int64_t kTicketBytes = (int64_t)16384 * kTicketStride * 4;
-// Of the 16384 64-byte slots of that region the first kMaxTickets hold counters (word 0: the
-// device-scope ticket, word 1: the ticket of the exchange inside one L2 domain).  Behind them, on
-// cache lines that are only ever written device-coherently: one word per slot that says "this
-// slot's heads are computed by one workgroup alone", then one 8-byte record per hardware queue
-// (128 of them) with the XCC at which the queue starts dealing out workgroups (see sparse_attn.cuh).
-constexpr int kMaxTickets = 15360;
-constexpr int64_t kSoloFlagsOffset = (int64_t)kMaxTickets * kTicketStride * 4;
-constexpr int64_t kQueueRecordsOffset = kSoloFlagsOffset + (int64_t)kMaxTickets * 4;
-static_assert(kQueueRecordsOffset + 128 * 8 <= kTicketBytes, "marks and queue records fit behind the counters");
 
 // The short-list kernel (sparse_attn.cuh) covers a list in one pass of at most 64 workgroups per
 // head; longer lists go to the streaming kernel, whose waves pipeline several tiles.
@@ -54,101 +42,7 @@ static bool is_pow2(int64_t x) { return x > 0 && (x & (x - 1)) == 0; }
 // loaded; every launch leaves the ticket counters zero again.
 static __device__ __align__(256) unsigned char scratch[TD_STATIC_SCRATCH_BYTES];
 
-// ---------------------------------------------------------------------------------------------
-// Which L2 domain (XCC) a workgroup lands on.  MI300-class parts hand the workgroups of a dispatch
-// to their XCCs round-robin by linear workgroup id; each XCC has an L2 of its own, coherent for the
-// workgroups on it.  When all split workgroups of a head row share an XCC, their partial results
-// can be exchanged through that L2 instead of through memory.  The library does not take the
-// placement for granted: a probe launch per device records the XCC of every workgroup of a small
-// 3-D grid, and the feature is used only if the pattern is periodic in the linear id with a period
-// of 1, 2, 4 or 8 distinct XCCs and the same on a second launch behind a dispatch of odd size.
-// (The XCC at which a dispatch starts depends on the hardware queue: 0 on the null stream, other
-// values on created streams, the same for every dispatch of a queue.)  Every workgroup of the
-// attention kernel checks its own placement before it relies on any of this (sparse_attn.cuh).
-// ---------------------------------------------------------------------------------------------
-__global__ void xcc_probe_kernel(uint32_t* out) {
-  if (threadIdx.x == 0) {
-    const uint32_t lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
-    out[lin] = (uint32_t)__builtin_amdgcn_s_getreg(20 | (3 << 11)) & 15u;  // XCC_ID, bits 3:0
-  }
-}
-
 namespace tidal {
-
-struct XccMap {
-  int count;  // period of the round-robin = distinct XCCs (0: unknown or irregular -- feature off)
-  int twist;  // test aid, see probe_xcc_map
-};
-
-// Probed once per device, outside any stream capture (from td_decode_make_plan).  Any failure, an
-// irregular pattern or TIDAL_XCC_LOCAL=0 in the environment leaves the feature off.
-static XccMap probe_xcc_map() {
-  const XccMap none = {0, 0};
-  const char* env = getenv("TIDAL_XCC_LOCAL");
-  if (env && env[0] == '0') return none;
-  // the probe allocates, launches on a stream of its own and waits for it: legal next to another
-  // stream's capture only in the relaxed capture mode, which this thread takes for the duration
-  hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
-  if (hipThreadExchangeStreamCaptureMode(&mode) != hipSuccess) {
-    (void)hipGetLastError();
-    return XccMap{-1, 0};  // not now: try again at the next plan
-  }
-  const dim3 grid(24, 3, 2);
-  const int n = grid.x * grid.y * grid.z;
-  uint32_t* dev = nullptr;
-  hipStream_t st = nullptr;
-  uint32_t host[2][24 * 3 * 2];
-  bool ok = hipMalloc(&dev, 2 * n * sizeof(uint32_t)) == hipSuccess &&
-            hipStreamCreateWithFlags(&st, hipStreamNonBlocking) == hipSuccess;
-  if (ok) {
-    hipLaunchKernelGGL(xcc_probe_kernel, grid, dim3(64), 0, st, dev);
-    hipLaunchKernelGGL(xcc_probe_kernel, dim3(3), dim3(64), 0, st, dev + n);  // an odd-sized dispatch between
-    hipLaunchKernelGGL(xcc_probe_kernel, grid, dim3(64), 0, st, dev + n);
-    ok = hipMemcpyAsync(host, dev, sizeof(host), hipMemcpyDeviceToHost, st) == hipSuccess &&
-         hipStreamSynchronize(st) == hipSuccess;
-  }
-  if (st) (void)hipStreamDestroy(st);
-  if (dev) (void)hipFree(dev);
-  (void)hipThreadExchangeStreamCaptureMode(&mode);
-  if (!ok) {
-    (void)hipGetLastError();
-    return none;
-  }
-  for (int count : {1, 2, 4, 8}) {
-    bool periodic = true, distinct = true;
-    // workgroup i on XCC (start + i) mod count, both times: what the kernels' placement check assumes
-    for (int i = 0; i < n && periodic; ++i)
-      periodic = host[0][i] == ((host[0][0] + (uint32_t)i) & (uint32_t)(count - 1)) && host[1][i] == host[0][i];
-    for (int a = 0; a < count; ++a)
-      for (int c = a + 1; c < count; ++c) distinct = distinct && host[0][a] != host[0][c];
-    if (periodic && distinct) {
-      // Test aid: TIDAL_XCC_LOCAL=twist makes the workgroups 2 and 3 (mod 8) of every dispatch take
-      // themselves for misplaced, so that a test can follow what the kernels do then without any
-      // workgroup being misplaced.
-      return XccMap{count, env && strcmp(env, "twist") == 0 ? 1 : 0};
-    }
-  }
-  return none;
-}
-
-static XccMap xcc_map(bool may_probe) {
-  constexpr int kMaxDevices = 64;
-  static XccMap maps[kMaxDevices];
-  static int state[kMaxDevices] = {};  // 0: not probed, 1: probed
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
-    (void)hipGetLastError();
-    return XccMap{0, 0};
-  }
-  if (__atomic_load_n(&state[dev], __ATOMIC_ACQUIRE) == 0) {
-    if (!may_probe) return XccMap{0, 0};
-    const XccMap m = probe_xcc_map();
-    if (m.count < 0) return XccMap{0, 0};
-    maps[dev] = m;
-    __atomic_store_n(&state[dev], 1, __ATOMIC_RELEASE);
-  }
-  return maps[dev];
-}
 
 // Device address of `scratch` on the current device.  The array's name is a host-side handle, not
 // a device address: the address is looked up once per device (each device holds its own copy)
@@ -207,7 +101,6 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
     // device the lookup fails and is simply tried again by that entry point.
     void* unused = nullptr;
     (void)static_scratch(&unused);
-    (void)xcc_map(true);  // the same holds for the probe of the device's workgroup placement
   }
 
   // ---- short lists: the sparse-layer kernel -------------------------------------------------------
@@ -258,9 +151,9 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
   if (sparse) {
     if (plan->fused_merge < 0) plan->fused_merge = 1;
     plan->fused_merge = plan->fused_merge ? 1 : 0;
-    TD_REQUIRE((int64_t)batch * n_hrows * qpg <= kMaxTickets,
-               "td_decode_make_plan: batch %d x %d heads exceeds the %d ticket counters", batch,
-               n_hrows * qpg, kMaxTickets);
+    TD_REQUIRE((int64_t)batch * n_hrows * qpg * kTicketStride * 4 <= kTicketBytes,
+               "td_decode_make_plan: batch %d x %d heads exceeds the %lld ticket counters", batch,
+               n_hrows * qpg, (long long)(kTicketBytes / (kTicketStride * 4)));
     const int64_t n_part = (int64_t)batch * n_hrows * qpg * plan->max_splits;
     plan->workspace_bytes = kTicketBytes + align256(n_part * head_dim * 4) + align256(n_part * 2 * 4);
     return TD_OK;
@@ -308,9 +201,9 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
   plan->tile_rows = rows;
   if (plan->fused_merge < 0) plan->fused_merge = 1;
   plan->fused_merge = plan->fused_merge ? 1 : 0;
-  TD_REQUIRE((int64_t)batch * n_hrows <= kMaxTickets,
-             "td_decode_make_plan: batch %d x %d head rows exceeds the %d ticket counters", batch,
-             n_hrows, kMaxTickets);
+  TD_REQUIRE((int64_t)batch * n_hrows * kTicketStride * 4 <= kTicketBytes,
+             "td_decode_make_plan: batch %d x %d head rows exceeds the %lld ticket counters", batch,
+             n_hrows, (long long)(kTicketBytes / (kTicketStride * 4)));
   const int64_t n_part = (int64_t)batch * n_hrows * qpg * max_splits;  // head slots incl. padding
   plan->workspace_bytes = kTicketBytes + align256(n_part * head_dim * 4) + align256(n_part * 2 * 4);
   return TD_OK;
@@ -386,7 +279,7 @@ static int build_params(const td_paged_kv* kv, const td_index_list* list, const 
   const int64_t off_o = kTicketBytes;
   const int64_t off_ml = off_o + align256(n_part * D * 4);
   const int64_t need = off_ml + align256(n_part * 2 * 4);
-  TD_REQUIRE((int64_t)batch * n_hrows <= kMaxTickets,
+  TD_REQUIRE((int64_t)batch * n_hrows * kTicketStride * 4 <= kTicketBytes,
              "td_decode_attn: batch %d x %d head rows exceeds the ticket counters", batch, n_hrows);
   TD_REQUIRE(plan->max_splits <= 64, "td_decode_attn: plan has %d splits (limit 64)",
              plan->max_splits);
@@ -466,20 +359,6 @@ static int build_params(const td_paged_kv* kv, const td_index_list* list, const 
   p.ticket_stride = kTicketStride;
   p.ws_o = reinterpret_cast<float*>(ws ? ws + off_o : nullptr);
   p.ws_ml = reinterpret_cast<float*>(ws ? ws + off_ml : nullptr);
-  // exchange of the split partials inside one L2 domain (short-list kernel only; see sparse_attn.cuh):
-  // every split of a head row has the same linear workgroup id modulo the XCC count when the head
-  // rows, the fastest grid dimension, are a multiple of it
-  p.ws_solo = reinterpret_cast<int32_t*>(ws ? ws + kSoloFlagsOffset : nullptr);
-  p.ws_queue = reinterpret_cast<int32_t*>(ws ? ws + kQueueRecordsOffset : nullptr);
-  p.xcc_count = 0;
-  p.xcc_twist = 0;
-  if (ws && plan->fused_merge && plan->max_splits > 1) {
-    const XccMap m = xcc_map(false);
-    if (m.count > 0 && n_hrows % m.count == 0) {
-      p.xcc_count = m.count;
-      p.xcc_twist = m.twist;
-    }
-  }
 
   return TD_OK;
 }
@@ -525,7 +404,7 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
   const int fits = sparse_kernel_fits(p, plan, list, qpg, D, scores != nullptr);
   if (fits != kSparseNo) {
     const bool wide = fits == kSparseWide;
-    TD_REQUIRE((int64_t)batch * n_hrows * qpg <= kMaxTickets,
+    TD_REQUIRE((int64_t)batch * n_hrows * qpg * kTicketStride * 4 <= kTicketBytes,
                "td_decode_attn: batch %d x %d heads exceeds the ticket counters", batch, n_hrows * qpg);
     if (qpg > 1)
       rc = kv->dtype == TD_F16
@@ -537,10 +416,7 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
       rc = launch_sparse_bf16(p, plan->sparse_waves, plan->sparse_rows, false, wide, merge_kernel, grid, st);
     if (rc != TD_OK) return rc;
     TD_HIP_CHECK(hipGetLastError());
-    static const char* const kNames[2][2] = {
-        {"short-list", "short-list, partials meet in L2"},
-        {"short-list, 64-bit offsets", "short-list, 64-bit offsets, partials meet in L2"}};
-    g_last_kernel = kNames[wide ? 1 : 0][p.xcc_count > 0 ? 1 : 0];
+    g_last_kernel = wide ? "short-list, 64-bit offsets" : "short-list";
     return TD_OK;
   }
   if (fresh && !p.lean)

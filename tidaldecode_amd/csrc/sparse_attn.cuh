@@ -135,99 +135,14 @@ __device__ __forceinline__ void scalar_load4(const int32_t* a0, const int32_t* a
       : "memory");
 }
 
-// The same four words plus the OR of N consecutive words at `af` (N = 1, 2, 4, 8) and the two words
-// at `aq`, one round trip.
-typedef int32_t i32x2 __attribute__((ext_vector_type(2)));
-typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
-typedef int32_t i32x8 __attribute__((ext_vector_type(8)));
-template <int N>
-__device__ __forceinline__ void scalar_load_state(const int32_t* a0, const int32_t* a1, const int32_t* a2,
-                                                  const int32_t* a3, const int32_t* af, const int32_t* aq,
-                                                  int32_t& v0, int32_t& v1, int32_t& v2, int32_t& v3,
-                                                  int32_t& any, int32_t& q0, int32_t& q1) {
-  static_assert(N == 1 || N == 2 || N == 4 || N == 8, "flag words per head row");
-  i32x2 qv;
-#define TD_STATE_LOADS(WIDTH)                                                    \
-  asm volatile("s_load_dword %0, %6, 0x0\n\t"                                    \
-               "s_load_dword %1, %7, 0x0\n\t"                                    \
-               "s_load_dword %2, %8, 0x0\n\t"                                    \
-               "s_load_dword %3, %9, 0x0\n\t"                                    \
-               "s_load_" WIDTH " %4, %10, 0x0\n\t"                               \
-               "s_load_dwordx2 %5, %11, 0x0\n\t"                                 \
-               "s_waitcnt lgkmcnt(0)"                                            \
-               : "=&s"(v0), "=&s"(v1), "=&s"(v2), "=&s"(v3), "=&s"(f), "=&s"(qv) \
-               : "s"(a0), "s"(a1), "s"(a2), "s"(a3), "s"(af), "s"(aq)            \
-               : "memory")
-  if constexpr (N == 1) {
-    int32_t f;
-    TD_STATE_LOADS("dword");
-    any = f;
-  } else if constexpr (N == 2) {
-    i32x2 f;
-    TD_STATE_LOADS("dwordx2");
-    any = f.x | f.y;
-  } else if constexpr (N == 4) {
-    i32x4 f;
-    TD_STATE_LOADS("dwordx4");
-    any = f.x | f.y | f.z | f.w;
-  } else {
-    i32x8 f;
-    TD_STATE_LOADS("dwordx8");
-    any = f[0] | f[1] | f[2] | f[3] | f[4] | f[5] | f[6] | f[7];
-  }
-#undef TD_STATE_LOADS
-  q0 = qv.x;
-  q1 = qv.y;
-}
-
-// 8-byte accesses for partials that are exchanged inside one L2 domain: plain stores (the vector L1
-// writes through to the L2), loads that miss the L1 (sc0)
-__device__ __forceinline__ void store_l2(float* dst, float a, float b) {
-  *reinterpret_cast<f32x2*>(dst) = f32x2{a, b};
-}
-__device__ __forceinline__ void load_l2(const float* src, float& a, float& b) {
-  const uint64_t v = __hip_atomic_load(reinterpret_cast<const uint64_t*>(src), __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_WORKGROUP);
-  a = __builtin_bit_cast(float, (uint32_t)v);
-  b = __builtin_bit_cast(float, (uint32_t)(v >> 32));
-}
-
 // The tail of a head's computation, run by ONE wave that holds the workgroup's partial result of
 // that head (lane: dimensions 2 lane, 2 lane + 1; M, L uniform): write the result if the head was
 // not split, else publish the partial, take the head's ticket and, as the last of the splits to
 // arrive, merge all partials.
-//
-// Two forms of the exchange between the split workgroups of a head:
-//
-// Through memory (local == false).  The partial was stored by this wave alone, with device-scope
-// write-through stores (sc1): such a store is acknowledged -- vmcnt decremented -- only once it
-// has reached memory, the point where all XCDs meet, so after s_waitcnt vmcnt(0) the partial is
-// visible device-wide.  Only then is the ticket taken; the increment is a device-scope atomic
-// performed at memory, so a wave that draws the last ticket knows that every other partial of the
-// head had been acknowledged before its own ticket was even issued.  It reads them with
-// device-scope loads (sc1), which do not hit lines a non-coherent cache level may still hold from
-// earlier launches.  What would break this: a plain (non-sc1) store or load on ws_o / ws_ml, a
-// compiler that moved the ticket above the wait (hence asm volatile with a memory clobber), or
-// partials stored by several waves without a barrier between their waits and the ticket.
-//
-// Through the L2 of one XCC (local == true; the caller has established that every split workgroup
-// of this head runs on the same XCC, see the kernel).  An XCC's L2 is the point of coherence for
-// all of its compute units: the vector L1s write through to it, a store is acknowledged once the
-// L2 has taken it, and atomics are executed there.  The partial is stored with plain stores;
-// after s_waitcnt vmcnt(0) it is in that L2.  The ticket (word 1 of the head's slot; word 0 is the
-// memory-side ticket and is left alone) is incremented by an atomic without device scope, that
-// is by the L2 itself; the wave that draws the last one reads the other partials with loads that
-// bypass its L1 (sc0) and therefore sees what the L2 holds, which is what every other wave's
-// stores had been acknowledged for before their tickets.  No line of the partial arrays can be
-// stale in that L2: it is written back and invalidated at the kernel boundaries, and inside a
-// launch these lines are written only by workgroups of the same XCC.  What would break this: a
-// split workgroup of the head on another XCC (its stores and its ticket would sit in another L2);
-// the kernel therefore never lets such a workgroup take part.
 template <typename T>
 __device__ __forceinline__ void finish_head(const DecodeParams& p, int lane, int n_splits, int split,
                                             int64_t part0, int32_t* ticket, uint32_t* o32,
-                                            float* lse_out, float o0, float o1, float M, float L,
-                                            bool local) {
+                                            float* lse_out, float o0, float o1, float M, float L) {
   constexpr int D = 128;
   if (n_splits == 1) {
     const float inv = L > 0.f ? 1.f / L : 0.f;
@@ -235,34 +150,31 @@ __device__ __forceinline__ void finish_head(const DecodeParams& p, int lane, int
     if (lse_out && lane == 0) *lse_out = L > 0.f ? (M + fast_log2(L)) * kLn2 : -INFINITY;
     return;
   }
+  store_coherent(p.ws_o + (part0 + split) * D + 2 * lane, o0, o1);
+  if (lane == 0) store_coherent(p.ws_ml + (part0 + split) * 2, M, L);
+  if (!p.fused_merge) return;  // a second launch (merge_partials_kernel) reduces the partials
+
+  // Ordering.  The partial was stored by this wave alone, with device-scope write-through stores
+  // (sc1): such a store is acknowledged -- vmcnt decremented -- only once it has reached memory, the
+  // point where all XCDs meet, so after s_waitcnt vmcnt(0) the partial is visible device-wide.
+  // Only then is the ticket taken; the increment is a device-scope atomic performed at memory,
+  // so a wave that draws the last ticket knows that every other partial of the head had been
+  // acknowledged before its own ticket was even issued.  It reads them with device-scope loads
+  // (sc1), which do not hit lines a non-coherent cache level may still hold from earlier
+  // launches.  What would break this: a plain (non-sc1) store or load on ws_o / ws_ml, a compiler
+  // that moved the ticket above the wait (hence asm volatile with a memory clobber), or partials
+  // stored by several waves without a barrier between their waits and the ticket.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   int tk = 0;
-  if (local) {
-    store_l2(p.ws_o + (part0 + split) * D + 2 * lane, o0, o1);
-    if (lane == 0) store_l2(p.ws_ml + (part0 + split) * 2, M, L);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    if (lane == 0)
-      tk = __hip_atomic_fetch_add(ticket + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-  } else {
-    store_coherent(p.ws_o + (part0 + split) * D + 2 * lane, o0, o1);
-    if (lane == 0) store_coherent(p.ws_ml + (part0 + split) * 2, M, L);
-    if (!p.fused_merge) return;  // a second launch (merge_partials_kernel) reduces the partials
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    if (lane == 0) tk = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
+  if (lane == 0) tk = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   tk = __builtin_amdgcn_readfirstlane(tk);
   if (tk != n_splits - 1) return;
 
-  auto load2 = [&](const float* src, float& a, float& c) {
-    if (local)
-      load_l2(src, a, c);
-    else
-      load_coherent(src, a, c);
-  };
   float pm = kNegBig, pl = 0.f;  // (m, l) of split `lane`
   {
     const int sidx = lane < n_splits ? lane : n_splits - 1;
     float a, c;
-    load2(p.ws_ml + (part0 + sidx) * 2, a, c);
+    load_coherent(p.ws_ml + (part0 + sidx) * 2, a, c);
     if (lane < n_splits) { pm = a; pl = c; }
   }
   constexpr int PRE = 16;  // partial loads in flight
@@ -272,7 +184,7 @@ __device__ __forceinline__ void finish_head(const DecodeParams& p, int lane, int
     for (int u = 0; u < PRE; ++u) {
       int sidx = base + u;
       sidx = sidx < n_splits ? sidx : n_splits - 1;
-      load2(p.ws_o + (part0 + sidx) * D + 2 * lane, pa[u], pb[u]);
+      load_coherent(p.ws_o + (part0 + sidx) * D + 2 * lane, pa[u], pb[u]);
     }
   };
   issue(0);
@@ -296,12 +208,7 @@ __device__ __forceinline__ void finish_head(const DecodeParams& p, int lane, int
   const float inv = Lx > 0.f ? 1.f / Lx : 0.f;
   *o32 = pack2<T>(ra * inv, rb * inv);
   if (lse_out && lane == 0) *lse_out = Lx > 0.f ? (Mx + fast_log2(Lx)) * kLn2 : -INFINITY;
-  if (lane == 0) {
-    if (local)
-      __hip_atomic_store(ticket + 1, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    else
-      __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
+  if (lane == 0) __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // QPG query heads per loaded K/V row: 1 (every head row is a query head with its own walk of a
@@ -315,8 +222,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int g = lane >> 4, li = lane & 15;
-  const int hrow = blockIdx.x, b = blockIdx.z;
-  int split = blockIdx.y;
+  const int hrow = blockIdx.x, split = blockIdx.y, b = blockIdx.z;
   // One batch of scalar loads for every kernel argument the main path uses: the compiler would
   // otherwise fetch them where they are first needed, a dependent round trip each time.
 #define TD_TOUCH(x) asm volatile("" ::"s"(x))
@@ -326,7 +232,6 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
   TD_TOUCH(p.chunk_shift); TD_TOUCH(p.max_splits); TD_TOUCH(p.page_shift); TD_TOUCH(p.max_slot);
   TD_TOUCH(p.page_stride_b); TD_TOUCH(p.entry_stride_b); TD_TOUCH(p.head_stride);
   TD_TOUCH(p.last_len); TD_TOUCH(p.last_idx); TD_TOUCH(p.scale_log2); TD_TOUCH(p.num_qo_heads);
-  TD_TOUCH(p.xcc_count); TD_TOUCH(p.xcc_twist); TD_TOUCH(p.ws_solo); TD_TOUCH(p.ws_queue);
   if constexpr (FRESH) {
     TD_TOUCH(p.fresh_k); TD_TOUCH(p.fresh_v); TD_TOUCH(p.fresh_cos); TD_TOUCH(p.fresh_sin);
     TD_TOUCH(p.fresh_slot);
@@ -343,7 +248,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
   // device-resident count says: at most n_list_host columns (which the host has checked against
   // the row stride for a segment that starts at column 0), no further than the segment's end
   // indptr[b + 1], and never beyond the row itself.
-  int t0 = (split * NW + wave) * TILE;
+  const int t0 = (split * NW + wave) * TILE;
   const int idx_row = (QPG > 1 || p.idx_per_kv) ? kv_head : hrow;
   int list_beg = 0, list_end = 0;
   if (p.indptr) scalar_load2(p.indptr + b, p.indptr + b + 1, list_beg, list_end);
@@ -402,27 +307,13 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
   // inside one asm statement, so that no register allocation can read it before it has landed; the
   // list entry, which the row loads wait for anyway, is in flight over the same round trip
   uint32_t new_slot = 0xffffffffu;
-  // first ticket slot of this head row (one slot per query head of the row); when partials may be
-  // exchanged inside one L2 domain: whether any of its slots is marked "one workgroup alone", and
-  // what this workspace has on record about the hardware queue the launch runs on
-  const int64_t slot0 = ((int64_t)b * gridDim.x + hrow) * QPG;
-  int32_t solo_mark = 0, rec_start = 0, rec_tag = 0;
-  uint32_t queue_id = 0;
-  if (p.xcc_count) {
-    // HW_ID: PIPE_ID bits 7:6, QUEUE_ID bits 26:24, ME_ID bits 31:30 -- the same for every wave of a dispatch
-    const uint32_t hw = (uint32_t)__builtin_amdgcn_s_getreg(4 | (31 << 11));
-    queue_id = ((hw >> 30) & 3u) << 5 | ((hw >> 6) & 3u) << 3 | ((hw >> 24) & 7u);
-  }
-  if (FRESH || p.count_arr || p.last_len_arr || p.last_idx_arr || p.xcc_count) {
+  if (FRESH || p.count_arr || p.last_len_arr || p.last_idx_arr) {
     // absent arrays read a dummy word (q is never NULL) and keep the host value
     const int32_t* dummy = reinterpret_cast<const int32_t*>(p.q);
     int32_t cnt, ll, lx, ns;
-    scalar_load_state<QPG>(p.count_arr ? p.count_arr + b : dummy, p.last_len_arr ? p.last_len_arr + b : dummy,
-                           p.last_idx_arr ? p.last_idx_arr + b : dummy, FRESH ? p.fresh_slot + b : dummy,
-                           p.xcc_count ? p.ws_solo + slot0 : dummy,
-                           p.xcc_count ? p.ws_queue + 2 * queue_id : dummy, cnt, ll, lx, ns, solo_mark,
-                           rec_start, rec_tag);
-    if (!p.xcc_count) solo_mark = 0;
+    scalar_load4(p.count_arr ? p.count_arr + b : dummy, p.last_len_arr ? p.last_len_arr + b : dummy,
+                 p.last_idx_arr ? p.last_idx_arr + b : dummy, FRESH ? p.fresh_slot + b : dummy, cnt, ll,
+                 lx, ns);
     if (p.indptr) s.n_list = p.count_arr ? cnt : list_end - list_beg;
     if (p.last_len_arr) s.last_len = ll;
     if (p.last_idx_arr) s.last_idx = lx;
@@ -438,61 +329,6 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
   n_splits = n_splits > p.max_splits ? p.max_splits : n_splits;
   n_splits = n_splits < 1 ? 1 : n_splits;
   if (split >= n_splits) return;  // uniform for the workgroup
-  // ---- where the split partials of this head row meet ---------------------------------------------
-  // The device deals the workgroups of a dispatch to its XCCs round-robin by linear id, starting
-  // at an XCC that depends on the hardware queue the dispatch runs on (the host's probe has found
-  // the round-robin; xcc_count is its period).  With the head rows, the fastest grid dimension, a
-  // multiple of that period all splits of a head row share an XCC, and the partials can meet in
-  // that XCC's L2 (finish_head, local form).  Nothing rests on the probe alone: a workgroup takes
-  // the local form only after it has checked its own placement.
-  //  * start = (own XCC - linear id) mod period is what the workgroup observes of the queue's
-  //    starting XCC.  The workspace keeps, per hardware queue, the start that the first launch on
-  //    that queue observed (one 8-byte record: start + 1 and a tag of the launch that wrote it,
-  //    written once, device-coherently, by that launch's first workgroup).  A launch never acts on
-  //    a record of its own making -- the tag, the address of the launch's dispatch packet in the
-  //    queue's ring, tells -- so every workgroup of a launch reads the same thing: either "nothing
-  //    on record" (then the whole launch exchanges through memory) or the recorded start.
-  //  * A workgroup whose observed start equals the recorded one sits where the round-robin puts
-  //    it; if all splits of a row pass, they share an XCC.
-  //  * A workgroup whose observed start differs is misplaced.  It takes no part in the exchange:
-  //    it computes the whole head row by itself, as if the row had one split, writes the result,
-  //    and marks the row's ticket slots (device-coherent stores to words that are never written in
-  //    any other way).  Its siblings cannot know; they publish partials that nobody merges and
-  //    leave an L2-side ticket that never completes.  From the next launch on -- the mark is read
-  //    at the start of every workgroup -- a marked row is computed by its first workgroup alone
-  //    and the others leave at once, so that ticket is never looked at again, whatever plan or
-  //    grid the slot serves.  A workgroup that sees the mark while siblings of the same launch did
-  //    not (it was set a moment ago) only repeats work: whoever computes a whole row writes the
-  //    same result.
-  bool local = false;
-  if (p.xcc_count && n_splits > 1) {  // uniform
-    const uint32_t lin = (uint32_t)hrow + gridDim.x * ((uint32_t)split + gridDim.y * (uint32_t)b);
-    const uint32_t mine = (uint32_t)__builtin_amdgcn_s_getreg(20 | (3 << 11)) & 15u;  // XCC_ID, bits 3:0
-    uint32_t start = (mine - lin) & (uint32_t)(p.xcc_count - 1);
-    if (p.xcc_twist && ((lin & 7u) >> 1) == 1u) start ^= 1u;  // test aid: workgroups 2, 3 (mod 8) see themselves misplaced
-    const uint32_t tag = (uint32_t)reinterpret_cast<uintptr_t>(__builtin_amdgcn_dispatch_ptr());
-    const bool on_record = rec_start != 0 && (uint32_t)rec_tag != tag;
-    if (solo_mark) {
-      if (split != 0) return;
-    } else if (!on_record) {
-      if (rec_start == 0 && lin == 0 && threadIdx.x == 0)
-        __hip_atomic_store(reinterpret_cast<uint64_t*>(p.ws_queue + 2 * queue_id),
-                           (uint64_t)(start + 1u) | ((uint64_t)tag << 32), __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
-    } else if ((uint32_t)rec_start != start + 1u) {
-      if (threadIdx.x < QPG)
-        __hip_atomic_store(p.ws_solo + slot0 + threadIdx.x, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      solo_mark = 1;
-    } else {
-      local = true;
-    }
-    if (solo_mark) {  // the whole row, alone
-      split = 0;
-      n_splits = 1;
-      t0 = wave * TILE;
-      ent = fetch_entry(t0);
-    }
-  }
   const uint32_t last_base = (uint32_t)s.last_idx * (uint32_t)p.page_size;
 
   const char* kbase = reinterpret_cast<const char*>(p.kv);
@@ -879,8 +715,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
     uint32_t* o32 = reinterpret_cast<uint32_t*>(p.o) + ((int64_t)b * p.num_qo_heads + qh) * (D / 2) + lane;
     float* lse_out = p.lse ? p.lse + (int64_t)b * p.num_qo_heads + qh : nullptr;
     const int64_t part0 = ((int64_t)b * p.vheads + qh) * p.max_splits;
-    int32_t* ticket = p.ws_cnt + (slot0 + j) * p.ticket_stride;
-    finish_head<T>(p, lane, n_splits, split, part0, ticket, o32, lse_out, o0, o1, M, L, local);
+    int32_t* ticket = p.ws_cnt + (((int64_t)b * gridDim.x + hrow) * QPG + j) * p.ticket_stride;
+    finish_head<T>(p, lane, n_splits, split, part0, ticket, o32, lse_out, o0, o1, M, L);
   }
 }
 
