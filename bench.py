@@ -73,6 +73,9 @@ def parse():
     ap.add_argument("--no-real-prompt", action="store_true",
                     help="end-to-end leg: skip the real prompt (prefill of random tokens through "
                          "the decoder, then greedy decoding)")
+    ap.add_argument("--no-sweep-e2e", action="store_true",
+                    help="skip the end-to-end budget x context sweep (Full / Quest-style / TidalDecode)")
+    ap.add_argument("--sweep-e2e-only", action="store_true", help="print only that sweep")
     ap.add_argument("--no-configs", action="store_true",
                     help="skip the legs of benchmark configurations 2 and 4 and the Quest bar")
     ap.add_argument("--extra-only", action="store_true",
@@ -456,6 +459,57 @@ def sweep(args):
     return out
 
 
+def sweep_e2e_leg(args):
+    """The reference's end-to-end evaluation (scripts/bench_efficiency_e2e.sh:1-10 through
+    scripts/bench_textgen.py:41-101; README figure llama_e2e_eval): per-token decode latency of the
+    Llama-2-7B shape for token budgets x context lengths -- full attention, a Quest-style decoder
+    (page estimate, page top-k and page-list attention from layer 2 on) and TidalDecode (selection
+    at layers 0 and 2).  Random bf16 weights, synthetic N(0,1) cache as the reference's harness
+    gets from random input embeddings, one decode step per point captured as a hipGraph and
+    replayed."""
+    import torch
+
+    from tidaldecode_amd.llama import TidalLlama, TidalLlamaConfig
+
+    budgets, ctxs = (32, 128, 512, 2048, 4096), (10240, 32768, 102400)
+    cfg = TidalLlamaConfig.llama2_7b(top_k=max(budgets), sparse_layer_start=0, correction_layer=2,
+                                     select_mode="per_head")
+    model = TidalLlama(cfg, "cuda:0", seed=0)
+    model.tidal_init(page_size=16, max_seq_len=max(ctxs) + 512, page_order_seed=0, with_metadata=True)
+    ctrl = model.iController
+    steps = max(5, args.steps // 5)
+
+    def point(kind, ctx, budget):
+        cfg.attn_type = kind
+        ctrl.set_token_budget(budget)
+        model.tidal_clear()
+        model.synthetic_prefill(ctx)
+        dt, how = model.timed_decode(steps=steps, warmup=2, use_graph=not args.no_graph)
+        return round(dt * 1e3, 4), how
+
+    rows = []
+    for ctx in ctxs:
+        full_ms, how = point("full", ctx, max(budgets))
+        for budget in budgets:
+            tidal_ms, _ = point("tidal", ctx, budget)
+            quest_ms, _ = point("quest", ctx, budget)
+            rows.append({"ctx": ctx, "budget": budget, "full_ms_per_token": full_ms,
+                         "quest_ms_per_token": quest_ms, "tidal_ms_per_token": tidal_ms,
+                         "tidal_speedup_vs_full": round(full_ms / tidal_ms, 3),
+                         "quest_speedup_vs_full": round(full_ms / quest_ms, 3), "launch": how})
+    cfg.attn_type = "tidal"
+    del model
+    torch.cuda.empty_cache()
+    return {"shape": "llama2-7b shape: 32 layers, hidden 4096, 32/32 heads x 128, bf16 random weights, "
+                     "page 16, per-head lists, selection at layers 0 and 2; Quest-style: full attention "
+                     "in layers 0 and 1, page budget = token budget / 16",
+            "rows": rows,
+            "reference_figure": {"hardware": "A100 (README llama_e2e_eval figure, budgets 32..4096)",
+                                 "ms_per_token": {"10240": {"full": 19.2, "quest": [19.4, 21.1], "tidal": [17.0, 17.6]},
+                                                  "32768": {"full": 25.7, "quest": [20.5, 22.1], "tidal": [17.7, 19.0]},
+                                                  "102400": {"full": 45.8, "quest": [24.9, 26.1], "tidal": [21.2, 22.4]}}}}
+
+
 def attention_path_row(args, layers, heads, kv_heads, ctx, top_k, select_mode, sel_layers):
     """Attention path of one decode step for one model shape at one context: the sparse-layer
     launch with its HBM roofline fraction, the whole step, and the same step with full attention in
@@ -527,6 +581,11 @@ def configs_leg(args):
     if not args.no_e2e:
         cfg2["e2e_decode"] = e2e_leg(args, "llama3_8b", [102400], 4096, "group_sum", steps=128,
                                      n_greedy=128)["102400"]
+    # the same shape with one list per query head, the reference's selection rule
+    # (src/tidal_build/modify_llama.py:118: top-k of [1, H, 1, N] logits per query head)
+    per_head = attention_path_row(args, 32, 32, 8, 102400, 4096, "per_head", (0, 13))
+    cfg2["per_query_head_lists"] = {k: per_head[k] for k in (
+        "sparse_layer", "tidal_attention_ms_per_step", "full_attention_ms_per_step", "attention_ratio_vs_full")}
     out["cfg2_llama3_8b_ctx100k_top4096"] = cfg2
     cfg4 = {"shape": "64 layers, 40/40 heads x 128, bf16, page 16, per_head lists, selection at layers 0 and 2",
             "attention_path": [attention_path_row(args, 64, 40, 40, ctx, 2048, "per_head", (0, 2))
@@ -710,6 +769,9 @@ def main():
     use_graph = not args.no_graph
     if args.sweep:
         print(json.dumps(sweep(args)))
+        return
+    if args.sweep_e2e_only:
+        print(json.dumps(sweep_e2e_leg(args)))
         return
     if args.calibrate_copy:
         src = torch.ones(64 << 20, dtype=torch.float32, device="cuda:0")  # 256 MiB
@@ -897,6 +959,8 @@ def main():
     if not args.no_configs and not args.only_sparse:
         line["configs"] = configs_leg(args)
         line["quest_comparison"] = quest_leg(args)
+    if not args.no_e2e and not args.no_sweep_e2e and not args.only_sparse:
+        line["sweep_e2e"] = sweep_e2e_leg(args)
     if not args.no_cpu and not args.only_sparse:
         line["cpu_baseline"] = cpu_baseline(args)
     print(json.dumps(line))

@@ -96,6 +96,34 @@ def test_budget_covering_the_context_equals_dense_attention(cuda, select_mode, u
     assert model.iController.kv_cache.seqlen == 0
 
 
+@pytest.mark.parametrize("head_dim,page", [(64, 16), (128, 8)])
+def test_quest_style_decoder_with_every_page_in_budget_equals_dense_attention(cuda, head_dim, page):
+    """attn_type "quest" (the comparison bar of the reference's end-to-end figure): with a page
+    budget that covers the cache, the chosen pages plus the page being filled are every token, so
+    the decoder must reproduce dense attention; with a small budget it still runs and differs."""
+    from tidaldecode_amd.llama import TidalLlama
+
+    torch.manual_seed(0)
+    cfg = _small(head_dim=head_dim, hidden_size=4 * head_dim)
+    cfg.attn_type = "quest"
+    model = TidalLlama(cfg, cuda, seed=4, init_std=0.05)
+    model.tidal_init(page_size=page, max_seq_len=256, page_order_seed=2, with_metadata=True)
+    ids = torch.randint(0, 1000, (70,), device=cuda)
+    logits = model.prefill(ids)
+    assert _close(logits, _reference_logits(model, ids))
+    seq = ids
+    for _ in range(4):
+        tok = logits.argmax().view(1)
+        seq = torch.cat([seq, tok])
+        logits = model.decode_step(tok)
+        assert _close(logits, _reference_logits(model, seq))
+    model.iController.set_token_budget(2 * page)      # two pages + the one being filled
+    tok = logits.argmax().view(1)
+    few = model.decode_step(tok)
+    assert torch.isfinite(few).all() and not _close(few, _reference_logits(model, torch.cat([seq, tok])), rel=1e-3)
+    model.tidal_clear()
+
+
 def test_sparse_layers_use_the_persisted_lists(cuda):
     """small budget: logits equal a dense evaluation masked with the lists the selection layers
     wrote (layers 2 and 4 reuse the lists of layers 1 and 3)"""

@@ -39,7 +39,10 @@ class TidalLlamaConfig:
     sparse_layer_start: int = 2
     correction_layer: int = 13
     select_mode: str = "per_head"
-    attn_type: str = "tidal"  # "tidal" or "full" (every layer attends to the whole cache)
+    # "tidal", "full" (every layer attends to the whole cache) or "quest" (the comparison bar of the
+    # reference's latency figures: full attention in layers 0 and 1, then per layer a page-score
+    # estimate, the best pages and attention over those pages plus the one being filled)
+    attn_type: str = "tidal"
     dtype: torch.dtype = torch.bfloat16
 
     @staticmethod
@@ -57,6 +60,8 @@ class TidalLlamaConfig:
         return TidalLlamaConfig(64, 5120, 40, 40, 128, 13824, 32000, 1e4, **kw)
 
     def layer_kind(self, layer: int) -> str:
+        if self.attn_type == "quest":
+            return "full" if layer < 2 else "quest"
         if self.attn_type == "full" or layer < self.sparse_layer_start:
             return "full"
         if layer in (self.sparse_layer_start, self.correction_layer):
@@ -102,16 +107,19 @@ class TidalLlama:
         # set by generate_graph: the sequence's step state lives on the device and every launch of
         # a decode step reads it there, so one captured step serves every token
         self._dev = None
+        self._quest = None  # per-step state of the Quest-style steps (begin_decode_step)
 
     # ----- cache lifecycle (tidal/models/llama.py:616-656) -----------------------------------
     def tidal_init(self, page_size: int, max_seq_len: int, token_budget: Optional[int] = None,
-                   page_order_seed=None):
+                   page_order_seed=None, with_metadata: bool = False):
+        """``with_metadata``: also keep the per-page key max / min pool that the Quest-style steps
+        (``attn_type = "quest"``) estimate page scores from."""
         c = self.config
         self.iController = InferenceController(
             c.num_layers, c.num_heads, c.head_dim, page_size,
             c.top_k if token_budget is None else token_budget, max_seq_len, c.dtype, self.device,
             num_kv_heads=c.num_kv_heads, select_mode=c.select_mode, select_scope="all",
-            page_order_seed=page_order_seed)
+            page_order_seed=page_order_seed, with_metadata=with_metadata)
 
     def tidal_clear(self):
         self.iController.clean_states()
@@ -169,6 +177,8 @@ class TidalLlama:
         (what the reference's harness gets from random input embeddings)."""
         ctrl = self.iController
         ctrl.kv_cache.pool.buf.normal_()
+        if ctrl.metadata_cache is not None:
+            ctrl.metadata_cache.pool.buf.normal_()
         ctrl.prepare_metadata(n)
 
     # ----- decode -----------------------------------------------------------------------------
@@ -185,6 +195,37 @@ class TidalLlama:
         self._dst_slot.fill_(page * ctrl.page_size + pos % ctrl.page_size)
         _kernels.rope_table(self._positions, self.config.head_dim, self.config.rope_scale,
                             self.config.rope_theta, self._cos, self._sin)
+        self._quest = None
+        if self.config.attn_type == "quest":
+            if ctrl.metadata_cache is None:
+                raise RuntimeError('attn_type "quest" needs tidal_init(..., with_metadata=True)')
+            n_pages = len(ctrl.kv_cache.indicies)
+            budget = max(1, min(int(ctrl._token_budget) // ctrl.page_size, n_pages - 1))
+            self._quest = dict(
+                pos=pos, budget=budget,
+                page_ids=ctrl.kv_indices_without_last.expand(self.config.num_heads, -1).contiguous(),
+                chosen=torch.zeros((self.config.num_heads, budget), dtype=torch.int32, device=self.device))
+
+    def _attention_quest(self, idx, q, k, v):
+        """One layer of a Quest-style step built from the library's pieces: RoPE and append as
+        launches of their own (the append also updates the page's key bounds), then in layers 0 and 1
+        full attention, later an upper bound of the logits per page (decode_estimate), the best
+        pages (top-k over the bounds) and attention over those pages plus the page being filled.
+        Query heads of a group choose their own pages (one list per query head)."""
+        c, ctrl, qs = self.config, self.iController, self._quest
+        tidal_utils.apply_rope_in_place(q, k, qs["pos"], c.rope_scale, c.rope_theta)
+        tidal_utils.append_kv(k, v, ctrl, idx)
+        kv = ctrl.kv_cache.buf_layer(idx)
+        o = torch.empty_like(q)
+        if idx < 2:
+            ctrl._decode_handler.forward(q, o, kv, ctrl.kv_indices_without_last, None,
+                                         ctrl.kv_cache.last_page_len, ctrl.kv_last_page_idx, None)
+            return o
+        est = tidal_utils.decode_estimate(q, ctrl, idx)
+        _kernels.topk_filtering(est, qs["page_ids"], None, qs["chosen"], ctrl.topk_buf, qs["budget"])
+        ctrl._decode_handler.forward(q, o, kv, qs["chosen"], None, ctrl.kv_cache.last_page_len,
+                                     ctrl.kv_last_page_idx, None, index_kind="pages")
+        return o
 
     def _attention_dev(self, idx, q, k, v):
         """_attention with every per-step quantity (list lengths, last page, slot and position of
@@ -233,6 +274,8 @@ class TidalLlama:
         """attention of one decode step for layer idx; q [1, H, D], k/v [1, H_kv, D] un-rotated"""
         if self._dev is not None:
             return self._attention_dev(idx, q, k, v)
+        if self.config.attn_type == "quest":
+            return self._attention_quest(idx, q, k, v)
         c, ctrl = self.config, self.iController
         fresh = None
         if self.fuse_decode_step and ctrl.fused_step_ok:
