@@ -99,3 +99,71 @@ def test_strip_writes_and_reads_agree(shape):
                 assert idx not in seen, "a cell is stored twice"
                 seen.add(idx)
             assert seen == {i for i, c in written.items() if c[0] < n_waiting}
+
+
+def _plan(batch, hq, hkv, d, rows, items):
+    from tidaldecode_amd._lib import DecodePlan, lib
+
+    p = DecodePlan(0, 0, 0, 0, -1, -1, 0, 0)  # sparse_waves -1: the streaming kernel, as with score output
+    assert lib.td_decode_make_plan(batch, hq, hkv, d, rows, items, p) == 0
+    return p
+
+
+def emitted_tokens(n_items, chunk, max_splits, nw, u, d=128):
+    """Every (token, split, wave, tile of that wave) whose logit the selection-layer kernel stores:
+    the kernel's walk (tile t of the row belongs to split t mod splits, waves take interleaved
+    tiles) followed through the strip (emit_push / emit_flush: first token of the oldest waiting
+    tile, a fixed stride between a wave's tiles) down to the index `i` the store uses."""
+    lpr, tpi, tile, floats, strip_tiles = geometry(d, 1, nw, u)
+    n_splits = max(1, min(max_splits, -(-n_items // chunk)))
+    step = n_splits * nw * tile
+    out = []
+    for split in range(n_splits):
+        for wave in range(nw):
+            waiting, first, n_tile = 0, 0, 0
+            t = (split * nw + wave) * tile
+
+            def flush():
+                for n in range(waiting):
+                    for ltok in range(tile):
+                        i = first + n * step + ltok
+                        if i < n_items:
+                            out.append((i, split, wave, n_tile - waiting + n))
+
+            while t < n_items:
+                if waiting == 0:
+                    first = t
+                waiting += 1
+                n_tile += 1
+                if waiting == strip_tiles:
+                    flush()
+                    waiting = 0
+                t += step
+            flush()
+    return out
+
+
+@pytest.mark.parametrize("n", [1, 15, 16, 17, 1000, 4099, 32769, 33000, 102400])
+@pytest.mark.parametrize("hq,hkv", [(32, 32), (40, 40)])
+def test_every_logit_has_exactly_one_writer(n, hq, hkv):
+    """The selection layer of one sequence of n tokens, one query head per head row (the case of
+    the 33000-token logit observation): with the plan the library makes for it, every token's
+    logit is stored by exactly one (split, wave, tile), none beyond the sequence -- two writers of
+    one cell, say at a split edge or where the forced last page follows the listed pages, would be
+    the one way a cell could receive a second value."""
+    page = 16
+    n_pages = -(-n // page)
+    last_len = n - (n_pages - 1) * page
+    items = (n_pages - 1) * page + last_len   # listed pages, all full, then the forced last page
+    assert items == n
+    p = _plan(1, hq, hkv, 128, 1, items)
+    assert p.sparse_waves == 0 and p.chunk_tokens * p.max_splits >= items
+    stored = emitted_tokens(items, p.chunk_tokens, p.max_splits, p.waves_per_block, p.tile_rows)
+    tokens = sorted(i for i, *_ in stored)
+    assert tokens == list(range(n))
+    # the walk itself: token i of the list is entry i % page of page i // page, the forced last page
+    # taking over exactly where the listed pages end (decode_page.cuh:326-329 of the reference)
+    for i in (0, (n_pages - 1) * page - 1, (n_pages - 1) * page, n - 1):
+        if 0 <= i < n:
+            listed = i // page < n_pages - 1
+            assert listed == (i < (n_pages - 1) * page)
