@@ -363,6 +363,24 @@ int td_topk(const void* values, int32_t values_dtype, int64_t values_stride, int
             void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
+ * td_topk with a per-row upper bound of the scores: row_bound[r] (float, device, or NULL) is a
+ * value that no score of row r exceeds -- for the logits of a selection layer, the row's
+ * log-sum-exp as td_decode_attn writes it; for td_score_reduce's sums, the number of heads summed.
+ * The selection then measures every score from that bound instead of from the row's maximum and
+ * needs no pass to find the maximum: the row is counted while its loads arrive.  Same result as
+ * td_topk, bit for bit.  A NaN or infinite bound is ignored (td_decode_attn's lse is NaN whenever a
+ * logit is NaN or +inf, so such rows take the exact path and NaNs still rank first).  A finite
+ * bound below a score of the row, or above a NaN, gives an unspecified selection (never an access
+ * out of bounds).  No counterpart in the reference.
+ */
+int td_topk_bounded(const void* values, int32_t values_dtype, int64_t values_stride, int32_t rows,
+                    int32_t len, int32_t k, const int32_t* in_idx, int64_t in_idx_stride,
+                    const int32_t* page_table, int64_t page_table_stride, int32_t rows_per_table,
+                    const int32_t* len_arr, int32_t page_size, const float* row_bound,
+                    void* out_values, int32_t* out_idx, int64_t out_stride, void* workspace,
+                    int64_t workspace_bytes, void* stream);
+
+/*
  * Bytes of device scratch for td_topk.  Rows of up to 65536 elements never touch it (one launch,
  * every workgroup of a row selects on the whole row and emits a slice).  A few longer rows are
  * shared between workgroups through it (three launches; about 56 KiB per row); without it (NULL),

@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     raw = ctypes.CDLL(_lib.LIB_PATH)
     for n in names:
         assert hasattr(raw, n), n
-    assert _lib.lib.td_version() == 5
+    assert _lib.lib.td_version() == 6
     assert isinstance(_lib.last_error(), str)
 
 

@@ -28,7 +28,7 @@ def _shared_scratch(cuda, rows):
 
 
 def _gpu_topk(values, k, cuda, in_idx=None, page_table=None, page_size=1, want_vals=True,
-              scratch=False):
+              scratch=False, upper_bound=None):
     from tidaldecode_amd import _kernels
 
     rows = values.shape[0]
@@ -37,7 +37,8 @@ def _gpu_topk(values, k, cuda, in_idx=None, page_table=None, page_size=1, want_v
     _kernels.topk_filtering(values.to(cuda), None if in_idx is None else in_idx.to(cuda), out_val,
                             out_idx, _shared_scratch(cuda, rows) if scratch else None, k,
                             page_table=None if page_table is None else page_table.to(cuda),
-                            page_size=page_size)
+                            page_size=page_size,
+                            upper_bound=None if upper_bound is None else upper_bound.to(cuda))
     torch.cuda.synchronize()
     return out_idx.cpu(), None if out_val is None else out_val.cpu()
 
@@ -56,7 +57,26 @@ def _check(values, k, cuda):
     got2, vals2 = _gpu_topk(values, k, cuda, scratch=True)
     assert torch.equal(got2, got), "cooperative path differs"
     assert torch.equal(torch.nan_to_num(vals2.float(), nan=1e38), torch.nan_to_num(vals.float(), nan=1e38))
+    # with an upper bound per row (the row maximum itself, then looser ones: what a log-sum-exp or
+    # a head count is to the scores); rows that hold a NaN say "no bound", as an lse would
+    for bound in _bounds(values):
+        got3, vals3 = _gpu_topk(values, k, cuda, upper_bound=bound)
+        assert torch.equal(got3, got), "selection from a bound differs"
+        assert torch.equal(torch.nan_to_num(vals3.float(), nan=1e38), torch.nan_to_num(vals.float(), nan=1e38))
     return got
+
+
+def _bounds(values):
+    v = values.float()
+    no_bound = torch.isnan(v).any(dim=1)
+    # (not nan_to_num: it also turns +inf into the largest finite value, which is no bound of +inf)
+    top = torch.where(torch.isnan(v), torch.full_like(v, float("-inf")), v).amax(dim=1)
+    out = []
+    for b in (top, top + 0.37 * top.abs() + 3.0, top + 1e-3 * top.abs(), top.abs() * 64 + 1e-30):
+        b = b.clone()
+        b[no_bound] = float("nan")
+        out.append(b.contiguous())
+    return out
 
 
 @pytest.mark.parametrize("rows,n,k", [(32, 4096, 256), (32, 32768, 2048), (1, 32768, 2048),
@@ -199,6 +219,20 @@ def test_signed_zero_inf_and_nan(cuda):
         _check(v, k, cuda)
 
 
+def test_a_bound_below_the_scores_is_harmless(cuda):
+    """A bound that is none (below some score of its row) makes the selection unspecified, but the
+    call returns and writes nothing but positions of the row: scores above the bound are never
+    counted, and the search gives up when it has covered the whole range without finding k
+    elements (tests/test_topk_level_loop.py restates that rule)."""
+    g = torch.Generator().manual_seed(3)
+    for v, bound, k in ((torch.full((2, 64), float("inf")), 3.4028234663852886e38, 5),
+                        (torch.randn((4, 5000), generator=g), 0.0, 5000),
+                        (torch.randn((4, 5000), generator=g), -5.0, 4999),
+                        (torch.randn((3, 40000), generator=g), 1.0, 2048)):
+        got, _ = _gpu_topk(v, k, cuda, upper_bound=torch.full((v.shape[0],), bound), want_vals=False)
+        assert ((got >= -1) & (got < v.shape[1])).all()
+
+
 def test_closed_forms(cuda):
     g = torch.Generator().manual_seed(11)
     v = torch.randn((32, 5000), generator=g)
@@ -280,10 +314,13 @@ def test_lengths_per_row_group(cuda):
         n_pages = (n + page - 1) // page
         tables = torch.stack([torch.randperm(n_pages + 3, generator=g)[:n_pages] for _ in range(groups)]).int()
         lengths = torch.tensor(lens, dtype=torch.int32, device=cuda)
-        for scratch in (False, True):
+        # a bound of what is ranked: the columns behind a row's length exceed it and do not count
+        ranked_top = torch.stack([v[r, :lens[r // per]].max() for r in range(rows)]).to(cuda)
+        for scratch, bound in ((False, None), (True, None), (False, ranked_top + 0.5)):
             out = torch.full((rows, k), -1, dtype=torch.int32, device=cuda)
             _kernels.topk_filtering(v.to(cuda), None, None, out, _shared_scratch(cuda, rows) if scratch else None,
-                                    k, page_table=tables.to(cuda), page_size=page, lengths=lengths)
+                                    k, page_table=tables.to(cuda), page_size=page, lengths=lengths,
+                                    upper_bound=bound)
             torch.cuda.synchronize()
             out = out.cpu().long()
             for r in range(rows):
@@ -291,8 +328,8 @@ def test_lengths_per_row_group(cuda):
                 kr = min(k, ln)
                 pos = orc.stable_topk(v[r: r + 1, :ln], kr)[0]
                 want = tables[r // per].long()[pos // page] * page + pos % page
-                assert torch.equal(out[r, :kr], want), (n, r, scratch)
-                assert (out[r, kr:] == -1).all(), (n, r, scratch)
+                assert torch.equal(out[r, :kr], want), (n, r, scratch, bound is not None)
+                assert (out[r, kr:] == -1).all(), (n, r, scratch, bound is not None)
     with pytest.raises(RuntimeError, match="lengths"):
         _kernels.topk_filtering(torch.zeros((5, 100), device=cuda), None, None,
                                 torch.zeros((5, 10), dtype=torch.int32, device=cuda), None, 10,

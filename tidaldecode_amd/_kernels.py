@@ -161,7 +161,8 @@ def topk_filtering(estimated_value: torch.Tensor, estimated_indices: Optional[to
                    d_out: Optional[torch.Tensor], indices_out: torch.Tensor,
                    buf: Optional[torch.Tensor], page_budget: int, *,
                    page_table: Optional[torch.Tensor] = None, page_size: int = 1,
-                   lengths: Optional[torch.Tensor] = None) -> None:
+                   lengths: Optional[torch.Tensor] = None,
+                   upper_bound: Optional[torch.Tensor] = None) -> None:
     """bsk_ops.h:34-39 / topk.cu:7-44.  Row-wise top-``page_budget`` of ``estimated_value``
     ``[H, len]``; ``indices_out[h, j]`` is ``estimated_indices[h, p]`` of the selected position
     ``p``.  ``buf`` is scratch, as in the reference (there: RAFT's): a zero-initialised uint8 /
@@ -180,6 +181,9 @@ def topk_filtering(estimated_value: torch.Tensor, estimated_indices: Optional[to
     consecutive rows, the sequences of a batch); fp32 values.  ``lengths`` (int32 device
     ``[groups]``): rows of group g use only their first ``lengths[g]`` columns and select
     ``min(page_budget, lengths[g])`` of them, leaving the rest of their output row untouched.
+    ``upper_bound`` (fp32 device ``[H]``): a value per row that no score of the row exceeds (a
+    selection layer's log-sum-exp, the head count for summed probabilities); same result, without
+    the pass that finds the row maximum.  NaN entries mean "no bound".
     """
     _check_rows(estimated_value, "estimated_value")
     rows, length = estimated_value.shape
@@ -234,11 +238,18 @@ def topk_filtering(estimated_value: torch.Tensor, estimated_indices: Optional[to
         ws_bytes = buf.numel() * buf.element_size()
         if ws_bytes >= topk_workspace_bytes(rows):
             ws_ptr = buf.data_ptr()
-    check(lib.td_topk(estimated_value.data_ptr(),
-                      _dtype_code(estimated_value.dtype, "Top-k filtering"),
-                      estimated_value.stride(0), rows, length, k, in_ptr, in_stride, pt_ptr,
-                      pt_stride, rows_per_table, len_ptr, int(page_size), out_vals, indices_out.data_ptr(), indices_out.stride(0),
-                      ws_ptr, ws_bytes if ws_ptr else 0, _stream()))
+    bound_ptr = None
+    if upper_bound is not None:
+        _check_input(upper_bound, "upper_bound")
+        if upper_bound.dtype != torch.float32 or upper_bound.numel() != rows:
+            raise RuntimeError(f"upper_bound must hold {rows} float32 values")
+        bound_ptr = upper_bound.data_ptr()
+    check(lib.td_topk_bounded(estimated_value.data_ptr(),
+                              _dtype_code(estimated_value.dtype, "Top-k filtering"),
+                              estimated_value.stride(0), rows, length, k, in_ptr, in_stride,
+                              pt_ptr, pt_stride, rows_per_table, len_ptr, int(page_size),
+                              bound_ptr, out_vals, indices_out.data_ptr(), indices_out.stride(0),
+                              ws_ptr, ws_bytes if ws_ptr else 0, _stream()))
 
 
 def topk_workspace_bytes(rows: int) -> int:

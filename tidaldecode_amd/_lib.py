@@ -143,6 +143,12 @@ SIGNATURES = {
          c_int64, c_int32, c_void_p, c_int32, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
          c_void_p],
     ),
+    "td_topk_bounded": (
+        c_int32,
+        [c_void_p, c_int32, c_int64, c_int32, c_int32, c_int32, c_void_p, c_int64, c_void_p,
+         c_int64, c_int32, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
+         c_int64, c_void_p],
+    ),
     "td_topk_workspace_bytes": (c_int64, [c_int32]),
     "td_gather_probe": (
         c_int32,

@@ -9,4 +9,4 @@ char* error_buffer() {
 }  // namespace tidal
 
 extern "C" const char* td_last_error(void) { return tidal::error_buffer(); }
-extern "C" int td_version(void) { return 5; }
+extern "C" int td_version(void) { return 6; }

@@ -41,6 +41,7 @@ struct TopkParams {
   void* out_values;
   int32_t* out_idx;
   int64_t out_stride;
+  const float* row_bound;  // per row: a value no score of the row exceeds (NaN: none known), or null
 };
 
 // physical slot of position i through the page table
@@ -788,124 +789,147 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(const TopkPara
 
   __shared__ SliceLds L;
 
-  // ---- 1. the row's scores as raw fp32 bits; the extremes that fix the mapping to d ---------------
+  // ---- 1. the row's scores as raw fp32 bits; the reference point that fixes the mapping to d -------
+  // d: 0 for the reference point, growing as the scores fall, equal for equal scores (-0 == +0).
+  //   kMixed  the reference is >= +0: d = top - u for the non-negative scores (integer order is
+  //           value order there), top + |u| for the negative ones, top = bits of the reference
+  //   kNeg    the reference is negative (so is every score): d = u - top
+  //   kCanon  a NaN in the row: d = kmax - key with the canonical keys (every NaN the maximum)
+  // The reference is the caller's bound of the row when there is one (the row is then mapped and
+  // counted as its loads arrive), else the row's largest score, found by a pass of its own.
+  enum { kMixed, kNeg, kCanon };
   const __amdgpu_buffer_rsrc_t scores = row_descriptor<T>(vals, len);
+  float bound = __builtin_nanf("");
+  if (p.row_bound) bound = p.row_bound[row];
+  const bool bounded = __builtin_fabsf(bound) < __builtin_inff();  // not for NaN or an infinity
   uint32_t reg[IPT > 0 ? IPT : 1];
-  const uint32_t reg0 = score_bits<T>(scores, 0, 0);  // element 0, which every row has
-  int32_t imax = INT32_MIN;       // largest as signed integers: the largest non-negative score, if any
-  uint32_t umax = 0u, umin = ~0u;  // as unsigned integers: most negative score / smallest non-negative
-  // (only the row's last run has slots past the end; the empty asm keeps the compiler from turning
-  // the scalar branch around that case into selects on every run)
-  auto extremes = [&](int j, uint32_t u) {
-    if ((j + 1) * kTopkThreads > len) {
-      asm volatile("");
-      if (j * kTopkThreads + tid >= len) u = reg0;
-    }
-    imax = (int32_t)u > imax ? (int32_t)u : imax;
-    umax = u > umax ? u : umax;
-    umin = u < umin ? u : umin;
-  };
   if constexpr (IPT > 0) {
 #pragma unroll
     for (int j = 0; j < IPT; ++j) reg[j] = score_bits<T>(scores, tid, j);  // all in flight
   }
-  if constexpr (IPT > 0) {
-#pragma unroll
-    for (int j8 = 0; j8 < IPT; j8 += 8) {
-      if (j8 < nruns) {
-#pragma unroll
-        for (int j = j8; j < j8 + 8; ++j) extremes(j, reg[j]);
-      }
-    }
-  } else {
-    for (int jb = 0; jb < nruns; jb += kStream) {
-      uint32_t uu[kStream];
-#pragma unroll
-      for (int u = 0; u < kStream; ++u) uu[u] = score_bits<T>(scores, tid, jb + u);
-#pragma unroll
-      for (int u = 0; u < kStream; ++u) extremes(jb + u, uu[u]);
-    }
-  }
-  imax = wave_max_i32(imax);
-  umax = (uint32_t)wave_max_i32((int32_t)(umax ^ 0x80000000u)) ^ 0x80000000u;
-  umin = ~((uint32_t)wave_max_i32((int32_t)(~umin ^ 0x80000000u)) ^ 0x80000000u);
-  if (lane == 0) {
-    L.wa[wave] = (uint32_t)imax;
-    L.wb[wave] = umax ^ 0x80000000u;
-    L.wc[wave] = ~umin ^ 0x80000000u;
-  }
-  __syncthreads();
-  imax = wave_max_i32((int32_t)L.wa[lane & 15]);
-  umax = (uint32_t)wave_max_i32((int32_t)L.wb[lane & 15]) ^ 0x80000000u;
-  umin = ~((uint32_t)wave_max_i32((int32_t)L.wc[lane & 15]) ^ 0x80000000u);
-
-  // d: 0 for the row's largest score, growing as the scores fall, equal for equal scores (-0 == +0).
-  //   kMixed  some score is >= +0: d = top - u for the non-negative ones (integer order is value
-  //           order there), top + |u| for the negative ones, top = bits of the largest score
-  //   kNeg    all scores negative: d = u - (bits of the one closest to zero)
-  //   kCanon  a NaN in the row: d = kmax - key with the canonical keys (every NaN the maximum)
-  enum { kMixed, kNeg, kCanon };
   int mode;
   uint32_t top, dmax;
-  if (imax > 0x7f800000 || umax > 0xff800000u) {
-    mode = kCanon;
-    uint32_t kx = 0u, kn = ~0u;
-    auto key_extremes = [&](int j, uint32_t u) {
-      const uint32_t kv = KeyTraits<F32>::key(__builtin_bit_cast(float, u));
-      if (j * kTopkThreads + tid < len) {
-        kx = kv > kx ? kv : kx;
-        kn = kv < kn ? kv : kn;
+  if (bounded) {
+    top = __builtin_bit_cast(uint32_t, bound + 0.f);  // -0 becomes +0
+    if constexpr (!std::is_same<T, F32>::value) {
+      // 16-bit scores may have been rounded up past a bound formed in fp32: one bf16 step of room
+      if ((int32_t)top >= 0) top += 0x10000u;
+      else top = top - 0x10000u >= 0x80000000u ? top - 0x10000u : 0u;
+    }
+    mode = (int32_t)top >= 0 ? kMixed : kNeg;
+    // the largest d a score can have: -inf under a non-negative bound, -inf under a negative one
+    dmax = mode == kMixed ? top + 0x7f800000u : 0xff800000u - top;
+  } else {
+    const uint32_t reg0 = score_bits<T>(scores, 0, 0);  // element 0, which every row has
+    int32_t imax = INT32_MIN;       // largest as signed integers: the largest non-negative score, if any
+    uint32_t umax = 0u, umin = ~0u;  // as unsigned integers: most negative score / smallest non-negative
+    // (only the row's last run has slots past the end; the empty asm keeps the compiler from turning
+    // the scalar branch around that case into selects on every run)
+    auto extremes = [&](int j, uint32_t u) {
+      if ((j + 1) * kTopkThreads > len) {
+        asm volatile("");
+        if (j * kTopkThreads + tid >= len) u = reg0;
       }
+      imax = (int32_t)u > imax ? (int32_t)u : imax;
+      umax = u > umax ? u : umax;
+      umin = u < umin ? u : umin;
     };
     if constexpr (IPT > 0) {
 #pragma unroll
-      for (int j = 0; j < IPT; ++j) key_extremes(j, reg[j]);
+      for (int j8 = 0; j8 < IPT; j8 += 8) {
+        if (j8 < nruns) {
+#pragma unroll
+          for (int j = j8; j < j8 + 8; ++j) extremes(j, reg[j]);
+        }
+      }
     } else {
-      for (int j = 0; j < nruns; ++j) key_extremes(j, score_bits<T>(scores, tid, j));
+      for (int jb = 0; jb < nruns; jb += kStream) {
+        uint32_t uu[kStream];
+#pragma unroll
+        for (int u = 0; u < kStream; ++u) uu[u] = score_bits<T>(scores, tid, jb + u);
+#pragma unroll
+        for (int u = 0; u < kStream; ++u) extremes(jb + u, uu[u]);
+      }
     }
-    kx = (uint32_t)wave_max_i32((int32_t)(kx ^ 0x80000000u));
-    kn = (uint32_t)wave_max_i32((int32_t)(~kn ^ 0x80000000u));
-    __syncthreads();  // wa, wb have been read
+    imax = wave_max_i32(imax);
+    umax = (uint32_t)wave_max_i32((int32_t)(umax ^ 0x80000000u)) ^ 0x80000000u;
+    umin = ~((uint32_t)wave_max_i32((int32_t)(~umin ^ 0x80000000u)) ^ 0x80000000u);
     if (lane == 0) {
-      L.wa[wave] = kx;
-      L.wb[wave] = kn;
+      L.wa[wave] = (uint32_t)imax;
+      L.wb[wave] = umax ^ 0x80000000u;
+      L.wc[wave] = ~umin ^ 0x80000000u;
     }
     __syncthreads();
-    top = (uint32_t)wave_max_i32((int32_t)L.wa[lane & 15]) ^ 0x80000000u;
-    dmax = top - ~((uint32_t)wave_max_i32((int32_t)L.wb[lane & 15]) ^ 0x80000000u);
-  } else if (imax >= 0) {
-    mode = kMixed;
-    top = (uint32_t)imax;
-    dmax = umax >= 0x80000000u ? top + (umax - 0x80000000u) : top - umin;
-  } else {
-    mode = kNeg;
-    top = umin;
-    dmax = umax - umin;
+    imax = wave_max_i32((int32_t)L.wa[lane & 15]);
+    umax = (uint32_t)wave_max_i32((int32_t)L.wb[lane & 15]) ^ 0x80000000u;
+    umin = ~((uint32_t)wave_max_i32((int32_t)L.wc[lane & 15]) ^ 0x80000000u);
+    if (imax > 0x7f800000 || umax > 0xff800000u) {
+      mode = kCanon;
+      uint32_t kx = 0u, kn = ~0u;
+      auto key_extremes = [&](int j, uint32_t u) {
+        const uint32_t kv = KeyTraits<F32>::key(__builtin_bit_cast(float, u));
+        if (j * kTopkThreads + tid < len) {
+          kx = kv > kx ? kv : kx;
+          kn = kv < kn ? kv : kn;
+        }
+      };
+      if constexpr (IPT > 0) {
+#pragma unroll
+        for (int j = 0; j < IPT; ++j) key_extremes(j, reg[j]);
+      } else {
+        for (int j = 0; j < nruns; ++j) key_extremes(j, score_bits<T>(scores, tid, j));
+      }
+      kx = (uint32_t)wave_max_i32((int32_t)(kx ^ 0x80000000u));
+      kn = (uint32_t)wave_max_i32((int32_t)(~kn ^ 0x80000000u));
+      __syncthreads();  // wa, wb have been read
+      if (lane == 0) {
+        L.wa[wave] = kx;
+        L.wb[wave] = kn;
+      }
+      __syncthreads();
+      top = (uint32_t)wave_max_i32((int32_t)L.wa[lane & 15]) ^ 0x80000000u;
+      dmax = top - ~((uint32_t)wave_max_i32((int32_t)L.wb[lane & 15]) ^ 0x80000000u);
+    } else if (imax >= 0) {
+      mode = kMixed;
+      top = (uint32_t)imax;
+      dmax = umax >= 0x80000000u ? top + (umax - 0x80000000u) : top - umin;
+    } else {
+      mode = kNeg;
+      top = umin;
+      dmax = umax - umin;
+    }
   }
-  const uint32_t neg_add = top - 0x80000000u;  // kMixed: d = u + neg_add for u with the sign bit
+  // kMixed: d = u + neg_add for u with the sign bit; kNeg: the same form gives u - top
+  const uint32_t neg_add = mode == kMixed ? top - 0x80000000u : 0u - top;
   auto to_d = [&](uint32_t u) -> uint32_t {
-    if (mode == kMixed) return (int32_t)u >= 0 ? top - u : u + neg_add;
-    if (mode == kNeg) return u - top;
+    if (mode != kCanon) return (int32_t)u >= 0 ? top - u : u + neg_add;
     return top - KeyTraits<F32>::key(__builtin_bit_cast(float, u));
   };
+  // the registers from scores to d (slots past the end of the row: beyond every window)
+  auto map_run = [&](int j) {
+    reg[j] = (int32_t)reg[j] >= 0 ? top - reg[j] : reg[j] + neg_add;
+    if ((j + 1) * kTopkThreads > len) {  // uniform: only the row's last run has slots past the end
+      asm volatile("");
+      reg[j] = j * kTopkThreads + tid < len ? reg[j] : kNoElement;
+    }
+  };
+  bool raw = false;  // the registers still hold scores: the first level maps them as they arrive
   if constexpr (IPT > 0) {
-    if (mode == kMixed) {
+    if (bounded) {
+      raw = true;
+    } else if (mode != kCanon) {
 #pragma unroll
-      for (int j = 0; j < IPT; ++j) reg[j] = (int32_t)reg[j] >= 0 ? top - reg[j] : reg[j] + neg_add;
-    } else if (mode == kNeg) {
-#pragma unroll
-      for (int j = 0; j < IPT; ++j) reg[j] -= top;
+      for (int j = 0; j < IPT; ++j) map_run(j);
     } else {
 #pragma unroll
-      for (int j = 0; j < IPT; ++j)
+      for (int j = 0; j < IPT; ++j) {
         reg[j] = top - KeyTraits<F32>::key(__builtin_bit_cast(float, reg[j]));
-    }
-#pragma unroll
-    for (int j = 0; j < IPT; ++j)
-      if ((j + 1) * kTopkThreads > len) {  // uniform: only the row's last run has slots past the end
-        asm volatile("");
-        reg[j] = j * kTopkThreads + tid < len ? reg[j] : kNoElement;
+        if ((j + 1) * kTopkThreads > len) {
+          asm volatile("");
+          reg[j] = j * kTopkThreads + tid < len ? reg[j] : kNoElement;
+        }
       }
+    }
   }
   // f(j, d of element j * 1024 + tid) for the runs j0 <= j < j1 (j uniform); all = true: every
   // run of the row, without the checks (the runs past the end hold nothing)
@@ -946,10 +970,37 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(const TopkPara
   }
   while (dmax != 0u) {  // (all scores equal: the first k positions, nothing to search)
     const bool found = slice_level(
-        L, [&](auto f) { for_runs(0, nruns, every_run, [&](int, uint32_t d) { f(d); }); }, lo, s, limit,
-        krem, tb,
-        n_in, tid, lane, wave);
+        L,
+        [&](auto f) {
+          if constexpr (IPT > 0) {
+            if (raw) {
+#pragma unroll
+              for (int j8 = 0; j8 < IPT; j8 += 8) {
+                if (j8 < nruns) {
+#pragma unroll
+                  for (int j = j8; j < j8 + 8; ++j) {
+                    map_run(j);
+                    f(reg[j]);
+                  }
+                }
+              }
+              raw = false;
+              return;
+            }
+          }
+          for_runs(0, nruns, every_run, [&](int, uint32_t d) { f(d); });
+        },
+        lo, s, limit, krem, tb, n_in, tid, lane, wave);
     if (!found) {  // the threshold lies beyond the window: the rest of the range, as finely as fits
+      if (limit > dmax - lo) {
+        // The window reached the end of the range and the row still holds fewer than k elements:
+        // the caller's bound lies below some score (such scores wrap to d > dmax and are never
+        // counted).  The selection is unspecified then; take every element, the writes stop at k.
+        lo = kNoElement;
+        krem = 0u;
+        s = 0;
+        break;
+      }
       lo += limit;
       const uint32_t rem = dmax - lo;
       s = nbits(rem) - 13;
@@ -1226,12 +1277,13 @@ __global__ __launch_bounds__(256) void score_reduce_kernel(const float* __restri
 
 using namespace tidal;
 
-extern "C" int td_topk(const void* values, int32_t values_dtype, int64_t values_stride,
-                       int32_t rows, int32_t len, int32_t k, const int32_t* in_idx,
-                       int64_t in_idx_stride, const int32_t* page_table,
-                       int64_t page_table_stride, int32_t rows_per_table,
-                       const int32_t* len_arr, int32_t page_size, void* out_values, int32_t* out_idx, int64_t out_stride, void* workspace,
-                       int64_t workspace_bytes, void* stream) {
+extern "C" int td_topk_bounded(const void* values, int32_t values_dtype, int64_t values_stride,
+                               int32_t rows, int32_t len, int32_t k, const int32_t* in_idx,
+                               int64_t in_idx_stride, const int32_t* page_table,
+                               int64_t page_table_stride, int32_t rows_per_table,
+                               const int32_t* len_arr, int32_t page_size, const float* row_bound,
+                               void* out_values, int32_t* out_idx, int64_t out_stride,
+                               void* workspace, int64_t workspace_bytes, void* stream) {
   TD_REQUIRE(values && out_idx, "td_topk: NULL values or out_idx");
   TD_REQUIRE(rows >= 1, "td_topk: rows %d < 1", rows);
   TD_REQUIRE(len >= 0 && k >= 0, "td_topk: len %d / k %d", len, k);
@@ -1262,6 +1314,7 @@ extern "C" int td_topk(const void* values, int32_t values_dtype, int64_t values_
   p.out_values = out_values;
   p.out_idx = out_idx;
   p.out_stride = out_stride;
+  p.row_bound = row_bound;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   TD_REQUIRE(values_dtype == TD_F32 || values_dtype == TD_F16 || values_dtype == TD_BF16,
              "Top-k filtering failed to dispatch with dtype %d", values_dtype);
@@ -1295,6 +1348,17 @@ extern "C" int td_topk(const void* values, int32_t values_dtype, int64_t values_
   }
   TD_HIP_CHECK(hipGetLastError());
   return TD_OK;
+}
+
+extern "C" int td_topk(const void* values, int32_t values_dtype, int64_t values_stride,
+                       int32_t rows, int32_t len, int32_t k, const int32_t* in_idx,
+                       int64_t in_idx_stride, const int32_t* page_table,
+                       int64_t page_table_stride, int32_t rows_per_table, const int32_t* len_arr,
+                       int32_t page_size, void* out_values, int32_t* out_idx, int64_t out_stride,
+                       void* workspace, int64_t workspace_bytes, void* stream) {
+  return td_topk_bounded(values, values_dtype, values_stride, rows, len, k, in_idx, in_idx_stride,
+                         page_table, page_table_stride, rows_per_table, len_arr, page_size, nullptr,
+                         out_values, out_idx, out_stride, workspace, workspace_bytes, stream);
 }
 
 extern "C" int64_t td_topk_workspace_bytes(int32_t rows) {

@@ -260,14 +260,14 @@ class TidalLlama:
                                      n_list=dev["table"].numel() - 1,
                                      counts=word(_lib.TD_STEP_PAGES_BEFORE_LAST), fresh=fresh)
         if select:
-            scores, n = ctrl.qk_product, dev["final_len"]
+            scores, bound, n = ctrl.qk_product, ctrl.lse.view(-1), dev["final_len"]
             if ctrl.select_mode != "per_head":   # columns past the current length are never ranked
                 _kernels.score_reduce(ctrl.qk_product, ctrl.lse.view(-1), ctrl.num_kv_heads, n,
                                       ctrl.select_mode, out=ctrl.score_sum)
-                scores = ctrl.score_sum
+                scores, bound = ctrl.score_sum, ctrl.score_bound
             _kernels.topk_filtering(scores[:, :n], None, None, dev["lists"], ctrl.topk_buf,
                                     dev["k"], page_table=dev["table"], page_size=ctrl.page_size,
-                                    lengths=word(_lib.TD_STEP_SEQ_LEN))
+                                    lengths=word(_lib.TD_STEP_SEQ_LEN), upper_bound=bound)
         return o
 
     def _attention(self, idx, q, k, v):

@@ -110,13 +110,15 @@ def decode_topk(iController: InferenceController):
     k, n = c.num_selected, c.num_candidates
     if k == 0:
         return
-    scores = c.qk_product
+    # no logit exceeds its head's log-sum-exp, no summed probability the head count
+    scores, bound = c.qk_product, c.lse.view(-1)
     if c.select_mode != "per_head":
         _kernels.score_reduce(c.qk_product, c.lse.view(-1), c.num_kv_heads, n, c.select_mode,
                               out=c.score_sum)
-        scores = c.score_sum
+        scores, bound = c.score_sum, c.score_bound
     _kernels.topk_filtering(scores[:, :n], None, None, c.topk_dindices_buffer, c.topk_buf, k,
-                            page_table=c.kv_indices_with_last, page_size=c.page_size)
+                            page_table=c.kv_indices_with_last, page_size=c.page_size,
+                            upper_bound=bound)
 
 
 def decode_sparse_attn(q: torch.Tensor, iController: InferenceController, layer_idx: int,
@@ -147,5 +149,6 @@ def decode_sparse_attn(q: torch.Tensor, iController: InferenceController, layer_
                                   c.kv_cache.last_page_len if forced else 0,
                                   c.kv_last_page_idx if forced else 0,
                                   c.qk_product if output_qk_product else None, rope_scale,
-                                  rope_theta, index_kind="slots", fresh=fresh)
+                                  rope_theta, index_kind="slots",
+                                  lse=c.lse if output_qk_product else None, fresh=fresh)
     return o

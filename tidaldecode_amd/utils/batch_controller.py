@@ -84,6 +84,10 @@ class BatchInferenceController:
         if select_mode != "per_head":
             self.score_sum = torch.zeros((max_batch * self.index_rows, self.score_cols),
                                          dtype=torch.float32, device=device)
+            # a probability is at most 1: the head count bounds every summed score
+            self.score_bound = torch.full((max_batch * self.index_rows,),
+                                          num_heads // self.index_rows + 1.0,
+                                          dtype=torch.float32, device=device)
         # lists: row r of sequence b lives in columns [b * budget, b * budget + selected[b])
         self.topk_dindices_buffer = torch.zeros((self.index_rows, max_batch * self.budget), **i32)
         self._slots = torch.zeros((max_batch * self.index_rows, self.budget), **i32)
@@ -277,19 +281,19 @@ class BatchInferenceController:
         B, P, k = self.batch, self.page_size, self.budget
         n = max(self._cap)   # an upper bound; every sequence's own length is read on the device
         rows = self.index_rows
-        scores = self.qk_product[: B * self.num_heads]
+        scores, bound = self.qk_product[: B * self.num_heads], self.lse[:B].view(-1)
         if self.select_mode != "per_head":
             # the B * H_q logit rows form B * rows groups of consecutive heads: one grouped sum
             _kernels.score_reduce(scores, self.lse[:B].view(-1), B * rows, n, "group_sum",
                                   out=self.score_sum[: B * rows])
-            scores = self.score_sum[: B * rows]
+            scores, bound = self.score_sum[: B * rows], self.score_bound[: B * rows]
         k_eff = min(k, n)
         # one call: row b * rows + r is row r of sequence b, ranks that sequence's tokens only
         # (its length is read on the device) and goes through that sequence's page table
         out = self._slots[: B * rows, :k_eff]
         _kernels.topk_filtering(scores[:, :n], None, None, out, self.topk_buf, k_eff,
                                 page_table=self.page_table[:B], page_size=P,
-                                lengths=self._row(_SEQ_LEN))
+                                lengths=self._row(_SEQ_LEN), upper_bound=bound)
         self.topk_dindices_buffer.view(rows, self.max_batch, k)[:, :B, :k_eff] = \
             out.view(B, rows, k_eff).permute(1, 0, 2)
 

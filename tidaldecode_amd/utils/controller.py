@@ -85,6 +85,9 @@ class InferenceController:
         if select_mode != "per_head":
             self.score_sum = torch.zeros((self.index_rows, score_cols), dtype=torch.float32,
                                          device=device)
+            # a probability is at most 1: the head count bounds every summed score
+            self.score_bound = torch.full((self.index_rows,), num_heads // self.index_rows + 1.0,
+                                          dtype=torch.float32, device=device)
         self._index_capacity = min(int(token_budget), score_cols)
         self.topk_dindices_buffer_full = torch.zeros((self.index_rows, self._index_capacity),
                                                      dtype=torch.int32, device=device)
