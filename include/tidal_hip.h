@@ -100,7 +100,8 @@ typedef struct {
 
 /*
  * Split plan of one decode-attention call: how many tokens one workgroup covers and how many
- * partial results per head that makes.  Pure host arithmetic (no device access); replaces
+ * partial results per head that makes.  Filled by td_decode_make_plan on the host (no launch, no
+ * allocation, no device memory is read; see there for the two runtime queries it makes); replaces
  * BatchDecodeHandler::BeginForward + BatchDecodeWithPagedKVCacheWorkEstimation +
  * PartitionPagedKVCacheComputeAuxiliaryInfo (kernels/include/decode/decode_handler.cuh:39-175,
  * decode_attn.cuh:687-906; binding tidal/ops/csrc/approx_attn.cu:27-66).
@@ -189,7 +190,12 @@ int td_rope_append_decode(const td_paged_kv* kv, void* q, const void* k, const v
  * sequence attends to; idx_rows as in td_index_list.  chunk_tokens / waves_per_block / tile_rows /
  * sparse_waves / sparse_rows (non-zero) and fused_merge (non-negative) may be preset in *plan to
  * override the heuristics; pass a zero-initialised struct with fused_merge = -1 for defaults.
- * Host arithmetic only.
+ * The plan itself is host arithmetic: no launch, no allocation, no synchronisation.  Two read-only
+ * runtime queries ride along, each made once per process and device: the compute-unit count of
+ * the current device (hipDeviceGetAttribute; 256 is assumed when there is no device) and the
+ * device address of the static scratch of td_decode_attn_noalloc (hipGetSymbolAddress, so that
+ * the entry point that must not allocate finds it resolved; a failure here is ignored and the
+ * lookup is tried again there).  Call it outside stream capture.
  * Replaces BatchDecodeWithPagedKVCacheWorkEstimation and PartitionPagedKVCacheComputeAuxiliaryInfo
  * (kernels/include/decode/decode_attn.cuh:815-906, :687-748), reached through
  * BatchDecodeHandler::BeginForward (decode_handler.cuh:39-121, binding approx_attn.cu:27-62).

@@ -160,7 +160,8 @@ def test_full_attention_with_scores(cuda, dtype, hq, hkv, n):
     scores = torch.full((hq, stride), float("nan"), dtype=torch.float32, device=cuda)
     lse = torch.empty((1, hq), dtype=torch.float32, device=cuda)
     table = case.page_table[:-1].to(torch.int32).unsqueeze(0)
-    w.forward(qd, od, case.pool.to(cuda), table.to(cuda), None, case.last_page_len,
+    pool_d = case.pool.to(cuda)
+    w.forward(qd, od, pool_d, table.to(cuda), None, case.last_page_len,
               int(case.page_table[-1]), scores, lse=lse)
     torch.cuda.synchronize()
     assert tolerance_report(od[0], want) <= ATOL[dtype]
@@ -177,11 +178,19 @@ def test_full_attention_with_scores(cuda, dtype, hq, hkv, n):
         where = (f"split {(i // wg_tokens) % n_splits} of {n_splits}, wave {(i % wg_tokens) // (plan.tile_rows * 4)}, "
                  f"tile {(i // wg_tokens) // n_splits} of that wave, row {i % (plan.tile_rows * 4)} of the tile")
         scores2 = torch.full_like(scores, float("nan"))
-        w.forward(qd, od, case.pool.to(cuda), table.to(cuda), None, case.last_page_len,
+        w.forward(qd, od, pool_d, table.to(cuda), None, case.last_page_len,
                   int(case.page_table[-1]), scores2, lse=lse)
         torch.cuda.synchronize()
+        # which side is off: the logit once more in float64, from the K row of the CPU inputs and
+        # from the K row as it sits in the pool on the GPU
+        kvh = h // (hq // hkv)
+        k_gpu = pool_d[int(case.page_table[i // page_size]), 0, i % page_size, kvh].double().cpu()
+        q64 = q[h].to(dtype).double()
+        ref_cpu = float(q64 @ case.k[i, kvh].double()) / d ** 0.5
+        ref_gpu_row = float(q64 @ k_gpu) / d ** 0.5
         raise AssertionError(f"logit of head {h}, token {i} ({where}): {got_logits[h, i].item()!r}, oracle "
-                             f"{logits[h, i].item()!r}, second launch {scores2[h, i].item()!r}; "
+                             f"{logits[h, i].item()!r}, second launch {scores2[h, i].item()!r}, float64 from "
+                             f"the CPU's K row {ref_cpu!r}, from the K row in the GPU pool {ref_gpu_row!r}; "
                              f"{int((err > bound).sum())} entries beyond {bound:.2e}")
     assert torch.isnan(scores[:, n:]).all()  # nothing written past the sequence
     assert (lse[0].cpu() - torch.logsumexp(logits, -1)).abs().max() <= 1e-3
