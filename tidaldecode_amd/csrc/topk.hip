@@ -743,23 +743,29 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t row_descriptor(const void* row
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(row), 0,
                                            len * (int)sizeof(typename ElemOf<T>::type), 0x00020000);
 }
+// stored_bits: element run * 1024 + tid as it is stored (16-bit types zero-extended); widen: the
+// bits of its fp32 value; score_bits: both at once.  A row kept in registers is kept as stored
+// and widened where it is used, so that it occupies one register per element on every path.
 template <typename T>
-__device__ __forceinline__ uint32_t score_bits(__amdgpu_buffer_rsrc_t row, int tid, int run);
-template <>
-__device__ __forceinline__ uint32_t score_bits<F32>(__amdgpu_buffer_rsrc_t row, int tid, int run) {
-  return __builtin_amdgcn_raw_buffer_load_b32(row, tid * 4, run * (kTopkThreads * 4), 0);
+__device__ __forceinline__ uint32_t stored_bits(__amdgpu_buffer_rsrc_t row, int tid, int run) {
+  if constexpr (std::is_same<T, F32>::value)
+    return __builtin_amdgcn_raw_buffer_load_b32(row, tid * 4, run * (kTopkThreads * 4), 0);
+  else
+    return (uint32_t)(uint16_t)__builtin_amdgcn_raw_buffer_load_b16(row, tid * 2, run * (kTopkThreads * 2), 0);
 }
-template <>
-__device__ __forceinline__ uint32_t score_bits<F16>(__amdgpu_buffer_rsrc_t row, int tid, int run) {
-  return __builtin_bit_cast(
-      uint32_t, to_float<F16>(__builtin_amdgcn_raw_buffer_load_b16(row, tid * 2, run * (kTopkThreads * 2), 0)));
+template <typename T>
+__device__ __forceinline__ uint32_t widen(uint32_t stored) {
+  if constexpr (std::is_same<T, F32>::value)
+    return stored;
+  else
+    return __builtin_bit_cast(uint32_t, to_float<T>((uint16_t)stored));
 }
-template <>
-__device__ __forceinline__ uint32_t score_bits<BF16>(__amdgpu_buffer_rsrc_t row, int tid, int run) {
-  return __builtin_bit_cast(
-      uint32_t, to_float<BF16>(__builtin_amdgcn_raw_buffer_load_b16(row, tid * 2, run * (kTopkThreads * 2), 0)));
+template <typename T>
+__device__ __forceinline__ uint32_t score_bits(__amdgpu_buffer_rsrc_t row, int tid, int run) {
+  return widen<T>(stored_bits<T>(row, tid, run));
 }
 
+constexpr int kRunGroup = 8;              // runs of a register-held row that share one "is there such a run" test
 constexpr int kStream = 16;               // loads in flight per thread where a row is re-read per pass
 constexpr int kOwn = 8;                   // runs of a slice that stay in registers for the emission
 constexpr uint32_t kNoElement = ~0u;      // d of the slots past the end of the row: beyond every window
@@ -805,7 +811,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(const TopkPara
   uint32_t reg[IPT > 0 ? IPT : 1];
   if constexpr (IPT > 0) {
 #pragma unroll
-    for (int j = 0; j < IPT; ++j) reg[j] = score_bits<T>(scores, tid, j);  // all in flight
+    for (int j = 0; j < IPT; ++j) reg[j] = stored_bits<T>(scores, tid, j);  // all in flight
   }
   int mode;
   uint32_t top, dmax;
@@ -836,10 +842,10 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(const TopkPara
     };
     if constexpr (IPT > 0) {
 #pragma unroll
-      for (int j8 = 0; j8 < IPT; j8 += 8) {
+      for (int j8 = 0; j8 < IPT; j8 += kRunGroup) {
         if (j8 < nruns) {
 #pragma unroll
-          for (int j = j8; j < j8 + 8; ++j) extremes(j, reg[j]);
+          for (int j = j8; j < j8 + kRunGroup; ++j) extremes(j, widen<T>(reg[j]));
         }
       }
     } else {
@@ -875,7 +881,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(const TopkPara
       };
       if constexpr (IPT > 0) {
 #pragma unroll
-        for (int j = 0; j < IPT; ++j) key_extremes(j, reg[j]);
+        for (int j = 0; j < IPT; ++j) key_extremes(j, widen<T>(reg[j]));
       } else {
         for (int j = 0; j < nruns; ++j) key_extremes(j, score_bits<T>(scores, tid, j));
       }
@@ -899,47 +905,38 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(const TopkPara
       dmax = umax - umin;
     }
   }
+  // (uniform values: keep them in scalar registers, the rows held in registers need the others)
+  mode = __builtin_amdgcn_readfirstlane(mode);
+  top = __builtin_amdgcn_readfirstlane(top);
+  dmax = __builtin_amdgcn_readfirstlane(dmax);
   // kMixed: d = u + neg_add for u with the sign bit; kNeg: the same form gives u - top
   const uint32_t neg_add = mode == kMixed ? top - 0x80000000u : 0u - top;
   auto to_d = [&](uint32_t u) -> uint32_t {
     if (mode != kCanon) return (int32_t)u >= 0 ? top - u : u + neg_add;
     return top - KeyTraits<F32>::key(__builtin_bit_cast(float, u));
   };
-  // the registers from scores to d (slots past the end of the row: beyond every window)
-  auto map_run = [&](int j) {
-    reg[j] = (int32_t)reg[j] >= 0 ? top - reg[j] : reg[j] + neg_add;
+  // The registers go from scores to d inside the first radix level, run by run as the loads arrive
+  // (slots past the end of the row: beyond every window).  canon: the canonical keys of a NaN row.
+  auto map_run = [&](int j, auto canon) {
+    const uint32_t u = widen<T>(reg[j]);
+    if constexpr (decltype(canon)::value)
+      reg[j] = top - KeyTraits<F32>::key(__builtin_bit_cast(float, u));
+    else
+      reg[j] = (int32_t)u >= 0 ? top - u : u + neg_add;
     if ((j + 1) * kTopkThreads > len) {  // uniform: only the row's last run has slots past the end
       asm volatile("");
       reg[j] = j * kTopkThreads + tid < len ? reg[j] : kNoElement;
     }
   };
-  bool raw = false;  // the registers still hold scores: the first level maps them as they arrive
-  if constexpr (IPT > 0) {
-    if (bounded) {
-      raw = true;
-    } else if (mode != kCanon) {
-#pragma unroll
-      for (int j = 0; j < IPT; ++j) map_run(j);
-    } else {
-#pragma unroll
-      for (int j = 0; j < IPT; ++j) {
-        reg[j] = top - KeyTraits<F32>::key(__builtin_bit_cast(float, reg[j]));
-        if ((j + 1) * kTopkThreads > len) {
-          asm volatile("");
-          reg[j] = j * kTopkThreads + tid < len ? reg[j] : kNoElement;
-        }
-      }
-    }
-  }
   // f(j, d of element j * 1024 + tid) for the runs j0 <= j < j1 (j uniform); all = true: every
   // run of the row, without the checks (the runs past the end hold nothing)
   auto for_runs = [&](int j0, int j1, auto all, auto f) {
     if constexpr (IPT > 0) {
 #pragma unroll
-      for (int j8 = 0; j8 < IPT; j8 += 8) {
+      for (int j8 = 0; j8 < IPT; j8 += kRunGroup) {
         if (j8 < nruns) {  // (rows of a batch can be much shorter than the longest one)
 #pragma unroll
-          for (int j = j8; j < j8 + 8; ++j)
+          for (int j = j8; j < j8 + kRunGroup; ++j)
             if (decltype(all)::value || (j >= j0 && j < j1)) f(j, reg[j]);
         }
       }
@@ -968,29 +965,43 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(const TopkPara
     s = 16;
     limit = (uint32_t)(kSliceBins - 1) << 16;
   }
-  while (dmax != 0u) {  // (all scores equal: the first k positions, nothing to search)
-    const bool found = slice_level(
+  // The first level always runs (a row of one value, dmax == 0, ends it at once: one bin, s == 0)
+  // and is the one place where the registers are written: every later pass only reads them.
+  // (Rows of 56 and 64 runs have no registers to spare for the interleaving: they are mapped in a
+  // pass of their own before the first level, which then only reads, like the others.)
+  constexpr bool kMapInLevel = IPT > 0 && IPT <= 48;
+  if constexpr (IPT > 0 && !kMapInLevel) {
+    if (mode == kCanon) {
+#pragma unroll
+      for (int j = 0; j < IPT; ++j) map_run(j, std::true_type());
+    } else {
+#pragma unroll
+      for (int j = 0; j < IPT; ++j) map_run(j, std::false_type());
+    }
+  }
+  auto first_level = [&](auto canon) {
+    return slice_level(
         L,
         [&](auto f) {
-          if constexpr (IPT > 0) {
-            if (raw) {
+          if constexpr (kMapInLevel) {
 #pragma unroll
-              for (int j8 = 0; j8 < IPT; j8 += 8) {
-                if (j8 < nruns) {
+            for (int j8 = 0; j8 < IPT; j8 += kRunGroup) {
+              if (j8 < nruns) {
 #pragma unroll
-                  for (int j = j8; j < j8 + 8; ++j) {
-                    map_run(j);
-                    f(reg[j]);
-                  }
+                for (int j = j8; j < j8 + kRunGroup; ++j) {
+                  map_run(j, canon);
+                  f(reg[j]);
                 }
               }
-              raw = false;
-              return;
             }
+          } else {
+            for_runs(0, nruns, every_run, [&](int, uint32_t d) { f(d); });
           }
-          for_runs(0, nruns, every_run, [&](int, uint32_t d) { f(d); });
         },
         lo, s, limit, krem, tb, n_in, tid, lane, wave);
+  };
+  bool found = mode == kCanon ? first_level(std::true_type()) : first_level(std::false_type());
+  for (;;) {
     if (!found) {  // the threshold lies beyond the window: the rest of the range, as finely as fits
       if (limit > dmax - lo) {
         // The window reached the end of the range and the row still holds fewer than k elements:
@@ -1006,12 +1017,15 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(const TopkPara
       s = nbits(rem) - 13;
       if (s < 0) s = 0;
       limit = rem + 1u;
-      continue;
+    } else {
+      lo += tb << s;
+      if (s == 0 || n_in <= (uint32_t)kSliceCand) break;
+      limit = 1u << s;  // a crowded bin: its own range, 13 bits further down
+      s = s > 13 ? s - 13 : 0;
     }
-    lo += tb << s;
-    if (s == 0 || n_in <= (uint32_t)kSliceCand) break;
-    limit = 1u << s;  // a crowded bin: its own range, 13 bits further down
-    s = s > 13 ? s - 13 : 0;
+    found = slice_level(
+        L, [&](auto f) { for_runs(0, nruns, every_run, [&](int, uint32_t d) { f(d); }); }, lo, s, limit,
+        krem, tb, n_in, tid, lane, wave);
   }
   // the first runs of the own slice once more, as raw bits (they come from L2 while the members are
   // ranked): the emission works on them with constant register numbers
