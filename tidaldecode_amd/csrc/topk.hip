@@ -1054,34 +1054,26 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(const TopkPara
     });
     __syncthreads();
     if (n_in <= (uint32_t)kSliceRank) {
-      // every member against every other: thread (part, c) compares member c with members
-      // 16 part .. 16 part + 15
-      const int n_parts = ((int)n_in + 15) >> 4;
-      const int c = tid & (kSliceRank - 1), part = tid >> 7;  // part: the same in a wavefront
-      const uint32_t my_d = L.cd[c];
-      const int32_t my_i = L.ci[c];
-      if (part < n_parts) {
-        uint32_t g = 0, e = 0;
-        const uint4* d4 = reinterpret_cast<const uint4*>(L.cd) + part * 4;
-        const int4* i4 = reinterpret_cast<const int4*>(L.ci) + part * 4;
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const uint4 dd = d4[u];
-          const int4 ii = i4[u];
-          g += (dd.x < my_d) + (dd.y < my_d) + (dd.z < my_d) + (dd.w < my_d);
-          e += (dd.x == my_d && ii.x < my_i) + (dd.y == my_d && ii.y < my_i) +
-               (dd.z == my_d && ii.z < my_i) + (dd.w == my_d && ii.w < my_i);
+      // Every member against every other, without another pass through LDS: each wave holds the
+      // whole list in its lanes (members q and q + 64 per lane; the padding ranks behind every
+      // member) and ranks the members c = wave, wave + 16, ...: g = members above c, e = equal
+      // members at lower positions, both by ballot.  The member with g + e = krem - 1 is the last
+      // element taken; exactly one member is, so exactly one wave writes.
+      const uint32_t d0 = L.cd[lane], d1 = L.cd[lane + 64];
+      const int32_t i0 = L.ci[lane], i1 = L.ci[lane + 64];
+      const bool two = n_in > 64u;
+      for (int c = wave; c < (int)n_in; c += kTopkWaves) {
+        const uint32_t dc = (uint32_t)__builtin_amdgcn_readlane((int)(c < 64 ? d0 : d1), c & 63);
+        const int32_t ic = __builtin_amdgcn_readlane(c < 64 ? i0 : i1, c & 63);
+        uint32_t g = (uint32_t)__popcll(__ballot(d0 < dc));
+        uint32_t e = (uint32_t)__popcll(__ballot(d0 == dc && i0 < ic));
+        if (two) {
+          g += (uint32_t)__popcll(__ballot(d1 < dc));
+          e += (uint32_t)__popcll(__ballot(d1 == dc && i1 < ic));
         }
-        L.hist[part * kSliceRank + c] = g | (e << 16);
-      }
-      __syncthreads();
-      if (tid < (int)n_in) {
-        uint32_t t = 0;
-        for (int q = 0; q < n_parts; ++q) t += L.hist[q * kSliceRank + tid];
-        const uint32_t gg = t & 0xffffu, ee = t >> 16;
-        if (gg + ee == krem - 1u) {  // the last element taken: exactly one member
-          L.sh[0] = my_d;
-          L.sh[1] = ee + 1u;
+        if (g + e == krem - 1u && lane == 0) {
+          L.sh[0] = dc;
+          L.sh[1] = e + 1u;
         }
       }
       __syncthreads();
@@ -1126,10 +1118,22 @@ __global__ __launch_bounds__(kTopkThreads) void topk_slice_kernel(const TopkPara
     // the slice's runs from registers; every wave turns the (run, wave) counts into the offsets of
     // its own 64-element pieces by itself: run jj, wave w is entry 16 jj + w, two entries per lane
     uint32_t od[kOwn];
+    if (mode != kCanon) {  // (uniform: one formula per loop, not both and a select per element)
+#pragma unroll
+      for (int jj = 0; jj < kOwn; ++jj) od[jj] = (int32_t)own[jj] >= 0 ? top - own[jj] : own[jj] + neg_add;
+    } else {
+#pragma unroll
+      for (int jj = 0; jj < kOwn; ++jj)
+        od[jj] = top - KeyTraits<F32>::key(__builtin_bit_cast(float, own[jj]));
+    }
 #pragma unroll
     for (int jj = 0; jj < kOwn; ++jj) {
-      const bool in = jj < n_own && (j_lo + jj) * kTopkThreads + tid < len;
-      od[jj] = in ? to_d(own[jj]) : kNoElement;
+      if (jj >= n_own) {  // uniform
+        od[jj] = kNoElement;
+      } else if ((j_lo + jj + 1) * kTopkThreads > len) {  // uniform: the row's last run
+        asm volatile("");
+        od[jj] = (j_lo + jj) * kTopkThreads + tid < len ? od[jj] : kNoElement;
+      }
       const uint32_t ng = (uint32_t)__popcll(__ballot(od[jj] < thr));
       const uint32_t ne = (uint32_t)__popcll(__ballot(od[jj] == thr));
       if (lane == 0) {
