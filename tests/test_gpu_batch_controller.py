@@ -160,6 +160,108 @@ def _lockstep(cuda, hq, hkv, mode, dtype, page, stepping, lens, budget, steps):
     assert ctl.batch == 0 and torch.isinf(ctl.qk_product).all()
 
 
+@pytest.mark.parametrize("hq,hkv,mode,dtype", [(8, 8, "per_head", torch.float16),
+                                              (8, 2, "group_sum", torch.bfloat16)])
+def test_sequences_join_and_leave_between_steps(cuda, hq, hkv, mode, dtype):
+    """Sequences leave (release_sequences: the last ones move into the freed places) and join
+    (add_sequences + append_prompt) between decode steps while the others go on: every active
+    sequence's selection (bit-exact) and attention outputs follow its own oracle history."""
+    from oracle import tidal_oracle as orc
+    from tidaldecode_amd.utils import BatchInferenceController
+
+    d, page, budget, layers, theta = 128, 16, 24, 2, 1e4
+    ctl = BatchInferenceController(layers, hq, d, page, budget, 256, 5, dtype, cuda, num_kv_heads=hkv,
+                                   select_mode=mode, page_order_seed=5)
+    rows = ctl.index_rows
+    seqs = []          # per place: {"id", "k": [per layer], "v": [per layer]}
+
+    def join(ident, n):
+        ctl.add_sequences([n])
+        b = ctl.batch - 1
+        ks = [randn((n, hkv, d), 1000 * ident + l, dtype) for l in range(layers)]
+        vs = [randn((n, hkv, d), 1000 * ident + l + 50, dtype) for l in range(layers)]
+        for l in range(layers):
+            ctl.append_prompt(b, ks[l].to(dtype).to(cuda), vs[l].to(dtype).to(cuda), l)
+        seqs.append({"id": ident, "k": ks, "v": vs})
+
+    def leave(places):
+        moved = ctl.release_sequences(places)
+        keep = [s for i, s in enumerate(seqs) if i not in places]
+        # the controller's promise: untouched sequences keep their index, movers fill the holes
+        after = [None] * ctl.batch
+        for i, s_ in enumerate(seqs):
+            if i in places:
+                continue
+            after[moved.get(i, i)] = s_
+        assert all(a is not None for a in after) and sorted(a["id"] for a in after) == sorted(k_["id"] for k_ in keep)
+        seqs[:] = after
+
+    def step(t):
+        B = ctl.batch
+        ctl.begin_step()
+        cos, sin = ctl.rope_table(1.0, theta)
+        positions = [n - 1 for n in ctl.seq_lens]
+        outs, ins = [], []
+        for l in range(layers):
+            q, k, v = (randn(shape, 7000 * t + 10 * l + i, dtype)
+                       for i, shape in enumerate(((B, hq, d), (B, hkv, d), (B, hkv, d))))
+            ins.append((q, k, v))
+            qd, kd, vd = (x.to(dtype).to(cuda) for x in (q, k, v))
+            if l == 0:
+                outs.append(ctl.attend_full(qd, l, True, fresh=(kd, vd, cos, sin)))
+                ctl.select()
+            else:
+                outs.append(ctl.attend_sparse(qd, l, fresh=(kd, vd, cos, sin)))
+        torch.cuda.synchronize()
+        chosen = []
+        for l in range(layers):
+            q, k, v = ins[l]
+            q_rot, k_rot = _rot(q, positions, dtype, theta), _rot(k, positions, dtype, theta)
+            for b in range(B):
+                s_ = seqs[b]
+                s_["k"][l] = torch.cat([s_["k"][l], k_rot[b: b + 1]])
+                s_["v"][l] = torch.cat([s_["v"][l], v[b: b + 1]])
+                n = ctl.seq_lens[b]
+                assert s_["k"][l].shape[0] == n
+                if l == 0:
+                    logits = orc.attn_logits(q_rot[b], s_["k"][l])
+                    assert tolerance_report(outs[l][b], orc.softmax_pv(logits, s_["v"][l])) <= ATOL[dtype], (t, b)
+                    got_logits = ctl.qk_product[b * hq: (b + 1) * hq, :n].cpu()
+                    scores = got_logits if mode == "per_head" else ctl.score_sum[b * rows: (b + 1) * rows, :n].cpu()
+                    kb = min(budget, n)
+                    pos = orc.stable_topk(scores, kb)
+                    table = torch.tensor(ctl._pages[b])
+                    got = ctl.topk_dindices_buffer[:, b * ctl.budget: b * ctl.budget + kb].cpu().long()
+                    assert torch.equal(got, table[pos // page] * page + pos % page), (t, b, s_["id"])
+                    chosen.append(pos)
+                else:
+                    want = orc.sparse_layer_gather(q_rot[b], s_["k"][l], s_["v"][l], chosen[b])
+                    assert tolerance_report(outs[l][b], want) <= ATOL[dtype], (t, l, b, s_["id"])
+
+    for ident, n in ((0, 40), (1, 7), (2, 90), (3, 33)):
+        join(ident, n)
+    for t in range(3):
+        step(t)
+    free = ctl.pool.num_free_blocks
+    held = len(ctl._pages[1])
+    leave([1])                       # the last sequence (id 3) takes place 1
+    assert [s_["id"] for s_ in seqs] == [0, 3, 2] and ctl.pool.num_free_blocks == free + held
+    for t in range(3, 6):
+        step(t)
+    join(4, 21)                      # a newcomer mid-flight
+    join(5, 1)
+    for t in range(6, 9):
+        step(t)
+    leave([0, 4])                    # two at once, one of them the last: ids 0 and 5
+    assert sorted(s_["id"] for s_ in seqs) == [2, 3, 4]
+    for t in range(9, 12):
+        step(t)
+    with pytest.raises(IndexError):
+        ctl.release_sequences([7])
+    ctl.release_sequences(range(ctl.batch))
+    assert ctl.batch == 0
+
+
 def test_batch_controller_limits(cuda):
     from tidaldecode_amd.utils import BatchInferenceController
 

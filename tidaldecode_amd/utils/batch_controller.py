@@ -152,6 +152,39 @@ class BatchInferenceController:
             raise
         self._refresh()
 
+    def release_sequences(self, which: Sequence[int]) -> dict:
+        """Close the listed sequences between two decode steps and return their pages; the others
+        go on decoding.  The batch stays dense: the last sequences move into the freed places (their
+        page-table rows, persisted lists and host mirrors move with them), every other sequence
+        keeps its index.  Returns ``{old index: new index}`` of the sequences that moved.  New
+        sequences can join at any step boundary with ``add_sequences`` + ``append_prompt``; they
+        get their token lists in the first selection layer of their first step.  A captured step
+        has the batch size baked into its launches: capture it again after the batch changed."""
+        which = sorted(set(int(b) for b in which))
+        if any(b < 0 or b >= self.batch for b in which):
+            raise IndexError(f"no such sequence among {self.batch}: {which}")
+        moved = {}
+        H, rows, k = self.num_heads, self.index_rows, self.budget
+        lists = self.topk_dindices_buffer.view(rows, self.max_batch, k)
+        for b in reversed(which):
+            last = self.batch - 1
+            self.pool.give_back(self._pages[b])
+            if b != last:
+                self.page_table[b].copy_(self.page_table[last])
+                lists[:, b].copy_(lists[:, last])
+                self._pages[b], self.seq_lens[b], self._cap[b] = (self._pages[last], self.seq_lens[last],
+                                                                  self._cap[last])
+                origin = next((o for o, n in moved.items() if n == last), last)
+                moved.pop(origin, None)
+                moved[origin] = b
+            # logits of a closed place are stale: nothing of them may be ranked for its next owner
+            self.qk_product[b * H: (b + 1) * H].fill_(float("-inf"))
+            self.qk_product[last * H: (last + 1) * H].fill_(float("-inf"))
+            self._pages.pop(), self.seq_lens.pop(), self._cap.pop()
+        if self.batch:
+            self._refresh()
+        return moved
+
     def release(self) -> None:
         """Close every sequence and return its pages."""
         for pages in self._pages:
