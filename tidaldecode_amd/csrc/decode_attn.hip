@@ -127,6 +127,16 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
       chunk = 128;
       while (chunk < 512 && (int64_t)n_hrows * batch * ceil_div64(max_items, chunk) > num_cus() * 9 / 8)
         chunk <<= 1;
+      // Between one and 1.75 eight-wave workgroups of 256 tokens per compute unit neither 256 nor
+      // 512 tokens fill the chip evenly (36 heads x 2048 tokens: 288 workgroups, 32 compute units
+      // get a second one; 40 and 48 heads at 512 tokens: 160 and 192 workgroups for 256 compute
+      // units).  Four-wave workgroups of 128 tokens spread better there (measured, 2048 tokens:
+      // 36 heads 13.4 -> 12.0 us, 40 heads 12.95 -> 12.4, 48 heads 13.8 -> 13.2; no gain at 24,
+      // 32, 56 and 64 heads, which keep their plan).
+      const int64_t w256 = (int64_t)n_hrows * batch * ceil_div64(max_items, 256);
+      if (sw == 0 && (sr == 0 || sr == 8) && w256 > num_cus() && w256 * 4 < (int64_t)num_cus() * 7 &&
+          ceil_div64(max_items, 128) <= 64)
+        chunk = 128;
     }
     while (ceil_div64(max_items, chunk) > 64) chunk <<= 1;
     if (sr == 0) sr = 8;
