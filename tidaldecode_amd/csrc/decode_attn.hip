@@ -185,9 +185,16 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
   // tokens one pass of the workgroup covers: waves x instructions x rows per instruction
   const int tile = nw * rows * (64 / (head_dim / 8));
 
-  // Aim at ~2 workgroups per compute unit, never less than one pass per workgroup, never more
-  // than 64 partials per head.
-  const int64_t target_blocks = (int64_t)num_cus() * 2;
+  // Aim at one round of workgroups that fills the chip, never less than one pass per workgroup,
+  // never more than 64 partials per head.  The one-head-per-row kernels fit two 8-wave workgroups
+  // on a compute unit (128 registers: four waves per SIMD), so their round is 2 per compute unit.
+  // The shared-row kernels (141-256 registers) fit ONE: with twice as many workgroups the second
+  // half waits for the first, and a few workgroups over one round double the launch (32/8 heads
+  // x 128 at 100K tokens: 31 splits = 248 workgroups 84 us, 62 splits = 496 workgroups 90 us,
+  // 34 splits = 272 workgroups 120 us; at 32K 33 us against 41, at 10K 18 against 26).  Their
+  // round is kept a little under the compute-unit count: 256 workgroups on 256 compute units
+  // measured like a round and a bit (124 us), 248 and fewer did not.
+  const int64_t target_blocks = qpg > 1 ? (int64_t)num_cus() - num_cus() / 32 : (int64_t)num_cus() * 2;
   int64_t splits = target_blocks / ((int64_t)n_hrows * batch);
   if (splits < 1) splits = 1;
   if (splits > 64) splits = 64;
