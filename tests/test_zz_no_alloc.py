@@ -108,13 +108,14 @@ def test_plans_beyond_the_scratch_are_refused(cuda):
     from tidaldecode_amd import _lib
 
     dtype, h, d, page = torch.float16, 32, 128, 16
-    b, k = 64, 2048                             # 64 x 32 head rows x 4 splits of 520 bytes > 3 MiB of partials
+    b, k = 64, 2048                             # 64 x 32 head rows x 5 splits of 520 bytes > 4 MiB of partials
     pool = torch.zeros((8, 2, page, h, d), dtype=dtype, device=cuda)
     q = torch.zeros((b, h, d), dtype=dtype, device=cuda)
     idx = torch.zeros((h, b * k), dtype=torch.int32, device=cuda)
     indptr = torch.arange(0, (b + 1) * k, k, dtype=torch.int32, device=cuda)
     zeros = torch.zeros(b, dtype=torch.int32, device=cuda)
     _, st = _pair(0, h, h, d, page, dtype)
-    assert st._plan(b, h, k).workspace_bytes > _lib.TD_STATIC_SCRATCH_BYTES
+    st.chunk_tokens = 512                       # (the default plan of this shape is one split per head)
+    assert st._plan(b, h, k + page).workspace_bytes > _lib.TD_STATIC_SCRATCH_BYTES
     with pytest.raises(RuntimeError, match="built-in scratch"):
         st.forward(q, q.clone(), pool, idx, indptr, zeros, zeros, None, index_kind="slots", n_list=k)

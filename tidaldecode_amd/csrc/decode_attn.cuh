@@ -271,9 +271,13 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int g = lane / LPR;   // lane group = token slot inside the instruction
   const int li = lane % LPR;  // 16-byte column of the row
+  // Splits are the slowest grid dimension: a sequence shorter than the planned maximum leaves its
+  // last splits without work, and those workgroups then reach the dispatcher after all the others
+  // instead of between them (where each one that ends at once hands its place to a workgroup that
+  // should have gone to an empty compute unit).
   const int hrow = blockIdx.x;
-  const int split = blockIdx.y;
-  const int b = blockIdx.z;
+  const int b = blockIdx.y;
+  const int split = blockIdx.z;
   const int qh0 = hrow * QPG;  // first head slot of this head row in the split workspace
   int kv_head, rq0, gsz;       // KV head, first query head, query heads that really exist in the row
   head_row_geom<QPG>(p, hrow, kv_head, rq0, gsz);
@@ -927,7 +931,7 @@ static void launch_variant(const DecodeParams& p, bool page_mode, bool emit, boo
       launch_lean<T, D, QPG, NW, U, false, false>(p, grid, st);
   }
   if (merge_kernel)
-    hipLaunchKernelGGL((merge_partials_kernel<T, D, QPG, 512>), dim3(grid.x, grid.z), dim3(512), 0,
+    hipLaunchKernelGGL((merge_partials_kernel<T, D, QPG, 512>), dim3(grid.x, grid.y), dim3(512), 0,
                        st, p);
 }
 

@@ -118,14 +118,20 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
   if (qpg > 1 && sr == 16) sparse = false;  // shared rows: 8 rows per lane only
   if (sparse) {
     // Chunk: the smallest power of two from 128 tokens up that leaves at most 9/8 workgroups per
-    // compute unit, but no more than 512 tokens -- the waves of this kernel do not pipeline their
-    // tiles, so large launches are better served by two workgroups per compute unit than by long
-    // loops (ragged batch of 8 x 32 heads x 1024 tokens: 29 us at 512 tokens per workgroup, 35 us
-    // at 1024).  Workgroup shape: 4 waves for 128-token chunks, 8 waves otherwise, 8 K rows per lane.
+    // compute unit.  Where even 512 tokens leave more than that (batches), the chunk grows on for
+    // as long as a full round of workgroups remains: fewer, longer workgroups then beat more
+    // partials to merge (8 sequences x 32 heads, lists of 1024: 27.0 us at 512 tokens, 25.3 at
+    // 1024; lists of 2048: 50.3 -> 47.5 at 2048; lists of 4096: 94.2 -> 90.4 at 4096; 16 sequences
+    // x 1024: 51.0 -> 49.4; a round that is not full loses: 4 sequences x 1024 at 1024 tokens are
+    // 128 workgroups and 20.3 us against 16.7).  Workgroup shape: 4 waves for 128-token chunks, 8
+    // waves otherwise, 8 K rows per lane.
     int64_t chunk = plan->chunk_tokens;
     if (chunk == 0) {
       chunk = 128;
-      while (chunk < 512 && (int64_t)n_hrows * batch * ceil_div64(max_items, chunk) > num_cus() * 9 / 8)
+      const int64_t rows_all = (int64_t)n_hrows * batch;
+      while (chunk < 512 && rows_all * ceil_div64(max_items, chunk) > num_cus() * 9 / 8) chunk <<= 1;
+      while (rows_all * ceil_div64(max_items, chunk) > num_cus() * 9 / 8 && chunk < max_items &&
+             rows_all * ceil_div64(max_items, chunk * 2) >= num_cus())
         chunk <<= 1;
       // Between one and 1.75 eight-wave workgroups of 256 tokens per compute unit neither 256 nor
       // 512 tokens fill the chip evenly (36 heads x 2048 tokens: 288 workgroups, 32 compute units
@@ -415,7 +421,7 @@ extern "C" int td_decode_attn(const td_paged_kv* kv, const td_index_list* list,
   const int D = kv->head_dim;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const bool page_mode = list->kind == TD_IDX_PAGES;
-  dim3 grid(n_hrows, plan->max_splits, batch);
+  dim3 grid(n_hrows, batch, plan->max_splits);
   const bool merge_kernel = plan->max_splits > 1 && !plan->fused_merge;
   int rc;
   const int fits = sparse_kernel_fits(p, plan, list, qpg, D, scores != nullptr);
@@ -484,7 +490,7 @@ __global__ __launch_bounds__(NW * 64) void gather_probe_kernel(const DecodeParam
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int g = lane / LPR, li = lane % LPR;
-  const int hrow = blockIdx.x, split = blockIdx.y, b = blockIdx.z;
+  const int hrow = blockIdx.x, b = blockIdx.y, split = blockIdx.z;
   const int kv_head = hrow / p.q_per_kv;
   SeqList s;
   int list_beg;
@@ -518,7 +524,7 @@ __global__ __launch_bounds__(NW * 64) void gather_probe_kernel(const DecodeParam
 #pragma unroll
   for (int off = 1; off < 64; off <<= 1) w ^= (uint32_t)__shfl_xor((int)w, off, 64);
   if (lane == 0)
-    out[(((int64_t)b * gridDim.x + hrow) * gridDim.y + split) * NW + wave] = w;
+    out[(((int64_t)b * gridDim.x + hrow) * gridDim.z + split) * NW + wave] = w;
 }
 
 extern "C" int td_gather_probe(const td_paged_kv* kv, const td_index_list* list,
@@ -537,7 +543,7 @@ extern "C" int td_gather_probe(const td_paged_kv* kv, const td_index_list* list,
     TD_REQUIRE(out_bytes >= (int64_t)batch * num_qo_heads * kv->head_dim * 2,
                "td_gather_probe: out holds %lld bytes, %lld needed", (long long)out_bytes,
                (long long)batch * num_qo_heads * kv->head_dim * 2);
-    const dim3 sgrid(n_hrows, plan->max_splits, batch);
+    const dim3 sgrid(n_hrows, batch, plan->max_splits);
     const bool wide = fits == kSparseWide;
     const int src =
         kv->dtype == TD_F16
@@ -557,7 +563,7 @@ extern "C" int td_gather_probe(const td_paged_kv* kv, const td_index_list* list,
   TD_REQUIRE(out_bytes >= (int64_t)batch * n_hrows * plan->max_splits * nw * 4,
              "td_gather_probe: out holds %lld bytes, %lld needed", (long long)out_bytes,
              (long long)batch * n_hrows * plan->max_splits * nw * 4);
-  const dim3 grid(n_hrows, plan->max_splits, batch);
+  const dim3 grid(n_hrows, batch, plan->max_splits);
   uint32_t* outw = reinterpret_cast<uint32_t*>(out);
   if (nw == 16)
     hipLaunchKernelGGL((gather_probe_kernel<128, 4, 16>), grid, dim3(1024), 0, st, p, outw);

@@ -222,7 +222,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(1, U ==
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int g = lane >> 4, li = lane & 15;
-  const int hrow = blockIdx.x, split = blockIdx.y, b = blockIdx.z;
+  const int hrow = blockIdx.x, b = blockIdx.y, split = blockIdx.z;
   // One batch of scalar loads for every kernel argument the main path uses: the compiler would
   // otherwise fetch them where they are first needed, a dependent round trip each time.
 #define TD_TOUCH(x) asm volatile("" ::"s"(x))

@@ -7,7 +7,7 @@ int launch_sparse_shared_f16(const DecodeParams& p, int nw, int qpg, bool wide, 
                              hipStream_t st) {
   const int rc = launch_sparse_shared<F16>(p, nw, qpg, wide, grid, st);
   if (rc == TD_OK && merge_kernel) {
-    const dim3 mg(grid.x, grid.z);
+    const dim3 mg(grid.x, grid.y);
     if (qpg == 2) hipLaunchKernelGGL((merge_partials_kernel<F16, 128, 2, 512>), mg, dim3(512), 0, st, p);
     if (qpg == 4) hipLaunchKernelGGL((merge_partials_kernel<F16, 128, 4, 512>), mg, dim3(512), 0, st, p);
     if (qpg == 8) hipLaunchKernelGGL((merge_partials_kernel<F16, 128, 8, 512>), mg, dim3(512), 0, st, p);
