@@ -208,7 +208,29 @@ extern "C" int td_decode_make_plan(int32_t batch, int32_t num_qo_heads, int32_t 
   // A batch is planned from its longest sequence: chunks of that size leave the short sequences
   // with one long-running workgroup per head and the launch waits for the longest.  Finer chunks
   // balance a ragged batch (8 sequences of 14K-63K tokens: 935 -> 769 us).
-  if (batch > 1 && chunk > 4096) chunk = 4096;
+  if (batch > 1 && qpg == 1 && chunk > 4096) chunk = 4096;
+  // Shared rows in a batch: whole rounds of one workgroup per compute unit.  The split count with
+  // the fewest rounds per split wins, chunks of 1024 tokens at least
+  // (32/8 heads, 16 sequences x 8192 tokens: 2 splits = 256 workgroups 94 us, 3 splits 110, 1
+  // split 130; 8 x 32768: 4 splits 172 us, 3 splits 187, 8 splits of 4096 tokens 182; 12 x 16384:
+  // 5 splits = 2 rounds 136 us, 8 splits = 3 rounds 136, 4 splits 151, 3 splits 187).
+  if (batch > 1 && qpg > 1 && max_items > 0) {
+    const int64_t r = (int64_t)n_hrows * batch, cus = num_cus();
+    int64_t s_max = max_items / 1024;
+    s_max = s_max < 1 ? 1 : (s_max > 64 ? 64 : s_max);
+    int64_t best_s = 1, best_rounds = ceil_div64(r, cus);
+    for (int64_t s_try = 2; s_try <= s_max; ++s_try) {
+      const int64_t rounds = ceil_div64(r * s_try, cus);
+      // more splits in as many rounds always gain; more rounds have to gain 1/16 per split
+      const bool better = rounds <= best_rounds ? rounds * best_s < best_rounds * s_try
+                                                : rounds * best_s * 16 < best_rounds * s_try * 15;
+      if (better) {
+        best_s = s_try;
+        best_rounds = rounds;
+      }
+    }
+    chunk = ceil_div64(max_items, best_s);
+  }
   if (plan->chunk_tokens > 0) chunk = plan->chunk_tokens;
   chunk = ceil_div64(chunk, tile) * tile;
   int64_t max_splits = max_items > 0 ? ceil_div64(max_items, chunk) : 1;
