@@ -196,15 +196,18 @@ def test_full_attention_with_scores(cuda, dtype, hq, hkv, n):
     assert (lse[0].cpu() - torch.logsumexp(logits, -1)).abs().max() <= 1e-3
 
 
-def test_batch_ragged_slots(cuda):
+@pytest.mark.parametrize("k_max", [300, 1800])
+def test_batch_ragged_slots(cuda, k_max):
     """Batch of 8 sequences with different lengths sharing one pool; per-head slot lists with
-    per-sequence counts through indptr."""
+    per-sequence counts through indptr.  Lists of up to 1800 entries are planned as one workgroup of
+    2048 tokens per head and sequence, the short ones as four-wave workgroups of 128."""
     from oracle import tidal_oracle as orc
 
     dtype, h, d, page_size = torch.float16, 32, 128, 16
     g = torch.Generator().manual_seed(0)
     lens = torch.randint(300, 5000, (8,), generator=g).tolist()
-    ks = [int(x) for x in torch.randint(1, 300, (8,), generator=g)]
+    ks = [min(int(x), n) for x, n in zip(torch.randint(1, k_max, (8,), generator=g), lens)]
+    ks[3] = min(k_max, lens[3])
     total_pages = sum((n + page_size - 1) // page_size for n in lens) + 5
     perm = torch.randperm(total_pages, generator=g)
     pool = torch.full((total_pages, 2, page_size, h, d), 55.0)
@@ -236,15 +239,19 @@ def test_batch_ragged_slots(cuda):
         assert tolerance_report(od[b], wants[b]) <= ATOL[dtype], b
 
 
-@pytest.mark.parametrize("hq,hkv,page_size,dtype", [(8, 2, 16, torch.float16), (4, 4, 16, torch.bfloat16),
-                                                    (8, 8, 5, torch.float16), (16, 2, 8, torch.bfloat16)])
-def test_batch_ragged_page_lists_with_logits(cuda, hq, hkv, page_size, dtype):
+@pytest.mark.parametrize("hq,hkv,page_size,dtype,lens", [
+    (8, 2, 16, torch.float16, None), (4, 4, 16, torch.bfloat16, None), (8, 8, 5, torch.float16, None),
+    (16, 2, 8, torch.bfloat16, None),
+    # several splits for the long sequences, workgroups without work for the short ones
+    (32, 8, 16, torch.float16, [9000, 37, 4100, 2500, 1]),
+    (16, 16, 16, torch.bfloat16, [700, 9100, 16, 5000, 3000])])
+def test_batch_ragged_page_lists_with_logits(cuda, hq, hkv, page_size, dtype, lens):
     """Selection-layer mode for a batch: every sequence's page table in order through indptr, its
     own last page and last-page length, logits and log-sum-exp per sequence and head."""
     from oracle import tidal_oracle as orc
 
     d = 128
-    lens = [37, 1000, page_size, 333, 1]
+    lens = lens or [37, 1000, page_size, 333, 1]
     b = len(lens)
     cases = [PagedCase(n, hkv, d, page_size, dtype, seed=60 + i, spare=2) for i, n in enumerate(lens)]
     offs = np.cumsum([0] + [c.max_pages for c in cases])
