@@ -492,7 +492,14 @@ __global__ __launch_bounds__(NW * 64) void decode_attn_kernel(const DecodeParams
   // holds back the wait for every younger K/V or list load until its write is acknowledged.  The
   // logits are therefore collected in a per-wave LDS strip and written EMIT_TILES tiles at a
   // time: the stores enter the memory queue once per batch (once per launch for most shapes).
-  constexpr int EMIT_FLOATS = EMIT ? (NW == 16 ? 512 : 1024) : 1;  // per wave
+  // The later the better: what the writes cost is their HBM traffic in the middle of the read
+  // stream (8 sequences x 32 heads x 32K tokens: 33.5 MB of logits beside 4.3 GB of K/V add 87 us to
+  // 665; the same stores aimed at one 16 KB window add 5; write-through, non-temporal or
+  // contiguous stores change nothing), and a workgroup that writes once, at its end, writes when
+  // the others of its round do.  The shared-row kernels have the LDS for that (one workgroup per
+  // compute unit): 12 KB per wave hold the 4 x 3328 logits of a 100K-token plan (32/8 heads at
+  // 100K tokens: 86 -> 80.6 us with 12 KB per wave instead of 4; 8 x 32K: 214 -> 204).
+  constexpr int EMIT_FLOATS = EMIT ? (NW == 16 ? 512 : (QPG > 1 ? 3072 : 1024)) : 1;  // per wave
   constexpr int EMIT_TILES = EMIT ? EMIT_FLOATS / (QPG * TILE) : 1;
   static_assert(EMIT_TILES >= 1, "logit strip too small for one tile");
   __shared__ float emit_buf[EMIT ? NW * EMIT_FLOATS : 1];
