@@ -27,7 +27,7 @@ def geometry(d, qpg, nw, u):
     lpr = d // 8
     tpi = 64 // lpr
     tile = u * tpi
-    floats = 512 if nw == 16 else 1024
+    floats = 512 if nw == 16 else (3072 if qpg > 1 else 1024)   # EMIT_FLOATS of decode_attn.cuh
     tiles = floats // (qpg * tile)
     return lpr, tpi, tile, floats, tiles
 
