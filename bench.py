@@ -27,7 +27,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # HBM bytes one sparse-layer launch of the default workload moves, from rocprofv3 FETCH_SIZE /
 # WRITE_SIZE scaled by a plain 256 MiB copy (profiles/sparse_attn_kernel_llama2-7b_ctx32k_top2048.md):
 # (16621.0 KiB x 2.00 + 169.0 KiB x 1.00) x 1024
-TRAFFIC_DEFAULT_WORKLOAD = 34208479
+TRAFFIC_DEFAULT_WORKLOAD = 34207456
 
 
 def parse():
