@@ -196,6 +196,47 @@ def test_full_attention_with_scores(cuda, dtype, hq, hkv, n):
     assert (lse[0].cpu() - torch.logsumexp(logits, -1)).abs().max() <= 1e-3
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("hq,hkv,n", [(32, 32, 4099), (32, 8, 9000), (8, 1, 700)])
+def test_logits_in_the_kv_dtype(cuda, dtype, hq, hkv, n):
+    """The reference keeps its logits buffer in the model's 16-bit type
+    (tidal/utils/controller.py:149-151).  A selection launch that is handed such a buffer stores
+    the fp32 logit rounded to that type (within one step of the type of the oracle's logit), the
+    attention output is unchanged, and the top-k of the stored rows -- with the launch's
+    log-sum-exp as the rows' bound -- is the oracle's stable top-k of exactly those values."""
+    from oracle import tidal_oracle as orc
+    from tidaldecode_amd import _kernels
+
+    d, page_size, k = 128, 16, 300
+    case = PagedCase(n, hkv, d, page_size, dtype, seed=n + 3)
+    q = randn((hq, d), n + 4, dtype)
+    logits = orc.attn_logits(q, case.k)
+    want = orc.softmax_pv(logits, case.v)
+    w = _wrapper(0, hq, hkv, d, page_size, dtype)
+    qd = q.to(dtype).to(cuda).unsqueeze(0)
+    od = torch.empty_like(qd)
+    stride = case.n_pages * page_size
+    scores = torch.full((hq, stride), float("nan"), dtype=dtype, device=cuda)
+    lse = torch.empty((1, hq), dtype=torch.float32, device=cuda)
+    table = case.page_table[:-1].to(torch.int32).unsqueeze(0)
+    w.forward(qd, od, case.pool.to(cuda), table.to(cuda), None, case.last_page_len,
+              int(case.page_table[-1]), scores, lse=lse)
+    torch.cuda.synchronize()
+    assert tolerance_report(od[0], want) <= ATOL[dtype]
+    got = scores[:, :n].cpu()
+    assert torch.isnan(scores[:, n:]).all()
+    # one step of the 16-bit type at the logit's magnitude: 2^-10 (fp16) / 2^-7 (bf16) relative
+    step = (2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7) * logits.abs().clamp_min(2.0 ** -14)
+    assert ((got.float() - logits).abs() <= step + 2e-4).all()
+    assert (lse[0].cpu() - torch.logsumexp(logits, -1)).abs().max() <= 1e-3
+    # the lse bounds the rounded logits as well?  Rounding up can pass an fp32 bound by half a step:
+    # the kernel leaves one bf16 step of room for 16-bit rows (csrc/topk.hip), enough for both types
+    out = torch.empty((hq, k), dtype=torch.int32, device=cuda)
+    _kernels.topk_filtering(scores[:, :n], None, None, out, None, k, upper_bound=lse.view(-1))
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu().long(), orc.stable_topk(got.float(), k))
+
+
 @pytest.mark.parametrize("k_max", [300, 1800])
 def test_batch_ragged_slots(cuda, k_max):
     """Batch of 8 sequences with different lengths sharing one pool; per-head slot lists with
