@@ -237,11 +237,12 @@ def test_logits_in_the_kv_dtype(cuda, dtype, hq, hkv, n):
     assert torch.equal(out.cpu().long(), orc.stable_topk(got.float(), k))
 
 
-@pytest.mark.parametrize("k_max", [300, 1800])
+@pytest.mark.parametrize("k_max", [300, 1800, 5000])
 def test_batch_ragged_slots(cuda, k_max):
     """Batch of 8 sequences with different lengths sharing one pool; per-head slot lists with
     per-sequence counts through indptr.  Lists of up to 1800 entries are planned as one workgroup of
-    2048 tokens per head and sequence, the short ones as four-wave workgroups of 128."""
+    2048 tokens per head and sequence (up to 5000: of 8192), the short ones as four-wave workgroups
+    of 128."""
     from oracle import tidal_oracle as orc
 
     dtype, h, d, page_size = torch.float16, 32, 128, 16
