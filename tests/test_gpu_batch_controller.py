@@ -37,7 +37,21 @@ def test_lockstep_decode_other_shapes(cuda, lens, budget, steps, stepping):
     _lockstep(cuda, 4, 4, "per_head", torch.float16, 16, stepping, lens, budget, steps)
 
 
-def _lockstep(cuda, hq, hkv, mode, dtype, page, stepping, lens, budget, steps):
+def test_lockstep_decode_with_logits_in_the_kv_dtype(cuda):
+    """logits_dtype = the KV dtype: the buffer type of the reference (tidal/utils/controller.py:149).
+    The selection is then the stable top-k of the ROUNDED logits, which is what the checks of
+    _lockstep compare with (they rank the scores that the launch stored)."""
+    _lockstep(cuda, 8, 2, "per_head", torch.float16, 16, "host", [5, 40, 200], 16, 6,
+              logits_dtype=torch.float16)
+    _lockstep(cuda, 4, 4, "per_head", torch.bfloat16, 8, "captured", [5, 40, 200], 16, 6,
+              logits_dtype=torch.bfloat16)
+    from tidaldecode_amd.utils import BatchInferenceController
+    with pytest.raises(ValueError, match="float32 logits"):
+        BatchInferenceController(1, 4, 128, 16, 8, 64, 2, torch.float16, cuda, num_kv_heads=2,
+                                 select_mode="group_sum", logits_dtype=torch.float16)
+
+
+def _lockstep(cuda, hq, hkv, mode, dtype, page, stepping, lens, budget, steps, logits_dtype=None):
     """stepping = "captured": pages are reserved ahead, the whole step (metadata advance on the
     device, RoPE table, the three layers, top-k) is captured once and replayed per token, with
     eager copies of the step's inputs and synchronisations between the replays."""
@@ -47,8 +61,9 @@ def _lockstep(cuda, hq, hkv, mode, dtype, page, stepping, lens, budget, steps):
     d, layers, theta = 128, 3, 1e4
     B = len(lens)
     ctl = BatchInferenceController(layers, hq, d, page, budget, 256, B + 1, dtype, cuda,
-                                   num_kv_heads=hkv, select_mode=mode, page_order_seed=3)
-    assert ctl.fused_step_ok
+                                   num_kv_heads=hkv, select_mode=mode, page_order_seed=3,
+                                   logits_dtype=logits_dtype)
+    assert ctl.fused_step_ok and ctl.qk_product.dtype == (logits_dtype or torch.float32)
     ctl.add_sequences(lens)
     hist_k = [[randn((n, hkv, d), 100 * l + b, dtype) for b, n in enumerate(lens)] for l in range(layers)]
     hist_v = [[randn((n, hkv, d), 100 * l + b + 50, dtype) for b, n in enumerate(lens)] for l in range(layers)]
@@ -129,7 +144,10 @@ def _lockstep(cuda, hq, hkv, mode, dtype, page, stepping, lens, budget, steps):
                     logits = orc.attn_logits(q_rot[b], hist_k[l][b])
                     assert tolerance_report(o[b], orc.softmax_pv(logits, hist_v[l][b])) <= ATOL[dtype], (step, b)
                     got_logits = ctl.qk_product[b * hq: (b + 1) * hq, :n].cpu()
-                    assert (got_logits - logits).abs().max() <= 2e-2, (step, b)
+                    tol = 2e-2
+                    if logits_dtype is not None:   # stored in 16 bits: half a step of the type
+                        tol += (2.0 ** -11 if logits_dtype == torch.float16 else 2.0 ** -8) * logits.abs()
+                    assert ((got_logits - logits).abs() <= tol).all(), (step, b)
                     assert torch.isinf(ctl.qk_product[b * hq: (b + 1) * hq, n:]).all()
                     scores = got_logits if mode == "per_head" else ctl.score_sum[b * rows: (b + 1) * rows, :n].cpu()
                     if mode != "per_head":   # the reduction itself, against the closed form

@@ -12,7 +12,7 @@ import numpy as np
 import pytest
 import torch
 
-from _util import PagedCase, randn
+from _util import ATOL, PagedCase, randn
 
 pytestmark = pytest.mark.gpu
 
@@ -276,6 +276,52 @@ def test_page_score_estimator(cuda, dtype, hq, hkv, d, page, layout):
         want = want[:, : n_pages - 1]
         tol = (2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7) * want.abs().clamp(min=1.0) + 1e-3
         assert ((got.float().cpu() - want).abs() <= tol).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("hq,hkv,page,n,budget", [(32, 32, 16, 4099, 300), (8, 2, 4, 1110, 40)])
+def test_selection_step_with_logits_in_the_kv_dtype(cuda, dtype, hq, hkv, page, n, budget):
+    """InferenceController(logits_dtype=<KV dtype>): the reference's buffer type
+    (tidal/utils/controller.py:149-151).  decode_sparse_attn over the whole cache stores the logits
+    rounded to that type, decode_topk ranks the stored values (bit-exact against the oracle's
+    stable top-k of the same values, through the page table), and a sparse layer over the chosen
+    slots matches the oracle's attention over those tokens."""
+    from oracle import tidal_oracle as orc
+    from tidaldecode_amd import utils as ops
+    from tidaldecode_amd.utils import InferenceController
+
+    d = 128
+    with pytest.raises(ValueError, match="logits_dtype"):
+        InferenceController(1, hq, d, page, budget, n + 64, dtype, cuda, logits_dtype=torch.float64)
+    c = InferenceController(1, hq, d, page, budget, n + 64, dtype, cuda, num_kv_heads=hkv,
+                            page_order_seed=4, logits_dtype=dtype)
+    assert c.qk_product.dtype == dtype
+    g = torch.Generator().manual_seed(n + budget)
+    k = torch.randn((n, hkv, d), generator=g).to(dtype)
+    v = torch.randn((n, hkv, d), generator=g).to(dtype)
+    q = torch.randn((1, hq, d), generator=g).to(dtype)
+    c.prepare_metadata(n - 1)
+    c.begin_forward(n - 1)
+    ops.append_kv(k[:n - 1].to(cuda), v[:n - 1].to(cuda), c, 0)
+    c.end_forward()
+    c.prepare_metadata(1)
+    c.begin_forward(1)
+    ops.append_kv(k[n - 1:].to(cuda), v[n - 1:].to(cuda), c, 0)
+    o = ops.decode_sparse_attn(q.to(cuda), c, 0, c.kv_indices_without_last, True)
+    ops.decode_topk(c)
+    o2 = ops.decode_sparse_attn(q.to(cuda), c, 0, c.topk_dindices_buffer, False)
+    torch.cuda.synchronize()
+    logits = orc.attn_logits(q[0], k)
+    assert (o[0].float().cpu() - orc.softmax_pv(logits, v)).abs().max() <= ATOL[dtype]
+    stored = c.qk_product[:, :n].float().cpu()
+    step = (2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7) * logits.abs().clamp_min(2.0 ** -14)
+    assert ((stored - logits).abs() <= step + 2e-4).all()
+    pos = orc.stable_topk(stored, budget)
+    table = c.kv_cache.indices_device.cpu().long()
+    got = c.topk_dindices_buffer[:, :budget].cpu().long()
+    assert torch.equal(got, table[pos // page] * page + pos % page)
+    assert (o2[0].float().cpu() - orc.sparse_layer_gather(q[0], k, v, pos)).abs().max() <= ATOL[dtype]
+    c.clean_states()
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])

@@ -26,6 +26,7 @@ from typing import List, Optional, Sequence
 import torch
 
 from .. import _kernels, _lib
+from .controller import _logits_dtype
 from .paged import BatchDecodeWithPagedKVCacheWrapper, KvPool, TensorLayout
 
 _SELECT_MODES = ("per_head", "group_sum", "head_sum")
@@ -41,7 +42,8 @@ class BatchInferenceController:
     def __init__(self, num_layers: int, num_heads: int, head_dim: int, page_size: int,
                  token_budget: int, max_seq_len: int, max_batch: int, dtype, device, *,
                  num_kv_heads: Optional[int] = None, select_mode: str = "per_head",
-                 kv_layout: str = "NHD", page_order_seed=None):
+                 kv_layout: str = "NHD", page_order_seed=None,
+                 logits_dtype: Optional[torch.dtype] = None):
         if select_mode not in _SELECT_MODES:
             raise KeyError(f"Invalid select_mode {select_mode}")
         num_kv_heads = num_heads if num_kv_heads is None else num_kv_heads
@@ -77,8 +79,10 @@ class BatchInferenceController:
         self.score_cols = self.pages_per_seq * page_size
         self.budget = min(int(token_budget), self.score_cols)
         self.index_rows = {"per_head": num_heads, "group_sum": num_kv_heads, "head_sum": 1}[select_mode]
+        # float32, or the KV dtype as in the reference (see controller._logits_dtype)
         self.qk_product = torch.full((max_batch * num_heads, self.score_cols), float("-inf"),
-                                     dtype=torch.float32, device=device)
+                                     dtype=_logits_dtype(logits_dtype, dtype, select_mode),
+                                     device=device)
         self.lse = torch.zeros((max_batch, num_heads), dtype=torch.float32, device=device)
         self.score_sum = None
         if select_mode != "per_head":

@@ -27,13 +27,29 @@ _SELECT_MODES = ("per_head", "group_sum", "head_sum")
 _SELECT_SCOPES = ("all", "exclude_last_page")
 
 
+def _logits_dtype(logits_dtype, kv_dtype, select_mode):
+    """The type of the logits buffer that a selection layer fills: float32 (default), or the KV
+    dtype, which is what the reference allocates (tidal/utils/controller.py:149-151: the logits
+    are then rounded to 16 bits before the top-k sees them).  The summed selection modes read
+    float32 logits only."""
+    if logits_dtype is None:
+        return torch.float32
+    if logits_dtype not in (torch.float32, kv_dtype):
+        raise ValueError(f"logits_dtype must be torch.float32 or the KV dtype {kv_dtype}, not {logits_dtype}")
+    if logits_dtype != torch.float32 and select_mode != "per_head":
+        raise ValueError(f"select_mode {select_mode} sums probabilities from float32 logits")
+    return logits_dtype
+
+
 class InferenceController:
     def __init__(self, num_layers, num_heads, head_dim, page_size, token_budget, max_seq_len,
                  dtype, device, *, num_kv_heads: Optional[int] = None,
                  select_mode: str = "per_head", select_scope: str = "all",
-                 kv_layout: str = "NHD", with_metadata: bool = False, page_order_seed=None):
+                 kv_layout: str = "NHD", with_metadata: bool = False, page_order_seed=None,
+                 logits_dtype: Optional[torch.dtype] = None):
         if select_mode not in _SELECT_MODES:
             raise KeyError(f"Invalid select_mode {select_mode}")
+        logits_dtype = _logits_dtype(logits_dtype, dtype, select_mode)
         if select_scope not in _SELECT_SCOPES:
             raise KeyError(f"Invalid select_scope {select_scope}")
         num_kv_heads = num_heads if num_kv_heads is None else num_kv_heads
@@ -79,7 +95,7 @@ class InferenceController:
         # selection state, allocated once
         self.index_rows = {"per_head": num_heads, "group_sum": num_kv_heads, "head_sum": 1}[select_mode]
         score_cols = max_kv_pages_num * page_size
-        self.qk_product = torch.zeros((num_heads, score_cols), dtype=torch.float32, device=device)
+        self.qk_product = torch.zeros((num_heads, score_cols), dtype=logits_dtype, device=device)
         self.lse = torch.zeros((1, num_heads), dtype=torch.float32, device=device)
         self.score_sum = None
         if select_mode != "per_head":
